@@ -1,0 +1,173 @@
+"""ctypes binding of the CPU oracle (oracle/liborin_oracle.so) -- TEST INFRASTRUCTURE.
+
+Importable only from tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg.
+The product package never imports this module.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liborin_oracle.so")
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_int = ctypes.c_int
+_flt = ctypes.c_float
+
+
+def build():
+    """Compile the C restatement (gcc, a few seconds)."""
+    subprocess.run(["make", "-C", _HERE, "liborin_oracle.so"], check=True, capture_output=True)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.orc_fp16_to_fp32_n.argtypes = [_u16p, _f32p, ctypes.c_size_t]
+    lib.orc_fp32_to_fp16_n.argtypes = [_f32p, _u16p, ctypes.c_size_t]
+    lib.orc_kv_store_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int]
+    lib.orc_kv_store_f16.argtypes = [_u16p, _u16p, _f32p, _f32p, _int, _int, _int, _int, _int]
+    lib.orc_attention_token_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
+    lib.orc_attention_token_f16.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
+    lib.orc_attention_row_f16.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _flt, _f32p]
+    lib.orc_flash_attention.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _int, _int, _flt]
+    lib.orc_flash_attention_decode_ind.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _i32p, _flt]
+    lib.orc_flash_attention_rows.argtypes = [_f32p, _u16p, _u16p, _f32p, _i32p, _int,
+                                             _int, _int, _int, _int, _int, _flt, _int]
+    lib.orc_max_threads.restype = _int
+    for name in ("orc_fp16_to_fp32_n", "orc_fp32_to_fp16_n", "orc_kv_store_f32", "orc_kv_store_f16",
+                 "orc_attention_token_f32", "orc_attention_token_f16", "orc_attention_row_f16",
+                 "orc_flash_attention", "orc_flash_attention_decode_ind", "orc_flash_attention_rows"):
+        getattr(lib, name).restype = None
+    return lib
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _load()
+    return _lib
+
+
+def _p(a, typ):
+    return a.ctypes.data_as(typ)
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def fp16_to_fp32(bits):
+    bits = _c(bits, np.uint16)
+    out = np.empty(bits.shape, np.float32)
+    lib().orc_fp16_to_fp32_n(_p(bits, _u16p), _p(out, _f32p), bits.size)
+    return out
+
+
+def fp32_to_fp16(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_fp32_to_fp16_n(_p(x, _f32p), _p(out, _u16p), x.size)
+    return out
+
+
+def kv_store_f16(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch):
+    """kc, vc: uint16 arrays [n_kv][n_ctx][d], modified in place; k, v: fp32 [batch][n_kv][d]."""
+    k, v = _c(k, np.float32), _c(v, np.float32)
+    assert kc.dtype == np.uint16 and kc.flags.c_contiguous and kc.size == n_kv * n_ctx * d
+    lib().orc_kv_store_f16(_p(kc, _u16p), _p(vc, _u16p), _p(k, _f32p), _p(v, _f32p), n_kv, d, n_ctx, pos_base, batch)
+
+
+def kv_store_f32(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch):
+    k, v = _c(k, np.float32), _c(v, np.float32)
+    assert kc.dtype == np.float32 and kc.flags.c_contiguous and kc.size == n_kv * n_ctx * d
+    lib().orc_kv_store_f32(_p(kc, _f32p), _p(vc, _f32p), _p(k, _f32p), _p(v, _f32p), n_kv, d, n_ctx, pos_base, batch)
+
+
+def attention_token_f32(q, kc, vc, n_head, n_kv, d, n_ctx, npos, scale):
+    q, kc, vc = _c(q, np.float32), _c(kc, np.float32), _c(vc, np.float32)
+    out = np.empty((n_head, d), np.float32)
+    score = np.empty(max(npos, 1), np.float32)
+    lib().orc_attention_token_f32(_p(q, _f32p), _p(kc, _f32p), _p(vc, _f32p), _p(out, _f32p),
+                                  n_head, n_kv, d, n_ctx, npos, scale, _p(score, _f32p))
+    return out
+
+
+def attention_token_f16(q, kc, vc, n_head, n_kv, d, n_ctx, npos, scale):
+    q, kc, vc = _c(q, np.float32), _c(kc, np.uint16), _c(vc, np.uint16)
+    out = np.empty((n_head, d), np.float32)
+    score = np.empty(max(npos, 1), np.float32)
+    lib().orc_attention_token_f16(_p(q, _f32p), _p(kc, _u16p), _p(vc, _u16p), _p(out, _f32p),
+                                  n_head, n_kv, d, n_ctx, npos, scale, _p(score, _f32p))
+    return out
+
+
+def flash_attention(q, kc, vc, n_head, n_kv, d, n_ctx, n_past, batch, scale):
+    """Same call shape as the operator API: q fp32 [batch][n_head][d]; caches uint16 [n_kv][n_ctx][d]."""
+    q, kc, vc = _c(q, np.float32), _c(kc, np.uint16), _c(vc, np.uint16)
+    assert q.size == batch * n_head * d and kc.size == n_kv * n_ctx * d == vc.size
+    out = np.empty((batch, n_head, d), np.float32)
+    lib().orc_flash_attention(_p(q, _f32p), _p(kc, _u16p), _p(vc, _u16p), _p(out, _f32p),
+                              n_head, n_kv, d, n_ctx, n_past, batch, scale)
+    return out
+
+
+def flash_attention_decode_ind(q, kc, vc, n_head, n_kv, d, n_ctx, pos, scale):
+    q, kc, vc = _c(q, np.float32), _c(kc, np.uint16), _c(vc, np.uint16)
+    assert q.size == n_head * d and kc.size == n_kv * n_ctx * d == vc.size
+    out = np.empty((n_head, d), np.float32)
+    p = ctypes.c_int(int(pos))
+    lib().orc_flash_attention_decode_ind(_p(q, _f32p), _p(kc, _u16p), _p(vc, _u16p), _p(out, _f32p),
+                                         n_head, n_kv, d, n_ctx, ctypes.byref(p), scale)
+    return out
+
+
+def flash_attention_rows(q, kc, vc, rows, n_head, n_kv, d, n_ctx, n_past, scale, threads=0):
+    """rows: int array [n_rows][2] of (token, head).  Returns fp32 [n_rows][d]."""
+    q, kc, vc = _c(q, np.float32), _c(kc, np.uint16), _c(vc, np.uint16)
+    rows = _c(rows, np.int32).reshape(-1, 2)
+    out = np.empty((rows.shape[0], d), np.float32)
+    if threads <= 0:
+        threads = max_threads()
+    lib().orc_flash_attention_rows(_p(q, _f32p), _p(kc, _u16p), _p(vc, _u16p), _p(out, _f32p),
+                                   _p(rows, _i32p), rows.shape[0], n_head, n_kv, d, n_ctx, n_past,
+                                   scale, threads)
+    return out
+
+
+def max_threads():
+    return min(int(lib().orc_max_threads()), 16)
+
+
+def attention_f64(q, k, v, n_past, scale):
+    """Textbook closed form in float64, independent of the C code.
+
+    q [batch][n_head][d]; k, v [n_kv][L][d] (any float dtype, L >= n_past + batch);
+    token b sees positions [0, n_past + b + 1).  Returns float64 [batch][n_head][d].
+    """
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    batch, n_head, d = q.shape
+    n_kv = k.shape[0]
+    out = np.empty((batch, n_head, d), np.float64)
+    L = n_past + batch
+    for h in range(n_head):
+        g = h * n_kv // n_head
+        s = (q[:, h, :] @ k[g, :L, :].T) * float(scale)  # [batch][L]
+        mask = np.arange(L)[None, :] > (n_past + np.arange(batch))[:, None]
+        s = np.where(mask, -np.inf, s)
+        s = s - s.max(axis=1, keepdims=True)
+        p = np.exp(s)
+        p /= p.sum(axis=1, keepdims=True)
+        out[:, h, :] = p @ v[g, :L, :]
+    return out

@@ -1,0 +1,215 @@
+"""Pins the CPU oracle (oracle/attention_ref.c) before anything is compared against it.
+
+1. Golden vectors: logits of the unmodified reference CPU build (config 1), bit for bit.
+2. fp16 codecs: exhaustive / dense against numpy float16.
+3. Float64 closed form and structural invariants that a dropped term, a wrong
+   index or a transposed operand would break.
+"""
+import numpy as np
+import pytest
+
+from oracle import ref
+from util import make_case, rel_err
+
+
+def _caches_f32(cfg, k, v, n_ctx):
+    n_kv, d = cfg["n_kv"], cfg["d"]
+    n_tok = k.shape[0]
+    kc = np.zeros((n_kv, n_ctx, d), np.float32)
+    vc = np.zeros((n_kv, n_ctx, d), np.float32)
+    ref.kv_store_f32(kc, vc, k.reshape(n_tok, n_kv, d), v.reshape(n_tok, n_kv, d), n_kv, d, n_ctx, 0, n_tok)
+    return kc, vc
+
+
+def _tail_logits(cfg, t, attn):
+    """What the synthetic model does after attention: residual add, final rms_norm
+    (double sum in index order, reference src/model_cpu.cpp:13-18) and the one-hot output rows."""
+    x = np.zeros(cfg["n_embd"], np.float32)
+    x[t] = 1.0
+    x[cfg["out_base"]:cfg["out_base"] + attn.size] = attn.reshape(-1)
+    ss = np.cumsum(x.astype(np.float64) * x.astype(np.float64))[-1]  # sequential, like the C loop
+    r = 1.0 / np.sqrt(ss / cfg["n_embd"] + 0.0)
+    y = (x.astype(np.float64) * r * 1.0).astype(np.float32)
+    return np.concatenate([y[cfg["out_base"]:cfg["out_base"] + attn.size], y[t:t + 1]])
+
+
+@pytest.mark.parametrize("variant", ["a", "b"])
+def test_golden_cfg1_bit_exact(cfg1, variant):
+    """Oracle outputs pushed through the model's tail reproduce the reference's logits exactly."""
+    c = cfg1
+    n_tok = c["n_prefill"] + c["n_decode"]
+    k, v = c["k"], c["v"]
+    if variant == "b":
+        k = k.astype(np.float16).astype(np.float32)
+        v = v.astype(np.float16).astype(np.float32)
+    n_ctx = 192
+    kc, vc = _caches_f32(c, k, v, n_ctx)
+    scale = np.float32(1.0) / np.sqrt(np.float32(c["d"]))
+    logits = c["logits_" + variant]
+    worst = 0.0
+    for t in range(n_tok):
+        attn = ref.attention_token_f32(c["q"][t], kc, vc, c["n_head"], c["n_kv"], c["d"], n_ctx, t + 1, scale)
+        mine = _tail_logits(c, t, attn)
+        assert np.array_equal(mine.view(np.uint32), logits[t].view(np.uint32)), f"token {t}"
+        # and the direct recovery attn_i = logits_i / logits_last, good to a few ulp
+        rec = logits[t, :-1] / logits[t, -1]
+        worst = max(worst, float(np.abs(rec - attn.reshape(-1)).max() / np.abs(attn).max()))
+    assert worst < 5e-7
+
+
+def test_f16_cache_variant_matches_f32_on_representable_values(cfg1):
+    c = cfg1
+    n_tok, n_ctx = 64, 80
+    k16 = c["k"][:n_tok].astype(np.float16)
+    v16 = c["v"][:n_tok].astype(np.float16)
+    kc, vc = _caches_f32(c, k16.astype(np.float32), v16.astype(np.float32), n_ctx)
+    kcb = np.zeros((c["n_kv"], n_ctx, c["d"]), np.uint16)
+    vcb = np.zeros_like(kcb)
+    ref.kv_store_f16(kcb, vcb, c["k"][:n_tok].reshape(n_tok, c["n_kv"], c["d"]),
+                     c["v"][:n_tok].reshape(n_tok, c["n_kv"], c["d"]), c["n_kv"], c["d"], n_ctx, 0, n_tok)
+    scale = np.float32(0.088388346)
+    for t in (0, 1, 17, 63):
+        a = ref.attention_token_f32(c["q"][t], kc, vc, c["n_head"], c["n_kv"], c["d"], n_ctx, t + 1, scale)
+        b = ref.attention_token_f16(c["q"][t], kcb, vcb, c["n_head"], c["n_kv"], c["d"], n_ctx, t + 1, scale)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    # whole-chunk form and the row-sampled, position-outermost form agree bit for bit
+    q = c["q"][:n_tok].reshape(n_tok, c["n_head"], c["d"])
+    full = ref.flash_attention(q[40:], kcb, vcb, c["n_head"], c["n_kv"], c["d"], n_ctx, 40, n_tok - 40, scale)
+    rows = np.array([(t, h) for t in range(n_tok - 40) for h in range(c["n_head"])], np.int32)
+    for threads in (1, 4):
+        samp = ref.flash_attention_rows(q[40:], kcb, vcb, rows, c["n_head"], c["n_kv"], c["d"], n_ctx, 40, scale,
+                                        threads=threads)
+        assert np.array_equal(samp.reshape(full.shape).view(np.uint32), full.view(np.uint32))
+    dec = ref.flash_attention_decode_ind(q[63], kcb, vcb, c["n_head"], c["n_kv"], c["d"], n_ctx, 63, scale)
+    assert np.array_equal(dec.view(np.uint32), full[63 - 40].view(np.uint32))
+
+
+def test_fp16_decode_exhaustive():
+    bits = np.arange(65536, dtype=np.uint16)
+    got = ref.fp16_to_fp32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_fp16_encode_dense():
+    rng = np.random.default_rng(7)
+    # every fp16 value, its neighbours' midpoints (ties), random bit patterns, and the range edges
+    h = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    h = h[np.isfinite(h)]
+    hs = np.sort(h)
+    mids = ((hs[:-1].astype(np.float64) + hs[1:].astype(np.float64)) / 2).astype(np.float32)
+    rnd = rng.integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    edge = np.array([65504, 65519.99, 65520, 65536, 1e10, -1e10, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                     2.0 ** -25 * 1.0001, 2.0 ** -26, 6.1e-5, -0.0, 0.0], np.float32)
+    x = np.concatenate([h, mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+                        rnd, edge])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    got = ref.fp32_to_fp16(x).view(np.float16)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16))
+
+
+def test_kv_store_layout():
+    rng = np.random.default_rng(3)
+    n_kv, d, n_ctx, pos, batch = 3, 64, 37, 11, 5
+    k = rng.standard_normal((batch, n_kv, d), dtype=np.float32) * 3
+    v = rng.standard_normal((batch, n_kv, d), dtype=np.float32)
+    kc = np.full(n_kv * n_ctx * d, 0xAAAA, np.uint16)
+    vc = np.full(n_kv * n_ctx * d, 0xBBBB, np.uint16)
+    ref.kv_store_f16(kc, vc, k, v, n_kv, d, n_ctx, pos, batch)
+    wk = np.full((n_kv, n_ctx, d), 0xAAAA, np.uint16)
+    wv = np.full((n_kv, n_ctx, d), 0xBBBB, np.uint16)
+    for b in range(batch):
+        for h in range(n_kv):
+            wk[h, pos + b] = k[b, h].astype(np.float16).view(np.uint16)
+            wv[h, pos + b] = v[b, h].astype(np.float16).view(np.uint16)
+    assert np.array_equal(kc, wk.reshape(-1)) and np.array_equal(vc, wv.reshape(-1))
+
+
+@pytest.mark.parametrize("n_head,n_kv,d", [(12, 2, 128), (32, 8, 128), (28, 4, 128), (8, 8, 64), (5, 1, 64)])
+def test_closed_form_f64(n_head, n_kv, d):
+    n_ctx, n_past, batch = 300, 131, 33
+    q, kc, vc = make_case(11 + n_head, n_head, n_kv, d, n_ctx, n_past + batch, batch, outliers=4)
+    scale = 1.0 / np.sqrt(d)
+    got = ref.flash_attention(q, kc, vc, n_head, n_kv, d, n_ctx, n_past, batch, np.float32(scale))
+    want = ref.attention_f64(q, kc.view(np.float16), vc.view(np.float16), n_past, np.float32(scale))
+    gated, glob, l2 = rel_err(got, want)
+    # the gated metric floors |ref| at 1% of the row maximum, so it can reach 100x the global figure
+    assert glob < 5e-6 and l2 < 2e-6 and gated < 5e-4, (gated, glob, l2)
+
+
+def test_closed_form_torch_sdpa():
+    """With n_kv == n_head and one token the path is plain scaled-dot-product attention."""
+    torch = pytest.importorskip("torch")
+    n_head, d, n_ctx, L = 6, 128, 96, 77
+    q, kc, vc = make_case(5, n_head, n_head, d, n_ctx, L, 1)
+    scale = 1.0 / np.sqrt(d)
+    got = ref.flash_attention_decode_ind(q[0], kc, vc, n_head, n_head, d, n_ctx, L - 1, np.float32(scale))
+    k = torch.from_numpy(kc.view(np.float16)[:, :L].astype(np.float64))
+    v = torch.from_numpy(vc.view(np.float16)[:, :L].astype(np.float64))
+    qq = torch.from_numpy(q[0].astype(np.float64))[:, None, :]
+    want = torch.nn.functional.scaled_dot_product_attention(qq, k, v, scale=float(np.float32(scale)))[:, 0].numpy()
+    assert rel_err(got, want)[1] < 5e-6
+
+
+def test_invariants():
+    n_head, n_kv, d, n_ctx = 12, 2, 128, 160
+    L = 131
+    scale = np.float32(1.0 / np.sqrt(d))
+    q, kc, vc = make_case(21, n_head, n_kv, d, n_ctx, L, 1, poison_tail=True)
+    base = ref.flash_attention_decode_ind(q[0], kc, vc, n_head, n_kv, d, n_ctx, L - 1, scale)
+    assert np.isfinite(base).all()  # NaN rows beyond npos are never touched
+
+    # one visible position: out == V[0] exactly
+    one = ref.flash_attention_decode_ind(q[0], kc, vc, n_head, n_kv, d, n_ctx, 0, scale)
+    for h in range(n_head):
+        assert np.array_equal(one[h], vc[h * n_kv // n_head, 0].view(np.float16).astype(np.float32))
+
+    # constant V => constant output (to rounding)
+    vconst = vc.copy()
+    vconst[:, :L] = np.float16(1.5).view(np.uint16)
+    o = ref.flash_attention_decode_ind(q[0], kc, vconst, n_head, n_kv, d, n_ctx, L - 1, scale)
+    assert np.abs(o - 1.5).max() < 1e-5
+
+    # all keys equal => mean of visible V
+    kconst = kc.copy()
+    kconst[:, :L] = kc[:, :1]
+    o = ref.flash_attention_decode_ind(q[0], kconst, vc, n_head, n_kv, d, n_ctx, L - 1, scale)
+    for h in range(n_head):
+        g = h * n_kv // n_head
+        mean = vc[g, :L].view(np.float16).astype(np.float64).mean(axis=0)
+        assert np.abs(o[h] - mean).max() < 1e-5
+
+    # heads of one group with equal q give equal output; a head of the other group does not
+    q2 = q.copy()
+    q2[0, 1] = q2[0, 0]
+    q2[0, 6] = q2[0, 0]
+    o = ref.flash_attention_decode_ind(q2[0], kc, vc, n_head, n_kv, d, n_ctx, L - 1, scale)
+    assert np.array_equal(o[0], o[1]) and not np.allclose(o[0], o[6])
+
+    # permuting visible positions (K and V together) changes nothing beyond rounding
+    perm = np.random.default_rng(1).permutation(L)
+    kp, vp = kc.copy(), vc.copy()
+    kp[:, :L] = kc[:, perm]
+    vp[:, :L] = vc[:, perm]
+    o = ref.flash_attention_decode_ind(q[0], kp, vp, n_head, n_kv, d, n_ctx, L - 1, scale)
+    assert rel_err(o, base)[0] < 1e-4
+
+    # prefill row t at (n_past, batch) == decode at position n_past + t; chunk-split invariance
+    qb, kc, vc = make_case(22, n_head, n_kv, d, n_ctx, 100, 40)
+    whole = ref.flash_attention(qb, kc, vc, n_head, n_kv, d, n_ctx, 60, 40, scale)
+    first = ref.flash_attention(qb[:13], kc, vc, n_head, n_kv, d, n_ctx, 60, 13, scale)
+    rest = ref.flash_attention(qb[13:], kc, vc, n_head, n_kv, d, n_ctx, 73, 27, scale)
+    assert np.array_equal(np.concatenate([first, rest]).view(np.uint32), whole.view(np.uint32))
+    dec = ref.flash_attention_decode_ind(qb[29], kc, vc, n_head, n_kv, d, n_ctx, 89, scale)
+    assert np.array_equal(dec.view(np.uint32), whole[29].view(np.uint32))
+    # causality: changing a future row of the cache leaves earlier tokens untouched
+    kc2 = kc.copy()
+    kc2[:, 95] = kc[:, 3]
+    again = ref.flash_attention(qb, kc2, vc, n_head, n_kv, d, n_ctx, 60, 40, scale)
+    assert np.array_equal(again[:35].view(np.uint32), whole[:35].view(np.uint32))
+    assert not np.array_equal(again[35:], whole[35:])
