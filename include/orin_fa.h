@@ -1,0 +1,88 @@
+/*
+ * orin_fa -- C ABI of the MI355X (gfx950) GQA flash-attention path.
+ *
+ * This is the drop-in boundary for the two attention operators of the orin_llm
+ * engine and the launch plumbing they need.  Every entry point takes plain
+ * pointers and sizes; all data pointers are DEVICE pointers owned by the caller.
+ * Launches are asynchronous on the stream given to orin_fa_set_stream (the null
+ * stream by default); the caller synchronises.  The library keeps process-global
+ * state (stream, workspace) exactly as the reference operator layer does
+ * (reference: src/kernels.cu:1726-1728), so it is not re-entrant.
+ *
+ * Return convention: 0 on success, a negative ORIN_FA_E_* code otherwise
+ * (orin_fa_error_string names it).  The C++ shim that carries the reference's own
+ * signatures (include/orin_llm_amd/kernels.h) turns a non-zero code into
+ * print + abort(), the reference's convention (src/common.h:14-22).
+ *
+ * Data formats (reference: src/kernels.h:77-81, src/kernels.cu:1675-1677):
+ *   q, out   fp32, [batch][n_head][head_dim] (batch = 1 for decode)
+ *   kc, vc   IEEE binary16 bit patterns in uint16_t, one layer's cache,
+ *            element (kv_head, pos, i) at (kv_head * n_ctx + pos) * head_dim + i
+ *   GQA map  query head h reads KV head h / (n_head / n_kv)
+ */
+#ifndef ORIN_FA_H
+#define ORIN_FA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    ORIN_FA_OK = 0,
+    ORIN_FA_E_INVALID = -1,      /* bad shape or null pointer */
+    ORIN_FA_E_HEAD_DIM = -2,     /* head_dim not in {64, 128} (reference: assert, src/kernels.cu:1979,1998) */
+    ORIN_FA_E_WORKSPACE = -3,    /* no workspace, or too small for this shape */
+    ORIN_FA_E_NOT_INIT = -4,     /* orin_fa_init has not succeeded */
+    ORIN_FA_E_HIP = -1000        /* -(1000 + hipError_t) for runtime failures */
+};
+
+/* Replaces llm::cuda::init (reference: src/kernels.h:8, src/kernels.cu:1730-1737).
+ * Selects the device, reads its CU count and allocates the default split-KV
+ * workspace once.  Must be called before any launch and outside stream capture. */
+int orin_fa_init(int device);
+
+/* Replaces llm::cuda::set_stream (reference: src/kernels.h:10, src/kernels.cu:1728).
+ * stream is a hipStream_t; NULL selects the null stream. */
+void orin_fa_set_stream(void* stream);
+
+/* Replace the attention share of llm::cuda::scratch_size / scratch_assign
+ * (reference: src/kernels.h:11-12, src/kernels.cu:1753-1776): the bytes of device
+ * scratch the decode path needs for its split-KV partial results, and the call that
+ * points the library at a caller-owned block of at least that size (256-byte
+ * aligned).  Optional: orin_fa_init already allocates a block of this size. */
+size_t orin_fa_workspace_bytes(void);
+int orin_fa_set_workspace(void* dev_ptr, size_t bytes);
+
+/* Replaces llm::cuda::flash_attention (reference: src/kernels.h:77-78,
+ * src/kernels.cu:1974-1981): causal GQA attention for a chunk of `batch` query
+ * tokens at cache positions [n_past, n_past + batch).  Token b attends to cache
+ * positions [0, n_past + b]; the cache must already hold the chunk's own K/V
+ * (call site: src/model_gpu.cu:383-384).  Writes every (token < batch, head, i). */
+int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                    int n_head, int n_kv, int head_dim, int n_ctx, int n_past, int batch, float scale);
+
+/* Replaces llm::cuda::flash_attention_decode_ind (reference: src/kernels.h:80-81,
+ * src/kernels.cu:1993-2000): one query token attending to cache positions
+ * [0, *d_pos]; d_pos is a DEVICE pointer read by the kernel, so the call is safe
+ * under stream capture and the captured graph can be replayed after the position
+ * changes (call site: src/model_gpu.cu:281-282, 295-316).  Performs no allocation,
+ * no synchronisation and no host read of *d_pos; the launch shape depends only on
+ * the arguments passed by value. */
+int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                       int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
+
+/* Introspection for tests and benchmarks: the number of KV splits a decode launch
+ * with these shapes uses (0 if the shape is rejected), and the CU count seen at init. */
+int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx);
+int orin_fa_cu_count(void);
+
+/* Human-readable name of a return code. */
+const char* orin_fa_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

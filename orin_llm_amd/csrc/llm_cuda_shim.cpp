@@ -1,0 +1,52 @@
+// llm::cuda::* entry points with the reference's signatures (reference:
+// src/kernels.h:8-10,77-81; definitions src/kernels.cu:1728-1737,1974-2000),
+// forwarding to the C ABI.  Plain C++: no HIP headers, no device code.
+#include "../../include/orin_llm_amd/kernels.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+
+#include "../../include/orin_fa.h"
+
+namespace {
+
+[[noreturn]] void die(const char* what, int code) {
+    fflush(stdout);
+    fprintf(stderr, "orin_fa error %d (%s) in %s\n", code, orin_fa_error_string(code), what);
+    abort();
+}
+
+} // namespace
+
+namespace llm::cuda {
+
+#ifndef ORIN_FA_SHIM_NO_PLUMBING
+int init() {
+    // The reference hard-codes device 0 and returns -1 on failure (src/kernels.cu:1730-1737).
+    const int rc = orin_fa_init(0);
+    if (rc != ORIN_FA_OK) {
+        fprintf(stderr, "[cuda::init] orin_fa_init(0) failed: %s\n", orin_fa_error_string(rc));
+        return -1;
+    }
+    return 0;
+}
+
+void set_stream(void* stream) { orin_fa_set_stream(stream); }
+#endif
+
+void flash_attention(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                     int n_head, int n_kv, int head_dim, int n_ctx, int n_past, int batch, float scale) {
+    const int rc = orin_fa_prefill(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, n_past, batch, scale);
+    if (rc != ORIN_FA_OK) die("flash_attention", rc);
+}
+
+void flash_attention_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                                int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
+    // The reference skips the post-launch check here because the call runs under stream
+    // capture (src/kernels.cu:1983-1991); argument validation is host-only and capture-safe,
+    // so it stays.
+    const int rc = orin_fa_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale);
+    if (rc != ORIN_FA_OK) die("flash_attention_decode_ind", rc);
+}
+
+} // namespace llm::cuda

@@ -1,0 +1,109 @@
+"""ctypes mirror of the operator API, same names and argument order as the reference's
+src/kernels.h:8-12,77-81.  Pointer arguments accept torch tensors (device memory) or raw
+integer addresses.  A non-zero return code from the library raises, the Python analogue of
+the reference's print-and-abort (src/common.h:14-22).  There is no fallback: a missing
+library is an ImportError.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liborin_fa.so")
+
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+_flt = ctypes.c_float
+
+_lib = None
+
+
+class OrinFaError(RuntimeError):
+    def __init__(self, what, code):
+        self.code = code
+        super().__init__(f"{what}: orin_fa error {code} ({error_string(code)})")
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built (python -m orin_llm_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                              "(hipcc --offload-arch=gfx950); there is no CPU fallback")
+        L = ctypes.CDLL(LIB_PATH)
+        L.orin_fa_init.argtypes = [_int]
+        L.orin_fa_init.restype = _int
+        L.orin_fa_set_stream.argtypes = [_vp]
+        L.orin_fa_set_stream.restype = None
+        L.orin_fa_workspace_bytes.argtypes = []
+        L.orin_fa_workspace_bytes.restype = ctypes.c_size_t
+        L.orin_fa_set_workspace.argtypes = [_vp, ctypes.c_size_t]
+        L.orin_fa_set_workspace.restype = _int
+        L.orin_fa_prefill.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _flt]
+        L.orin_fa_prefill.restype = _int
+        L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
+        L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
+        L.orin_fa_decode_splits.restype = _int
+        L.orin_fa_cu_count.argtypes = []
+        L.orin_fa_cu_count.restype = _int
+        L.orin_fa_error_string.argtypes = [_int]
+        L.orin_fa_error_string.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    return x.data_ptr()
+
+
+def error_string(code):
+    return lib().orin_fa_error_string(int(code)).decode()
+
+
+def init(device=0):
+    rc = lib().orin_fa_init(int(device))
+    if rc != 0:
+        raise OrinFaError("init", rc)
+    return 0
+
+
+def set_stream(stream):
+    """stream: a hipStream_t address (e.g. torch.cuda.Stream.cuda_stream), or None/0 for the null stream."""
+    lib().orin_fa_set_stream(_ptr(stream) or None)
+
+
+def workspace_bytes():
+    return int(lib().orin_fa_workspace_bytes())
+
+
+def set_workspace(dev_ptr, nbytes):
+    rc = lib().orin_fa_set_workspace(_ptr(dev_ptr), int(nbytes))
+    if rc != 0:
+        raise OrinFaError("set_workspace", rc)
+
+
+def flash_attention(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, n_past, batch, scale):
+    rc = lib().orin_fa_prefill(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), n_head, n_kv, head_dim, n_ctx,
+                               n_past, batch, scale)
+    if rc != 0:
+        raise OrinFaError("flash_attention", rc)
+
+
+def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):
+    rc = lib().orin_fa_decode_ind(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), n_head, n_kv, head_dim, n_ctx,
+                                  _ptr(d_pos), scale)
+    if rc != 0:
+        raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def decode_splits(n_head, n_kv, head_dim, n_ctx):
+    return int(lib().orin_fa_decode_splits(n_head, n_kv, head_dim, n_ctx))
+
+
+def cu_count():
+    return int(lib().orin_fa_cu_count())

@@ -84,6 +84,28 @@ def test_f16_cache_variant_matches_f32_on_representable_values(cfg1):
     assert np.array_equal(dec.view(np.uint32), full[63 - 40].view(np.uint32))
 
 
+def test_fp16_cache_format_error(cfg1):
+    """What the cache format alone costs on config 1: the oracle on the fp16 cache against the
+    reference CPU build on its fp32 cache (variant A), no GPU involved.  The row-normalised
+    figure is ~3e-4; the variant that floors |ref| at 1% of the row maximum is ~5e-2, which is
+    why that variant is reported but cannot be the gate for any fp16-cache implementation."""
+    c = cfg1
+    H, G, d = c["n_head"], c["n_kv"], c["d"]
+    n = c["n_prefill"] + c["n_decode"]
+    n_ctx = 256
+    kc = np.zeros((G, n_ctx, d), np.uint16)
+    vc = np.zeros_like(kc)
+    ref.kv_store_f16(kc, vc, c["k"].reshape(n, G, d), c["v"].reshape(n, G, d), G, d, n_ctx, 0, n)
+    got = ref.flash_attention(c["q"].reshape(n, H, d), kc, vc, H, G, d, n_ctx, 0, n, np.float32(1 / np.sqrt(d)))
+    lg = c["logits_a"]
+    row, floor1pct, l2 = rel_err(got, (lg[:, :-1] / lg[:, -1:]).reshape(n, H, d))
+    assert 1e-4 < row < 1e-3 and l2 < 5e-4
+    assert floor1pct > 2e-2
+    lg = c["logits_b"]  # same values on both sides: the restatement itself is exact
+    row, floor1pct, l2 = rel_err(got, (lg[:, :-1] / lg[:, -1:]).reshape(n, H, d))
+    assert floor1pct < 1e-6
+
+
 def test_fp16_decode_exhaustive():
     bits = np.arange(65536, dtype=np.uint16)
     got = ref.fp16_to_fp32(bits)
@@ -137,9 +159,8 @@ def test_closed_form_f64(n_head, n_kv, d):
     scale = 1.0 / np.sqrt(d)
     got = ref.flash_attention(q, kc, vc, n_head, n_kv, d, n_ctx, n_past, batch, np.float32(scale))
     want = ref.attention_f64(q, kc.view(np.float16), vc.view(np.float16), n_past, np.float32(scale))
-    gated, glob, l2 = rel_err(got, want)
-    # the gated metric floors |ref| at 1% of the row maximum, so it can reach 100x the global figure
-    assert glob < 5e-6 and l2 < 2e-6 and gated < 5e-4, (gated, glob, l2)
+    row, floor1pct, l2 = rel_err(got, want)
+    assert row < 5e-6 and l2 < 2e-6 and floor1pct < 5e-4, (row, floor1pct, l2)
 
 
 def test_closed_form_torch_sdpa():
@@ -153,7 +174,7 @@ def test_closed_form_torch_sdpa():
     v = torch.from_numpy(vc.view(np.float16)[:, :L].astype(np.float64))
     qq = torch.from_numpy(q[0].astype(np.float64))[:, None, :]
     want = torch.nn.functional.scaled_dot_product_attention(qq, k, v, scale=float(np.float32(scale)))[:, 0].numpy()
-    assert rel_err(got, want)[1] < 5e-6
+    assert rel_err(got, want)[0] < 5e-6
 
 
 def test_invariants():
@@ -197,7 +218,7 @@ def test_invariants():
     kp[:, :L] = kc[:, perm]
     vp[:, :L] = vc[:, perm]
     o = ref.flash_attention_decode_ind(q[0], kp, vp, n_head, n_kv, d, n_ctx, L - 1, scale)
-    assert rel_err(o, base)[0] < 1e-4
+    assert rel_err(o, base)[0] < 1e-5
 
     # prefill row t at (n_past, batch) == decode at position n_past + t; chunk-split invariance
     qb, kc, vc = make_case(22, n_head, n_kv, d, n_ctx, 100, 40)

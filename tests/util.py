@@ -1,29 +1,35 @@
 """Shared helpers for the parity tests: input generators and the error metric."""
 import numpy as np
 
-# Gate for GPU-vs-oracle comparisons: max relative error on fp32 outputs.
+# Gate for GPU-vs-oracle comparisons: max relative error on fp32 outputs (rel_err()[0]).
 TOL = 2e-3
 
 
 def rel_err(got, ref):
-    """Relative error with a per-row floor.
+    """Error figures for fp32 attention outputs, rows = one (token, head) vector of head_dim.
 
-    err = max_i |got_i - ref_i| / max(|ref_i|, tau), tau = 1e-2 * max_j |ref_j| over the
-    output row (one token, one head).  Plain element-wise relative error is undefined
-    where the reference crosses zero; the floor is 1% of the row's largest magnitude.
-    Returns (gated error, max|diff|/max|ref|, relative L2).
+    Returns (err_row, err_floor1pct, rel_l2):
+      err_row        max over rows of max_i |got_i - ref_i| / max_j |ref_j|  -- THE GATE (< TOL).
+                     Element-wise relative error is undefined where the reference crosses
+                     zero, so the error of each element is taken relative to the largest
+                     magnitude of its own output row.
+      err_floor1pct  max_i |got_i - ref_i| / max(|ref_i|, 0.01 * rowmax): a stricter variant,
+                     reported only.  The fp16 cache format alone (fp32 CPU cache vs the same
+                     values rounded to fp16, no GPU involved) already scores 4.9e-2 on it for
+                     config 1, see tests/test_oracle.py::test_fp16_cache_format_error.
+      rel_l2         ||got - ref|| / ||ref|| over the whole tensor.
     """
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     assert got.shape == ref.shape
     g = got.reshape(-1, got.shape[-1])
     r = ref.reshape(-1, ref.shape[-1])
-    tau = 1e-2 * np.abs(r).max(axis=1, keepdims=True)
-    tau = np.maximum(tau, 1e-30)
-    gated = float((np.abs(g - r) / np.maximum(np.abs(r), tau)).max())
-    glob = float(np.abs(g - r).max() / max(np.abs(r).max(), 1e-30))
+    rowmax = np.maximum(np.abs(r).max(axis=1, keepdims=True), 1e-30)
+    diff = np.abs(g - r)
+    err_row = float((diff / rowmax).max())
+    err_floor = float((diff / np.maximum(np.abs(r), 1e-2 * rowmax)).max())
     l2 = float(np.linalg.norm(g - r) / max(np.linalg.norm(r), 1e-30))
-    return gated, glob, l2
+    return err_row, err_floor, l2
 
 
 def normal_f16(rng, shape):
