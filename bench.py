@@ -1,0 +1,331 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X GQA flash-attention path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu]
+
+Prints ONE JSON line.  A "step" is one pass of the attention operator over a whole layer
+stack of synthetic inputs already resident in HBM (independent seeds and buffers per layer):
+
+  qwen1.5b-prefill512   (default; BASELINE configs[1]) 28 layers x two 512-token causal chunks,
+                        at cache depth 0 and 3584, 12 Q heads / 2 KV heads, d=128, K with 4
+                        outlier channels x8.  value = causal-exact TFLOP/s.
+  llama8b-prefill512-d4096, qwen7b-prefill512-d32256, qwen1.5b-decode-32k, llama8b-decode-8k,
+  qwen7b-decode-32k     the other BASELINE shapes; the north-star cases are also run after the
+                        default workload and reported under "also".
+
+FLOPs per prefill launch (causal-exact): 4*d*H*(B*P + B*(B+1)/2).  Bytes per decode launch:
+4*G*L*d (fp16 K and V read once) + 2*H*d*4 (q in, out).  Peaks: 2.5e15 FLOP/s dense fp16
+MFMA, 8.0e12 B/s HBM3E.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_FLOPS = 2.5e15
+PEAK_BYTES = 8.0e12
+
+SHAPES = {
+    "qwen1.5b": dict(H=12, G=2, d=128, layers=28, outliers=4),
+    "llama8b": dict(H=32, G=8, d=128, layers=32, outliers=0),
+    "qwen7b": dict(H=28, G=4, d=128, layers=28, outliers=4),
+}
+
+WORKLOADS = {
+    # name: (shape, kind, n_ctx, list of (P, B) for prefill | L for decode)
+    "qwen1.5b-prefill512": ("qwen1.5b", "prefill", 4096, [(0, 512), (3584, 512)]),
+    "llama8b-prefill512-d4096": ("llama8b", "prefill", 8192, [(4096, 512)]),
+    "llama8b-prefill512-d0": ("llama8b", "prefill", 8192, [(0, 512)]),
+    "llama8b-prefill512-d7680": ("llama8b", "prefill", 8192, [(7680, 512)]),
+    "qwen7b-prefill512-d32256": ("qwen7b", "prefill", 32768, [(32256, 512)]),
+    "qwen1.5b-decode-1k": ("qwen1.5b", "decode", 32768, 1024),
+    "qwen1.5b-decode-8k": ("qwen1.5b", "decode", 32768, 8192),
+    "qwen1.5b-decode-32k": ("qwen1.5b", "decode", 32768, 32768),
+    "llama8b-decode-8k": ("llama8b", "decode", 8192, 8192),
+    "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
+}
+ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k"]
+
+
+def prefill_flops(H, d, P, B):
+    return 4.0 * d * H * (B * P + B * (B + 1) / 2.0)
+
+
+def decode_bytes(H, G, d, L):
+    return 4.0 * G * L * d + 2.0 * H * d * 4.0
+
+
+def make_layer(torch, seed, H, G, d, n_ctx, n_filled, batch, outliers):
+    """Seeded N(0,1) values rounded to fp16; K gets `outliers` channels per KV head scaled by 8."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    q = torch.randn((batch, H, d), generator=g, device="cuda", dtype=torch.float32).half().float()
+    k = torch.randn((G, n_ctx, d), generator=g, device="cuda", dtype=torch.float32).half()
+    v = torch.randn((G, n_ctx, d), generator=g, device="cuda", dtype=torch.float32).half()
+    if outliers:
+        for kvh in range(G):
+            ch = torch.randperm(d, generator=g, device="cuda")[:outliers]
+            k[kvh, :, ch] *= 8.0
+    if n_filled < n_ctx:  # the engine never zero-fills the cache: poison what must not be read
+        k[:, n_filled:] = float("nan")
+        v[:, n_filled:] = float("nan")
+    return q, k.view(torch.int16), v.view(torch.int16)
+
+
+def parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, n_past, batch, scale, n_rows=48):
+    rng = np.random.default_rng(0)
+    toks = sorted({0, batch - 1, *(int(x) for x in rng.integers(0, batch, size=6))})
+    rows = np.array([(t, h) for t in toks for h in rng.choice(H, size=min(H, max(1, n_rows // len(toks))),
+                                                              replace=False)], np.int32)
+    want = ref.flash_attention_rows(q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
+                                    v.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, n_past,
+                                    np.float32(scale))
+    got = out.cpu().numpy()[rows[:, 0], rows[:, 1]]
+    return rel_err(got, want)
+
+
+def cpu_baseline_prefill(ref, q, k, v, H, G, d, n_ctx, P, B, scale, budget_s=12.0):
+    """The oracle's reference-order loop (fp32 cache, one thread) on a bounded token sample."""
+    kf = ref.fp16_to_fp32(k)
+    vf = ref.fp16_to_fp32(v)
+    toks = [int(t) for t in np.linspace(0, B - 1, 64).round()]
+    done, flops, t0 = 0, 0.0, time.perf_counter()
+    for t in toks:
+        ref.attention_token_f32(q[t], kf, vf, H, G, d, n_ctx, P + t + 1, np.float32(scale))
+        flops += 4.0 * d * H * (P + t + 1)
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                sample=f"{done} query tokens x {H} heads at depth {P} of layer 0 "
+                       f"({flops / 1e9:.2f} GFLOP in {dt:.1f} s), reference loop order, fp32 cache")
+
+
+def cpu_baseline_decode(ref, q, k, v, H, G, d, n_ctx, L, scale):
+    kf = ref.fp16_to_fp32(k)
+    vf = ref.fp16_to_fp32(v)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ref.attention_token_f32(q, kf, vf, H, G, d, n_ctx, L, np.float32(scale))
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 64:
+            break
+    dt = time.perf_counter() - t0
+    # the CPU backend keeps an fp32 cache; the bytes counted are the fp16 bytes of the same positions
+    return dict(value=decode_bytes(H, G, d, L) * reps / dt / 1e9, unit="GB/s", cores=1, kind="port",
+                sample=f"{reps} decode steps of layer 0 at L={L} in {dt:.1f} s, reference loop order, fp32 cache")
+
+
+def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
+    from oracle import ref
+    from util import rel_err
+
+    shape_name, _, n_ctx, chunks = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    H, G, d, layers = s["H"], s["G"], s["d"], s["layers"]
+    scale = float(1.0 / np.sqrt(d))
+    stacks = []
+    for ci, (P, B) in enumerate(chunks):
+        stack = []
+        for l in range(layers):
+            q, k, v = make_layer(torch, 1000 * ci + l, H, G, d, n_ctx, P + B, B, s["outliers"])
+            stack.append((q, k, v, torch.empty((B, H, d), dtype=torch.float32, device="cuda")))
+        stacks.append(stack)
+
+    def one_step(events=None):
+        for ci, (P, B) in enumerate(chunks):
+            if events is not None:
+                events[ci][0].record()
+            for q, k, v, out in stacks[ci]:
+                kernels.flash_attention(q, k, v, out, H, G, d, n_ctx, P, B, scale)
+            if events is not None:
+                events[ci][1].record()
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in chunks]
+           for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        one_step(evs[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    flops_step = sum(prefill_flops(H, d, P, B) for P, B in chunks) * layers
+    per_chunk = []
+    for ci, (P, B) in enumerate(chunks):
+        ms = sum(evs[i][ci][0].elapsed_time(evs[i][ci][1]) for i in range(steps)) / (steps * layers)
+        f = prefill_flops(H, d, P, B)
+        per_chunk.append(dict(P=P, B=B, launch_us=ms * 1e3, tflops=f / (ms * 1e-3) / 1e12,
+                              frac=f / (ms * 1e-3) / PEAK_FLOPS))
+    dom = max(range(len(chunks)), key=lambda ci: prefill_flops(H, d, *chunks[ci]))
+    P, B = chunks[dom]
+    q, k, v, out = stacks[dom][0]
+    err = parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, P, B, scale)
+    res = dict(
+        value=flops_step * steps / wall / 1e12, unit="TFLOP/s", ms_per_step=wall / steps * 1e3,
+        config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_ctx=n_ctx,
+                    chunks=[list(c) for c in chunks], flops_per_step=flops_step),
+        roofline=dict(bound="mfma", achieved=per_chunk[dom]["tflops"], peak=PEAK_FLOPS / 1e12, unit="TFLOP/s",
+                      frac=per_chunk[dom]["frac"], traffic=None,
+                      kernel=f"fa_fwd_kernel prefill P={P} B={B}", launch_us=per_chunk[dom]["launch_us"],
+                      flops_per_launch=prefill_flops(H, d, P, B)),
+        per_chunk=per_chunk,
+        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="sampled, layer 0, vs CPU oracle"),
+    )
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline_prefill(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
+                                                   v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, P, B, scale)
+    return res
+
+
+def run_decode(torch, kernels, name, steps, warmup, with_cpu):
+    from oracle import ref
+    from util import rel_err
+
+    shape_name, _, n_ctx, L = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    H, G, d, layers = s["H"], s["G"], s["d"], s["layers"]
+    scale = float(1.0 / np.sqrt(d))
+    bytes_layer = decode_bytes(H, G, d, L)
+    # The chip has 256 MB of last-level (Infinity) cache: rotate enough independent stacks that
+    # a sweep exceeds it, so the timed loop streams from HBM.
+    n_stacks = max(1, int(np.ceil(600e6 / (bytes_layer * layers))))
+    stacks = []
+    for si in range(n_stacks):
+        stack = []
+        for l in range(layers):
+            q, k, v = make_layer(torch, 5000 + 100 * si + l, H, G, d, n_ctx, L, 1, s["outliers"])
+            stack.append((q[0].contiguous(), k, v, torch.empty((H, d), dtype=torch.float32, device="cuda")))
+        stacks.append(stack)
+    dpos = torch.tensor([L - 1], dtype=torch.int32, device="cuda")
+
+    def one_stack(si):
+        for q, k, v, out in stacks[si]:
+            kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
+
+    # eager
+    for i in range(warmup):
+        one_stack(i % n_stacks)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        one_stack(i % n_stacks)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_eager = time.perf_counter() - t0
+    dev_eager_ms = e0.elapsed_time(e1)
+
+    # one HIP graph per stack, as the engine replays its decode step (reference src/model_gpu.cu:295-344)
+    graphs = []
+    for si in range(n_stacks):
+        g = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(g):
+                kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+                one_stack(si)
+        finally:
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+        graphs.append(g)
+    for i in range(warmup):
+        graphs[i % n_stacks].replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        graphs[i % n_stacks].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_graph = time.perf_counter() - t0
+    dev_graph_ms = e0.elapsed_time(e1)
+
+    q, k, v, out = stacks[(steps - 1) % n_stacks][0]
+    rows = np.array([(0, h) for h in range(H)], np.int32)
+    want = ref.flash_attention_rows(q.cpu().numpy()[None], k.view(torch.uint16).cpu().numpy(),
+                                    v.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, L - 1,
+                                    np.float32(scale))
+    err = rel_err(out.cpu().numpy(), want)
+    wall = min(wall_graph, wall_eager)
+    launch_us = min(dev_graph_ms, dev_eager_ms) * 1e3 / (steps * layers)
+    res = dict(
+        value=bytes_layer * layers * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+        config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_ctx=n_ctx, L=L,
+                    bytes_per_step=bytes_layer * layers, stacks_rotated=n_stacks,
+                    splits=kernels.decode_splits(H, G, d, n_ctx)),
+        roofline=dict(bound="hbm", achieved=bytes_layer / (launch_us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9,
+                      unit="GB/s", frac=bytes_layer / (launch_us * 1e-6) / PEAK_BYTES, traffic=None,
+                      kernel="fa_fwd_kernel decode split + fa_decode_combine_kernel (per layer, incl. launch gaps)",
+                      launch_us=launch_us, bytes_per_launch=bytes_layer),
+        eager=dict(ms_per_step=wall_eager / steps * 1e3, device_ms_per_step=dev_eager_ms / steps),
+        graph=dict(ms_per_step=wall_graph / steps * 1e3, device_ms_per_step=dev_graph_ms / steps),
+        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="all heads, layer 0, vs CPU oracle"),
+    )
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline_decode(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
+                                                  v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, L, scale)
+    del stacks, graphs
+    torch.cuda.empty_cache()
+    return res
+
+
+def run(torch, kernels, name, steps, warmup, with_cpu):
+    kind = WORKLOADS[name][1]
+    fn = run_prefill if kind == "prefill" else run_decode
+    return fn(torch, kernels, name, steps, warmup, with_cpu)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="qwen1.5b-prefill512", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-also", action="store_true", help="skip the extra north-star workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the path has no cross-GPU part); use --gpus 1")
+
+    import torch
+
+    from orin_llm_amd import kernels
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    kernels.init(0)
+    kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+
+    main_res = run(torch, kernels, args.workload, args.steps, args.warmup, not args.no_cpu)
+    line = dict(
+        metric="prefill attn TFLOP/s + decode attn HBM GB/s (% of peak), Qwen2.5-1.5B GQA",
+        value=main_res.pop("value"), unit=main_res.pop("unit"), n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=main_res.pop("ms_per_step"), higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="f16", data="synthetic",
+    )
+    line.update(main_res)
+    if not args.no_also:
+        also = []
+        for name in ALSO:
+            if name == args.workload:
+                continue
+            r = run(torch, kernels, name, max(3, min(args.steps, 10)), min(args.warmup, 2), False)
+            also.append(dict(workload=name, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
+                             roofline=r["roofline"], parity=r["parity"],
+                             **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {})))
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
