@@ -30,15 +30,31 @@
 namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef __fp16 fp16x4 __attribute__((ext_vector_type(4)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;             // waves per workgroup
-constexpr int kThreads = kWaves * 64;
+constexpr int kPrefillWaves = 4;      // waves per prefill workgroup (one per SIMD: the kernel fills the register file)
+constexpr int kDecodeWaves = 8;       // waves per decode workgroup (two per SIMD, one workgroup per CU)
 constexpr int kTile = 32;             // KV rows per wave tile
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kPShift = 12.0f;      // P is scaled by 2^12 before fp16 rounding (keeps small weights normal)
+// Softmax weights are computed against a reference maximum that is only moved when a
+// tile's maximum exceeds it by more than kLazy (log2 units), so the O accumulators are
+// rescaled on a handful of early tiles instead of every tile.  P = 2^(s - m_ref + kPShift)
+// therefore lies in (0, 2^(kLazy + kPShift)] = (0, 2^15], inside fp16 range, and the
+// common factor cancels in O / l.
+constexpr float kLazy = 8.0f;
+constexpr float kPShift = 7.0f;
 constexpr size_t kWorkspaceBytes = 8u << 20;
-constexpr int kMaxSplits = 512;
+constexpr int kMaxSplits = 256;
+#ifndef FA_PREFILL_KDIRECT
+#define FA_PREFILL_KDIRECT 0
+#endif
+#ifndef FA_DECODE_KDIRECT
+#define FA_DECODE_KDIRECT 1
+#endif
+constexpr bool kPrefillKDirect = FA_PREFILL_KDIRECT;
+constexpr bool kDecodeKDirect = FA_DECODE_KDIRECT;
 
 struct FaArgs {
     const float* q;
@@ -54,20 +70,54 @@ struct FaArgs {
     int n_hgroups;     // head groups per KV head
     int n_ttiles;      // prefill: token tiles
     int n_splits;      // decode: KV splits
-    float scale_log2e;
+    float c;           // |scale| * log2(e), clamped away from zero
+    float qsign;       // sign of scale, folded into Q
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// All-reduce over the four 16-lane groups of a wave (lanes l, l^16, l^32, l^48) with the
+// gfx950 lane-swap instructions: v_permlane32_swap exchanges the upper half of one register
+// with the lower half of the other, v_permlane16_swap does the same for odd/even 16-lane rows.
 __device__ __forceinline__ float xor_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
 }
 __device__ __forceinline__ float xor_sum(float v) {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(s.x) + __uint_as_float(s.y);
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(s.x) + __uint_as_float(s.y);
+}
+
+// 16-byte load through a buffer descriptor: the hardware returns zeros for offsets at or
+// past the descriptor's byte count, so cache rows beyond the visible range (which may hold
+// anything, NaN patterns included) are never fetched and need no branch.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+// (The whole offset travels in the vector operand: the scalar offset operand is not range-checked.)
+// STREAM marks data that is read once (decode): the load carries the non-temporal hint so the
+// stream does not displace useful lines in L2 / Infinity Cache (measured 5-7% faster).
+template <bool STREAM>
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, STREAM ? 2 : 0);
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element (i % 4) of the
+// 8 bytes addressed by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 -- a 4x16 transpose on the way
+// out of LDS.  With lane i pointing at row (i / 4), 8-byte column (i % 4) of a row-major
+// fp16 tile, lane i ends up with rows 0..3 at column i: an MFMA operand whose k index runs
+// down the tile's rows.
+__device__ __forceinline__ h4 lds_read_tr(const unsigned char* p) {
+    const fp16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+        (__attribute__((address_space(3))) fp16x4*)(p));
+    return __builtin_bit_cast(h4, t);
 }
 
 // Orders this wave's LDS writes before its later LDS reads (lanes of one wave
@@ -78,28 +128,33 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int D, int NQB>
+template <int D, int NQB, int NW, bool KDIRECT>
 struct Geom {
     static constexpr int kSteps = D / 32;            // MFMA k-steps over head_dim
     static constexpr int kDBlk = D / 16;             // 16-wide output blocks over head_dim
-    static constexpr int kRowB = D * 2 + 16;         // bytes per KV row in LDS (16 B pad: conflict-free b128 reads)
+    static constexpr int kRowBK = D * 2 + 16;        // bytes per K row in LDS (16 B pad: conflict-free b128 row reads)
+    static constexpr int kRowBV = D * 2 + 32;        // bytes per V row in LDS (32 B pad: spreads the transposing reads)
     static constexpr int kChunksPerRow = D / 8;      // 16-byte chunks per KV row
     static constexpr int kLoads = kTile * kChunksPerRow / 64; // 16-byte loads per lane per matrix per tile
-    static constexpr int kTileB = kTile * kRowB;     // bytes of one K (or V) tile in LDS
+    static constexpr int kTileBK = kTile * kRowBK;   // bytes of one K tile in LDS
+    static constexpr int kTileBV = kTile * kRowBV;   // bytes of one V tile in LDS
     static constexpr int kOStride = D + 4;           // floats per column in the merge buffer
     static constexpr int kMergeB = NQB * 16 * kOStride * 4;
-    static constexpr int kWaveB = (2 * kTileB > kMergeB) ? 2 * kTileB : kMergeB;
-    static constexpr int kMlOff = kWaves * kWaveB;   // (m, l) per wave per column follow the wave slices
-    static constexpr int kLdsB = kMlOff + kWaves * NQB * 16 * 2 * 4;
+    static constexpr int kTilesB = (KDIRECT ? 0 : kTileBK) + kTileBV; // K skips LDS when it is loaded in operand order
+    static constexpr int kWaveB = (kTilesB > kMergeB) ? kTilesB : kMergeB;
+    static constexpr int kMlOff = NW * kWaveB;       // (m, l) per wave per column follow the wave slices
+    static constexpr int kLdsB = kMlOff + NW * NQB * 16 * 2 * 4;
 };
 
 // D: head_dim; NQB: 16-column query blocks per workgroup; TQ: tokens per workgroup
 // (column c = local_head * TQ + local_token); PRECISE: carry Q and P as fp16 hi+lo
 // pairs (decode, where the matrix pipe is idle anyway); DECODE: position from *d_pos,
 // KV splits across workgroups, partial outputs.
-template <int D, int NQB, int TQ, bool PRECISE, bool DECODE>
-__global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
-    using G = Geom<D, NQB>;
+template <int D, int NQB, int TQ, bool PRECISE, bool DECODE, bool KDIRECT>
+__global__ __launch_bounds__((DECODE ? kDecodeWaves : kPrefillWaves) * 64) void fa_fwd_kernel(const FaArgs a) {
+    constexpr int kWaves = DECODE ? kDecodeWaves : kPrefillWaves;
+    constexpr int kThreads = kWaves * 64;
+    using G = Geom<D, NQB, kWaves, KDIRECT>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -133,12 +188,43 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
     const int kv_end = n_past + tok_hi;     // the workgroup's columns see rows [0, kv_end) at most
     const int full_end = n_past + t0 + 1;   // rows below this are visible to every column
     const int n_tiles = (kv_end + kTile - 1) / kTile;
-    int tile_lo = 0, tile_hi = n_tiles;
-    if (DECODE) {
-        const int tps = (n_tiles + a.n_splits - 1) / a.n_splits;
-        tile_lo = id * tps;
-        tile_hi = (tile_lo + tps < n_tiles) ? tile_lo + tps : n_tiles;
-        if (tile_lo >= tile_hi) return; // inactive split: the combine kernel never reads it
+    // Wave w of split s takes tiles s*4 + w, then every (4 * n_splits)-th tile after it.
+    const int tile_first = (DECODE ? id * kWaves : 0) + wave;
+    const int tile_step = DECODE ? kWaves * a.n_splits : kWaves;
+    if (DECODE && id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
+
+    unsigned char* const ks = smem + wave * G::kWaveB;
+    unsigned char* const vs = ks + (KDIRECT ? 0 : G::kTileBK);
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
+
+    // K: either coalesced 16-byte chunks bound for LDS, or (KDIRECT) straight into MFMA A-operand
+    // order -- lane (col, grp) takes row t*16 + col, bytes (kk*4 + grp)*16 .. +16 -- so that the
+    // score product needs no LDS round trip.  V always goes through LDS (it is read transposed).
+    constexpr int kKRegs = KDIRECT ? 2 * G::kSteps : G::kLoads;
+    u32x4 kreg[kKRegs], vreg[G::kLoads];
+    auto fetch_k = [&](int tile) {
+        const int soff = tile * kTile * D * 2;
+        if (KDIRECT) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int kk = 0; kk < G::kSteps; ++kk)
+                    kreg[t * G::kSteps + kk] = buf_load16<DECODE>(krs, soff + (t * 16 + col) * D * 2 + (kk * 4 + grp) * 16);
+        } else {
+#pragma unroll
+            for (int i = 0; i < G::kLoads; ++i) kreg[i] = buf_load16<DECODE>(krs, soff + (i * 64 + lane) * 16);
+        }
+    };
+    auto fetch_v = [&](int tile) {
+        const int soff = tile * kTile * D * 2;
+#pragma unroll
+        for (int i = 0; i < G::kLoads; ++i) vreg[i] = buf_load16<DECODE>(vrs, soff + (i * 64 + lane) * 16);
+    };
+    int tile = tile_first;
+    if (tile < n_tiles) { // in flight while the query columns are loaded and converted
+        fetch_k(tile);
+        fetch_v(tile);
     }
 
     // ---- query columns -> B operands (fp16, optionally hi + lo) ----
@@ -153,6 +239,7 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
         const bool valid = (hl < a.r) && (tok < batch);
         limit[qb] = valid ? n_past + tok + 1 : 0x7fffffff;
         const float* qp = a.q + ((size_t)(valid ? tok : 0) * a.n_head + (size_t)(valid ? kvh * a.r + hl : 0)) * D;
+        const float qmul = valid ? a.qsign : 0.0f;
 #pragma unroll
         for (int kk = 0; kk < G::kSteps; ++kk) {
             const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
@@ -161,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
             h8 hi, lo;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float xe = valid ? x[e] : 0.0f;
+                const float xe = x[e] * qmul;
                 hi[e] = (_Float16)xe;
                 lo[e] = (_Float16)(xe - (float)hi[e]);
             }
@@ -170,72 +257,69 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
         }
     }
 
-    unsigned char* const ks = smem + wave * G::kWaveB;
-    unsigned char* const vs = ks + G::kTileB;
-    const _Float16* const kbase = reinterpret_cast<const _Float16*>(a.kc) + (size_t)kvh * a.n_ctx * D;
-    const _Float16* const vbase = reinterpret_cast<const _Float16*>(a.vc) + (size_t)kvh * a.n_ctx * D;
-
-    float m_run[NQB], l_run[NQB];
+    // m_ref: reference maximum of the raw scores (S units, before the scale); l_run: this lane's
+    // share of the row sum; o: O^T accumulators, lane (col, grp) holds head_dim rows db*16 + grp*4 + i.
+    float m_ref[NQB], l_run[NQB];
     f4 o[NQB][G::kDBlk];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        m_run[qb] = -INFINITY;
+        m_ref[qb] = -INFINITY;
         l_run[qb] = 0.0f;
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db) o[qb][db] = f4{0.f, 0.f, 0.f, 0.f};
     }
 
-    uint4 kreg[G::kLoads], vreg[G::kLoads];
-    auto fetch = [&](int tile) {
-#pragma unroll
-        for (int i = 0; i < G::kLoads; ++i) {
-            const int c = i * 64 + lane;
-            const int row = tile * kTile + c / G::kChunksPerRow;
-            const int ch = c % G::kChunksPerRow;
-            if (row < kv_end) { // rows past the visible range are never read: the cache tail may hold anything
-                kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)row * D + ch * 8);
-                vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)row * D + ch * 8);
-            } else {
-                kreg[i] = uint4{0u, 0u, 0u, 0u};
-                vreg[i] = uint4{0u, 0u, 0u, 0u};
-            }
-        }
-    };
+    // per-lane LDS read offsets
+    const int k_rd = col * G::kRowBK + grp * 16;                              // + t*16 rows, + kk*64 bytes
+    const int v_rd = (grp * 4 + (col >> 2)) * G::kRowBV + (col & 3) * 8;      // + h*16 rows, + db*32 bytes
 
-    int tile = tile_lo + wave;
-    if (tile < tile_hi) fetch(tile);
-    for (; tile < tile_hi; tile += kWaves) {
+    for (; tile < n_tiles; tile += tile_step) {
+        const bool more = tile + tile_step < n_tiles;
         // registers -> this wave's LDS slice
 #pragma unroll
         for (int i = 0; i < G::kLoads; ++i) {
             const int c = i * 64 + lane;
-            const int off = (c / G::kChunksPerRow) * G::kRowB + (c % G::kChunksPerRow) * 16;
-            *reinterpret_cast<uint4*>(ks + off) = kreg[i];
-            *reinterpret_cast<uint4*>(vs + off) = vreg[i];
+            if (!KDIRECT)
+                *reinterpret_cast<u32x4*>(ks + (c / G::kChunksPerRow) * G::kRowBK + (c % G::kChunksPerRow) * 16) = kreg[i];
+            *reinterpret_cast<u32x4*>(vs + (c / G::kChunksPerRow) * G::kRowBV + (c % G::kChunksPerRow) * 16) = vreg[i];
         }
-        if (tile + kWaves < tile_hi) fetch(tile + kWaves);
+        if (!KDIRECT && more) fetch_k(tile + tile_step);
+        if (more) fetch_v(tile + tile_step);
         wave_lds_sync();
 
         // ---- S^T = K Q^T : rows = KV row (sub-tile t, row col), columns = query column ----
         f4 s[2][NQB];
+        f4 s2[PRECISE ? 2 : 1][PRECISE ? NQB : 1]; // the Q-lo product runs as its own accumulation chain
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) s[t][qb] = f4{0.f, 0.f, 0.f, 0.f};
+            for (int qb = 0; qb < NQB; ++qb) {
+                s[t][qb] = f4{0.f, 0.f, 0.f, 0.f};
+                if (PRECISE) s2[t][qb] = f4{0.f, 0.f, 0.f, 0.f};
+            }
 #pragma unroll
         for (int kk = 0; kk < G::kSteps; ++kk) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const h8 ka = *reinterpret_cast<const h8*>(ks + (t * 16 + col) * G::kRowB + (kk * 4 + grp) * 16);
+                h8 ka;
+                if (KDIRECT) ka = __builtin_bit_cast(h8, kreg[t * G::kSteps + kk]);
+                else ka = *reinterpret_cast<const h8*>(ks + k_rd + t * 16 * G::kRowBK + kk * 64);
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb) {
                     s[t][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[qb][kk], s[t][qb], 0, 0, 0);
-                    if (PRECISE) s[t][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[qb][kk], s[t][qb], 0, 0, 0);
+                    if (PRECISE) s2[t][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[qb][kk], s2[t][qb], 0, 0, 0);
                 }
             }
         }
+        if (PRECISE) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb) s[t][qb] += s2[t][qb];
+        }
+        if (KDIRECT && more) fetch_k(tile + tile_step); // the operand registers are free again
 
-        // ---- online softmax; lane (col, grp) holds rows t*16 + grp*4 + i of its column ----
+        // ---- softmax weights; lane (col, grp) holds rows t*16 + grp*4 + i of its column ----
         const bool need_mask = (tile * kTile + kTile > full_end);
         h8 phi[NQB];
         h8 plo[PRECISE ? NQB : 1];
@@ -245,7 +329,7 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[t * 4 + i] = s[t][qb][i] * a.scale_log2e;
+                for (int i = 0; i < 4; ++i) v[t * 4 + i] = s[t][qb][i];
             if (need_mask) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
@@ -255,40 +339,43 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
                         if (row >= limit[qb]) v[t * 4 + i] = -INFINITY;
                     }
             }
-            float mx = v[0];
+            float mx = fmaxf(fmaxf(v[0], v[1]), v[2]);
+            mx = fmaxf(fmaxf(mx, v[3]), v[4]);
+            mx = fmaxf(fmaxf(mx, v[5]), v[6]);
+            mx = xor_max(fmaxf(mx, v[7]));
+            // move the reference only when this tile's maximum is far above it (or it is unset)
+            const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                const float alpha = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f; // unset reference -> 0
+                if (move) m_ref[qb] = mx;
+                l_run[qb] *= alpha;
 #pragma unroll
-            for (int e = 1; e < 8; ++e) mx = fmaxf(mx, v[e]);
-            mx = xor_max(mx);
-            const float m_new = fmaxf(m_run[qb], mx);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float alpha = fast_exp2(m_run[qb] - m_use);
-            m_run[qb] = m_new;
+                for (int db = 0; db < G::kDBlk; ++db) o[qb][db] *= alpha;
+            }
+            // exponent = s*c - m_ref*c + shift; a column that has seen no visible row keeps weight 0
+            const float nb = (m_ref[qb] == -INFINITY) ? kPShift : kPShift - m_ref[qb] * a.c;
             float sum = 0.0f;
             h8 ph, pl;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = fast_exp2(v[e] - m_use + kPShift);
+                const float p = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
                 sum += p;
                 ph[e] = (_Float16)p;
                 pl[e] = (_Float16)(p - (float)ph[e]);
             }
-            l_run[qb] = l_run[qb] * alpha + sum;
+            l_run[qb] += sum;
             phi[qb] = ph;
             if (PRECISE) plo[qb] = pl;
-#pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db) o[qb][db] *= alpha;
         }
 
         // ---- O^T += V^T P : rows = head_dim index, columns = query column, k = the tile's 32 KV rows
-        //      in the order (grp, t, i) that matches the layout P already has ----
+        //      in the order (grp, t, i) that matches the layout P already has.  The LDS transpose
+        //      read hands lane (col, grp) the four rows h*16 + grp*4 + 0..3 at head_dim index db*16 + col. ----
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db) {
-            h8 va;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int row = (e >> 2) * 16 + grp * 4 + (e & 3);
-                va[e] = *reinterpret_cast<const _Float16*>(vs + row * G::kRowB + (db * 16 + col) * 2);
-            }
+            const h4 v0 = lds_read_tr(vs + v_rd + db * 32);
+            const h4 v1 = lds_read_tr(vs + v_rd + 16 * G::kRowBV + db * 32);
+            const h8 va = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) {
                 o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, phi[qb], o[qb][db], 0, 0, 0);
@@ -297,6 +384,10 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
         }
         wave_lds_sync(); // the slice is overwritten at the top of the next iteration
     }
+
+    float m_run[NQB]; // reference maximum in log2 units, as the merge steps expect
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) m_run[qb] = (m_ref[qb] == -INFINITY) ? -INFINITY : m_ref[qb] * a.c;
 
     // ---- merge the four waves through LDS ----
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
@@ -353,55 +444,82 @@ __global__ __launch_bounds__(kThreads) void fa_fwd_kernel(const FaArgs a) {
     }
 }
 
-// Log-sum-exp merge of the decode splits: one workgroup per query head.
+// Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
+// head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the
+// position, the (m, l) pairs and this thread's share of the partial outputs -- is issued
+// before anything is waited on, so the kernel is one memory round trip deep.  Slots of
+// splits that were inactive for this position hold stale data and are masked after the load.
 template <int D>
 __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) {
-    constexpr int kGroups = 256 / D;
-    __shared__ float sh_o[kGroups][D];
-    __shared__ float sh_m[kGroups];
-    __shared__ float sh_l[kGroups];
-    const int head = blockIdx.x;
-    const int d = threadIdx.x % D;
-    const int sg = threadIdx.x / D;
+    constexpr int kSlices = D / 32;
+    constexpr int kGroups = 8;
+    constexpr int kPer = kMaxSplits / kGroups; // partial-output loads per thread, at most
+    __shared__ float sh_w[kMaxSplits];
+    __shared__ float sh_red[kGroups][32];
+    __shared__ float sh_wave[4][2];
+    const int head = blockIdx.x / kSlices;
+    const int d = (blockIdx.x % kSlices) * 32 + (threadIdx.x & 31);
+    const int sg = threadIdx.x >> 5;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_splits = a.n_splits;
 
+    // loads first
+    const int s_mine = threadIdx.x; // kMaxSplits == 256 == blockDim.x
+    float m_s = -INFINITY, l_s = 0.0f;
+    if (s_mine < n_splits) {
+        const float2 ml = *reinterpret_cast<const float2*>(a.part_ml + ((size_t)s_mine * a.n_head + head) * 2);
+        m_s = ml.x;
+        l_s = ml.y;
+    }
+    float x[kPer];
+    const float* po = a.part_o + (size_t)head * D + d;
+    const size_t stride = (size_t)a.n_head * D;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int s = sg + j * kGroups;
+        x[j] = s < n_splits ? po[s * stride] : 0.0f;
+    }
     int p = *a.d_pos;
     p = p < 0 ? 0 : p;
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1;
     const int n_tiles = (npos + kTile - 1) / kTile;
-    const int tps = (n_tiles + a.n_splits - 1) / a.n_splits;
-    const int n_active = (n_tiles + tps - 1) / tps;
+    const int by_tiles = (n_tiles + kDecodeWaves - 1) / kDecodeWaves;
+    const int n_active = by_tiles < n_splits ? by_tiles : n_splits;
 
-    float m = -INFINITY, l = 0.0f, acc = 0.0f;
-    for (int s = sg; s < n_active; s += kGroups) {
-        const size_t pi = (size_t)s * a.n_head + head;
-        const float ms = a.part_ml[pi * 2 + 0];
-        const float ls = a.part_ml[pi * 2 + 1];
-        const float os = a.part_o[pi * D + d];
-        const float m_new = fmaxf(m, ms);
-        const float wa = fast_exp2(m - m_new);
-        const float wb = fast_exp2(ms - m_new);
-        acc = acc * wa + os * wb;
-        l = l * wa + ls * wb;
-        m = m_new;
+    // weights w_s = 2^(m_s - max m) and the total row sum
+    if (s_mine >= n_active) {
+        m_s = -INFINITY;
+        l_s = 0.0f;
     }
-    sh_o[sg][d] = acc;
-    if (d == 0) {
-        sh_m[sg] = m;
-        sh_l[sg] = l;
+    float m_all = m_s;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, off));
+    if (lane == 0) sh_wave[wave][0] = m_all;
+    __syncthreads();
+    m_all = fmaxf(fmaxf(sh_wave[0][0], sh_wave[1][0]), fmaxf(sh_wave[2][0], sh_wave[3][0]));
+    const float w = fast_exp2(m_s - m_all); // every active split has seen a visible row, so m_all is finite
+    sh_w[s_mine] = w;                       // 0 for inactive slots
+    float l_all = w * l_s;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) l_all += __shfl_xor(l_all, off);
+    if (lane == 0) sh_wave[wave][1] = l_all;
+    __syncthreads();
+    l_all = (sh_wave[0][1] + sh_wave[1][1]) + (sh_wave[2][1] + sh_wave[3][1]);
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int s = sg + j * kGroups;
+        if (s < n_active) acc = __builtin_fmaf(x[j], sh_w[s], acc);
     }
+    sh_red[sg][threadIdx.x & 31] = acc;
     __syncthreads();
     if (sg == 0) {
-        float m_all = sh_m[0];
+        float tot = 0.0f;
 #pragma unroll
-        for (int g = 1; g < kGroups; ++g) m_all = fmaxf(m_all, sh_m[g]);
-        float l_all = 0.0f, o_all = 0.0f;
-#pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-            const float w = fast_exp2(sh_m[g] - m_all); // a group with no split has m = -inf -> weight 0
-            l_all += sh_l[g] * w;
-            o_all += sh_o[g][d] * w;
-        }
-        a.out[(size_t)head * D + d] = l_all > 0.0f ? o_all / l_all : 0.0f;
+        for (int g = 0; g < kGroups; ++g) tot += sh_red[g][threadIdx.x];
+        a.out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
     }
 }
 
@@ -422,32 +540,43 @@ State g_state;
 
 inline int hip_code(hipError_t e) { return e == hipSuccess ? ORIN_FA_OK : ORIN_FA_E_HIP - (int)e; }
 
-template <int D, int NQB, int TQ, bool PRECISE, bool DECODE>
+// The kernels take max over raw scores and scale afterwards, which needs a positive
+// multiplier: the sign of `scale` moves into Q and a zero scale becomes a vanishing one.
+inline void set_scale(FaArgs& a, float scale) {
+    const float c = scale * kLog2e;
+    a.qsign = c < 0.0f ? -1.0f : 1.0f;
+    a.c = c < 0.0f ? -c : c;
+    if (!(a.c >= 1e-30f)) a.c = 1e-30f;
+}
+
+template <int D, int NQB, int TQ, bool PRECISE, bool DECODE, bool KDIRECT>
 int launch_fwd(const FaArgs& a, int grid) {
-    using G = Geom<D, NQB>;
-    hipLaunchKernelGGL((fa_fwd_kernel<D, NQB, TQ, PRECISE, DECODE>), dim3(grid), dim3(kThreads), G::kLdsB,
+    constexpr int kWaves = DECODE ? kDecodeWaves : kPrefillWaves;
+    using G = Geom<D, NQB, kWaves, KDIRECT>;
+    hipLaunchKernelGGL((fa_fwd_kernel<D, NQB, TQ, PRECISE, DECODE, KDIRECT>), dim3(grid), dim3(kWaves * 64), G::kLdsB,
                        g_state.stream, a);
     return hip_code(hipGetLastError());
 }
 
 // The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at
 // init so that no launch path touches function attributes (decode runs under capture).
-template <int D, int NQB, int TQ, bool PRECISE, bool DECODE>
+template <int D, int NQB, int TQ, bool PRECISE, bool DECODE, bool KDIRECT>
 hipError_t allow_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_kernel<D, NQB, TQ, PRECISE, DECODE>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, Geom<D, NQB>::kLdsB);
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_kernel<D, NQB, TQ, PRECISE, DECODE, KDIRECT>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               Geom<D, NQB, DECODE ? kDecodeWaves : kPrefillWaves, KDIRECT>::kLdsB);
 }
 
 template <int D>
 hipError_t allow_lds_all() {
     hipError_t e;
-    if ((e = allow_lds<D, 1, 16, false, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 2, 16, false, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 16, false, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 4, 16, false, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 8, false, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 4, 8, false, false>()) != hipSuccess) return e;
-    return allow_lds<D, 1, 1, true, true>();
+    if ((e = allow_lds<D, 1, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 2, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 3, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 4, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 3, 8, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 4, 8, false, false, kPrefillKDirect>()) != hipSuccess) return e;
+    return allow_lds<D, 1, 1, true, true, kDecodeKDirect>();
 }
 
 template <int D>
@@ -465,12 +594,12 @@ int launch_prefill(FaArgs a) {
     a.n_ttiles = (a.batch + tq - 1) / tq;
     const int grid = a.n_kv * a.n_hgroups * a.n_ttiles;
     switch (nqb * 100 + tq) {
-        case 116: return launch_fwd<D, 1, 16, false, false>(a, grid);
-        case 216: return launch_fwd<D, 2, 16, false, false>(a, grid);
-        case 316: return launch_fwd<D, 3, 16, false, false>(a, grid);
-        case 416: return launch_fwd<D, 4, 16, false, false>(a, grid);
-        case 308: return launch_fwd<D, 3, 8, false, false>(a, grid);
-        default:  return launch_fwd<D, 4, 8, false, false>(a, grid);
+        case 116: return launch_fwd<D, 1, 16, false, false, kPrefillKDirect>(a, grid);
+        case 216: return launch_fwd<D, 2, 16, false, false, kPrefillKDirect>(a, grid);
+        case 316: return launch_fwd<D, 3, 16, false, false, kPrefillKDirect>(a, grid);
+        case 416: return launch_fwd<D, 4, 16, false, false, kPrefillKDirect>(a, grid);
+        case 308: return launch_fwd<D, 3, 8, false, false, kPrefillKDirect>(a, grid);
+        default:  return launch_fwd<D, 4, 8, false, false, kPrefillKDirect>(a, grid);
     }
 }
 
@@ -478,8 +607,8 @@ int decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     const int r = n_head / n_kv;
     const int n_hgroups = (r + 15) / 16;
     const int cus = g_state.cu_count > 0 ? g_state.cu_count : 256;
-    int s = (2 * cus) / (n_kv * n_hgroups);
-    const int by_ctx = (n_ctx + kWaves * kTile - 1) / (kWaves * kTile);
+    int s = cus / (n_kv * n_hgroups); // one 8-wave workgroup per CU
+    const int by_ctx = (n_ctx + kDecodeWaves * kTile - 1) / (kDecodeWaves * kTile);
     if (s > by_ctx) s = by_ctx;
     if (s > kMaxSplits) s = kMaxSplits;
     const size_t per_split = (size_t)n_head * (head_dim + 2) * sizeof(float);
@@ -498,9 +627,9 @@ int launch_decode(FaArgs a) {
         a.part_ml = a.part_o + (size_t)a.n_splits * a.n_head * D;
     }
     const int grid = a.n_kv * a.n_hgroups * a.n_splits;
-    int rc = launch_fwd<D, 1, 1, true, true>(a, grid);
+    int rc = launch_fwd<D, 1, 1, true, true, kDecodeKDirect>(a, grid);
     if (rc != ORIN_FA_OK || a.n_splits == 1) return rc;
-    hipLaunchKernelGGL(fa_decode_combine_kernel<D>, dim3(a.n_head), dim3(256), 0, g_state.stream, a);
+    hipLaunchKernelGGL(fa_decode_combine_kernel<D>, dim3(a.n_head * (D / 32)), dim3(256), 0, g_state.stream, a);
     return hip_code(hipGetLastError());
 }
 
@@ -510,6 +639,7 @@ int check_common(const void* q, const void* kc, const void* vc, const void* out,
     if (!q || !kc || !vc || !out) return ORIN_FA_E_INVALID;
     if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return ORIN_FA_E_INVALID;
     if (head_dim != 64 && head_dim != 128) return ORIN_FA_E_HEAD_DIM;
+    if ((long long)n_ctx * head_dim * 2 >= (1ll << 31)) return ORIN_FA_E_INVALID; // 32-bit byte offsets per KV head
     if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kc) | reinterpret_cast<uintptr_t>(vc) |
          reinterpret_cast<uintptr_t>(out)) & 15u)
         return ORIN_FA_E_INVALID; // 128-bit loads and stores
@@ -573,7 +703,7 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
     a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.n_past = n_past; a.batch = batch;
     a.r = n_head / n_kv;
     a.n_splits = 1;
-    a.scale_log2e = scale * kLog2e;
+    set_scale(a, scale);
     return head_dim == 128 ? launch_prefill<128>(a) : launch_prefill<64>(a);
 }
 
@@ -586,7 +716,7 @@ int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, f
     a.q = q; a.kc = kc; a.vc = vc; a.out = out; a.d_pos = d_pos;
     a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.batch = 1;
     a.r = n_head / n_kv;
-    a.scale_log2e = scale * kLog2e;
+    set_scale(a, scale);
     return head_dim == 128 ? launch_decode<128>(a) : launch_decode<64>(a);
 }
 
