@@ -444,6 +444,380 @@ __global__ __launch_bounds__((DECODE ? kDecodeWaves : kPrefillWaves) * 64) void 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Prefill: software-pipelined kernel.
+//
+// Same decomposition as above (4 waves split the KV tiles of one KV head between them and
+// share a block of NQB*16 query columns), but the three stages of a tile
+//     A: S = K Q^T (MFMA)      B: P = 2^(S*c - m) (VALU)      C: O += V^T P (MFMA)
+// run skewed -- iteration t issues A(t+1), B(t) and C(t-1), which are independent of one
+// another, so the matrix pipe works while the vector pipe exponentiates.  K rows are loaded
+// straight into MFMA operand order (two register sets, filled two tiles ahead); V tiles are
+// copied global->LDS by the load unit itself (no staging registers, two buffers per wave) in
+// an XOR-swizzled layout that both the 1 KB copy bursts and the transposing reads hit
+// conflict-free.  Each wave walks its tiles from the diagonal backwards, so the only tile
+// that can need the causal mask is handled in the prologue and the steady state is mask-free.
+// ---------------------------------------------------------------------------
+template <int D, int NQB>
+struct PGeom {
+    static constexpr int kSteps = D / 32;
+    static constexpr int kDBlk = D / 16;
+    static constexpr int kRowB = D * 2;               // bytes per K/V row in LDS (no padding; chunks are XOR-swizzled)
+    static constexpr int kChunks = D / 8;             // 16-byte chunks per row
+    static constexpr int kTileB = kTile * kRowB;      // one K or V tile
+    static constexpr int kCopies = kTileB / 1024;     // one LDS copy instruction moves 64 lanes x 16 B
+    static constexpr int kRowsPerCopy = 1024 / kRowB; // 4 (d=128) or 8 (d=64)
+    static constexpr int kKOff = 0;                   // wave slice: K buffers 0/1, then V buffers 0/1
+    static constexpr int kVOff = 2 * kTileB;
+    static constexpr int kOStride = D + 4;
+    static constexpr int kMergeB = NQB * 16 * kOStride * 4;
+    static constexpr int kWaveB = (4 * kTileB > kMergeB) ? 4 * kTileB : kMergeB;
+    static constexpr int kMlOff = kPrefillWaves * kWaveB;
+    static constexpr int kLdsB = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4;
+};
+
+template <int N> struct IntC { static constexpr int value = N; };
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor words for the global->LDS copies below: base address, stride 0, byte
+// count, raw 32-bit format.  Offsets at or past the byte count are not fetched.
+__device__ __forceinline__ i32x4 make_desc(const void* base, unsigned bytes) {
+    const unsigned long long b = reinterpret_cast<unsigned long long>(base);
+    return i32x4{(int)(unsigned)b, (int)((unsigned)(b >> 32) & 0xffffu), (int)bytes, 0x00020000};
+}
+
+// Four 1 KB global->LDS copies (buffer_load ... lds): lane l of copy i fetches 16 bytes at
+// global offset off_i + i*1024 and the load unit writes them to LDS byte lds_base + i*1024 +
+// l*16 (the immediate offset advances both addresses).  They count on the vector-memory
+// counter and complete in issue order; callers wait with s_waitcnt vmcnt(n).  Written as one
+// asm block so that M0 (the LDS base) cannot change between the copies.
+__device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int off_even, int off_odd) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "buffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
+        "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds\n\t"
+        "buffer_load_dwordx4 %1, %3, 0 offen offset:2048 lds\n\t"
+        "buffer_load_dwordx4 %2, %3, 0 offen offset:3072 lds"
+        :
+        : "s"(lds_base), "v"(off_even), "v"(off_odd), "s"(desc)
+        : "memory", "m0");
+}
+
+template <int D, int NQB, int TQ>
+__global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const FaArgs a) {
+    using G = PGeom<D, NQB>;
+    constexpr int kWaves = kPrefillWaves;
+    constexpr int kThreads = kWaves * 64;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = lane & 15;
+    const int grp = lane >> 4;
+
+    int id = blockIdx.x;
+    const int kvh = id % a.n_kv;
+    id /= a.n_kv;
+    const int hg = id % a.n_hgroups;
+    id /= a.n_hgroups;
+    const int n_past = a.n_past, batch = a.batch;
+    const int t0 = (a.n_ttiles - 1 - id) * TQ; // longest rows first
+    constexpr int kHeadsPerGroup = NQB * 16 / TQ;
+    const int head_lo = hg * kHeadsPerGroup;
+    const int tok_hi = (t0 + TQ < batch) ? t0 + TQ : batch;
+    const int kv_end = n_past + tok_hi;
+    const int full_end = n_past + t0 + 1;
+    const int n_tiles = (kv_end + kTile - 1) / kTile;
+    // Wave w owns tiles w, w+4, ...; step j visits them from the highest down.  Steps past the
+    // end map to negative tiles, whose copies fall outside the buffer descriptor and fetch nothing.
+    const int n_mine = n_tiles > wave ? (n_tiles - 1 - wave) / kWaves + 1 : 0;
+    auto tile_of = [&](int j) { return wave + kWaves * (n_mine - 1 - j); };
+
+    unsigned char* const ws = smem + wave * G::kWaveB; // this wave's LDS slice
+    // wave-uniform by construction; readfirstlane tells the compiler so (it has to live in a scalar register)
+    const unsigned ws_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ws);
+    const i32x4 kdesc = make_desc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
+    const i32x4 vdesc = make_desc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
+
+    // ---- per-lane offsets ----
+    // Copy: lane l of copy i lands at LDS byte i*1024 + l*16 = row i*R + l/C, physical chunk l%C,
+    // and physical chunk p of row r holds logical chunk p ^ (r & 7).
+    int g_off[2];
+    {
+        const int r_in = lane / G::kChunks, pc = lane % G::kChunks;
+#pragma unroll
+        for (int par = 0; par < 2; ++par) {
+            const int sw = (par * G::kRowsPerCopy + r_in) & 7;
+            g_off[par] = r_in * G::kRowB + ((pc ^ sw) & (G::kChunks - 1)) * 16;
+        }
+    }
+    constexpr int kOdd = (G::kRowsPerCopy == 4) ? 1 : 0;
+    // K operand read: lane (col, grp) takes row t*16 + col, logical chunk kk*4 + grp.
+    int k_rd[G::kSteps];
+#pragma unroll
+    for (int kk = 0; kk < G::kSteps; ++kk) k_rd[kk] = col * G::kRowB + (((kk * 4 + grp) ^ (col & 7)) * 16);
+    // V transposing read: lane (col, grp) addresses row grp*4 + col/4 (+16 for the second half),
+    // 8-byte column db*4 + col%4.
+    int v_rd[G::kDBlk];
+    {
+        const int r0 = grp * 4 + (col >> 2), sw = r0 & 7;
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db)
+            v_rd[db] = r0 * G::kRowB + (((db * 2 + ((col & 3) >> 1)) ^ sw) * 16) + (col & 1) * 8;
+    }
+
+    auto copy_tile = [&](i32x4 desc, unsigned lds_dst, int tile) { // kCopies (4 or 8) copies
+        const int base = tile * G::kTileB;
+        lds_copy_4k(desc, lds_dst, base + g_off[0], base + g_off[kOdd]);
+        if (G::kCopies > 4) lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[kOdd]);
+    };
+    auto fetch_k = [&](auto par, int tile) { copy_tile(kdesc, ws_addr + G::kKOff + decltype(par)::value * G::kTileB, tile); };
+    auto fetch_v = [&](auto par, int tile) { copy_tile(vdesc, ws_addr + G::kVOff + decltype(par)::value * G::kTileB, tile); };
+
+    // ---- state ----
+    h8 q[NQB][G::kSteps];
+    int limit[NQB];
+    float m_ref[NQB], l_run[NQB];
+    f4 o[NQB][G::kDBlk];
+    f4 s[2][2][NQB]; // [parity][sub-tile][query block]
+    h8 pw[2][NQB];   // [parity][query block]
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        m_ref[qb] = -INFINITY;
+        l_run[qb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db) o[qb][db] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    auto stage_a = [&](auto kpar, auto spar) { // S[spar] = K[kpar] Q^T
+        constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
+        const unsigned char* const kb = ws + G::kKOff + KP * G::kTileB;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) s[SP][t][qb] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps; ++kk)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const h8 ka = *reinterpret_cast<const h8*>(kb + t * 16 * G::kRowB + k_rd[kk]);
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb)
+                    s[SP][t][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, q[qb][kk], s[SP][t][qb], 0, 0, 0);
+            }
+    };
+
+    float alpha[NQB];
+    // P[par] = 2^(S[par]*c - m_ref*c + shift); returns whether any column moved its reference
+    auto stage_b = [&](auto par, auto masked, int tile) -> bool {
+        constexpr int P = decltype(par)::value;
+        bool any_move = false;
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            float v[8];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[t * 4 + i] = s[P][t][qb][i];
+            if (decltype(masked)::value) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = tile * kTile + t * 16 + grp * 4 + i;
+                        if (row >= limit[qb]) v[t * 4 + i] = -INFINITY;
+                    }
+            }
+            float mx = fmaxf(fmaxf(v[0], v[1]), v[2]);
+            mx = fmaxf(fmaxf(mx, v[3]), v[4]);
+            mx = fmaxf(fmaxf(mx, v[5]), v[6]);
+            mx = xor_max(fmaxf(mx, v[7]));
+            const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
+            alpha[qb] = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f;
+            if (move) m_ref[qb] = mx;
+            any_move |= move;
+            const float nb = (m_ref[qb] == -INFINITY) ? kPShift : kPShift - m_ref[qb] * a.c;
+            float sum = 0.0f;
+            h8 ph;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
+                sum += p;
+                ph[e] = (_Float16)p;
+            }
+            l_run[qb] = l_run[qb] * alpha[qb] + sum;
+            pw[P][qb] = ph;
+        }
+        return __builtin_amdgcn_ballot_w64(any_move) != 0;
+    };
+
+    auto stage_c = [&](auto par) { // O += V[par]^T P[par]
+        constexpr int P = decltype(par)::value;
+        const unsigned char* const vb = ws + G::kVOff + P * G::kTileB;
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db) {
+            const h4 v0 = lds_read_tr(vb + v_rd[db]);
+            const h4 v1 = lds_read_tr(vb + 16 * G::kRowB + v_rd[db]);
+            const h8 va = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb)
+                o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pw[P][qb], o[qb][db], 0, 0, 0);
+        }
+    };
+    auto rescale = [&]() {
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db) o[qb][db] *= alpha[qb];
+    };
+    // The copies are tracked by the vector-memory counter and complete in issue order: waiting
+    // until at most `newer` younger ones are outstanding guarantees a tile has landed.
+    auto wait_copies = [&](auto newer) {
+        constexpr int n = decltype(newer)::value;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (n & 15) | ((n >> 4) << 14)); // vmcnt(n), other counters untouched
+        wave_lds_sync();
+    };
+    constexpr int kC = G::kCopies;
+
+    if (n_mine > 0) {
+        // Zero the slice once: a copy whose rows lie past the visible range fetches nothing, and
+        // must not expose stale bit patterns (their weights are zero, and 0 * NaN is not).
+#pragma unroll
+        for (int i = 0; i < 4 * G::kTileB / 1024; ++i)
+            *reinterpret_cast<u32x4*>(ws + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the zero fill is done before the first copy can land
+        wave_lds_sync();
+
+        fetch_k(IntC<0>{}, tile_of(0));
+        fetch_v(IntC<0>{}, tile_of(0));
+        fetch_k(IntC<1>{}, tile_of(1));
+        fetch_v(IntC<1>{}, tile_of(1));
+
+        // ---- query columns -> B operands ----
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            const int c = qb * 16 + col;
+            const int tok = t0 + c % TQ;
+            const int hl = head_lo + c / TQ;
+            const bool valid = (hl < a.r) && (tok < batch);
+            limit[qb] = valid ? n_past + tok + 1 : 0x7fffffff;
+            const float* qp = a.q + ((size_t)(valid ? tok : 0) * a.n_head + (size_t)(valid ? kvh * a.r + hl : 0)) * D;
+            const float qmul = valid ? a.qsign : 0.0f;
+#pragma unroll
+            for (int kk = 0; kk < G::kSteps; ++kk) {
+                const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
+                const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                h8 hv;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(x[e] * qmul);
+                q[qb][kk] = hv;
+            }
+        }
+
+        // Copy issue order: K0 V0 K1 V1 | K2 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
+        // ---- step 0: the diagonal tile, the only one that can need the causal mask ----
+        const int R = n_mine - 1; // steps after step 0
+        wait_copies(IntC<3 * kC>{});               // K0 landed (V0 K1 V1 may be in flight)
+        stage_a(IntC<0>{}, IntC<0>{});             // S(0)
+        __builtin_amdgcn_s_waitcnt(0xC07F);        // its LDS reads have returned: K buffer 0 is free
+        fetch_k(IntC<0>{}, tile_of(2));
+        if (R > 0) {
+            wait_copies(IntC<2 * kC>{});           // K1 landed (V1 K2 may be in flight)
+            stage_a(IntC<1>{}, IntC<1>{});         // S(1)
+        }
+        if (tile_of(0) * kTile + kTile > full_end) stage_b(IntC<0>{}, IntC<1>{}, tile_of(0));
+        else stage_b(IntC<0>{}, IntC<0>{}, tile_of(0));
+        // (O is still zero: no rescale)
+
+        // ---- steps t >= 1: issue A(t+1), B(t), C(t-1).  `newer` = copies issued after K(t+1):
+        //      K(t+2) only at t == 1 (step 0 issued no V), V(t) and K(t+2) afterwards. ----
+        auto body = [&](auto tpar, auto has_next, auto newer, int t) {
+            constexpr int TP = decltype(tpar)::value; // t & 1
+            __builtin_amdgcn_s_waitcnt(0xC07F);                         // A(t)'s LDS reads have returned
+            fetch_k(IntC<TP>{}, tile_of(t + 2));                       // K(t+2) -> the buffer A(t) read
+            if (decltype(has_next)::value) {
+                wait_copies(newer);                                     // K(t+1) landed
+                stage_a(IntC<TP ^ 1>{}, IntC<TP ^ 1>{});                // S(t+1)
+            }
+            const bool moved = stage_b(IntC<TP>{}, IntC<0>{}, 0);       // P(t)
+            wait_copies(newer);                                         // V(t-1) is older than K(t+1)
+            stage_c(IntC<TP ^ 1>{});                                    // O += V(t-1)^T P(t-1)
+            __builtin_amdgcn_s_waitcnt(0xC07F);                         // its LDS reads have returned
+            fetch_v(IntC<TP ^ 1>{}, tile_of(t + 1));                   // V(t+1) -> the buffer C just read
+            if (moved) rescale();
+        };
+        if (R >= 1) {
+            if (R == 1) body(IntC<1>{}, IntC<0>{}, IntC<kC>{}, 1);
+            else body(IntC<1>{}, IntC<1>{}, IntC<kC>{}, 1);
+        }
+        int t = 2;
+        while (t + 1 < R) { // t even
+            body(IntC<0>{}, IntC<1>{}, IntC<2 * kC>{}, t);
+            body(IntC<1>{}, IntC<1>{}, IntC<2 * kC>{}, t + 1);
+            t += 2;
+        }
+        if (t < R) { // steps t (even) and t + 1 == R
+            body(IntC<0>{}, IntC<1>{}, IntC<2 * kC>{}, t);
+            body(IntC<1>{}, IntC<0>{}, IntC<2 * kC>{}, t + 1);
+        } else if (t == R) {
+            body(IntC<0>{}, IntC<0>{}, IntC<2 * kC>{}, t);
+        }
+        // ---- drain: C(R) ----
+        wait_copies(IntC<0>{});
+        if (R & 1) stage_c(IntC<1>{});
+        else stage_c(IntC<0>{});
+        __builtin_amdgcn_s_waitcnt(0xC07F); // every read of the tile buffers has returned: the merge reuses them
+        wave_lds_sync();
+    }
+
+    // ---- merge the four waves through LDS ----
+    float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
+    float* const obuf = reinterpret_cast<float*>(smem + wave * G::kWaveB);
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const float l_tot = xor_sum(l_run[qb]);
+        if (grp == 0) {
+            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = (m_ref[qb] == -INFINITY) ? -INFINITY : m_ref[qb] * a.c;
+            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 1] = l_tot;
+        }
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db)
+            *reinterpret_cast<f4*>(obuf + (qb * 16 + col) * G::kOStride + db * 16 + grp * 4) = o[qb][db];
+    }
+    __syncthreads();
+
+    constexpr int kCols = NQB * 16;
+    for (int idx = threadIdx.x; idx < kCols * (D / 4); idx += kThreads) {
+        const int c = idx / (D / 4);
+        const int d4 = (idx % (D / 4)) * 4;
+        const int tok = t0 + c % TQ;
+        const int hl = head_lo + c / TQ;
+        if (hl >= a.r || tok >= batch) continue;
+        float mw[kWaves], lw[kWaves];
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mw[w] = ml[(w * kCols + c) * 2 + 0];
+            lw[w] = ml[(w * kCols + c) * 2 + 1];
+            m_all = fmaxf(m_all, mw[w]);
+        }
+        float l_all = 0.0f;
+        f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float wgt = fast_exp2(mw[w] - m_all); // a wave that saw no visible row has m = -inf -> weight 0
+            l_all += lw[w] * wgt;
+            const f4 ow = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4);
+            acc += ow * wgt;
+        }
+        const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+        *reinterpret_cast<f4*>(a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D + d4) = acc * inv;
+    }
+}
+
 // Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
 // head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the
 // position, the (m, l) pairs and this thread's share of the partial outputs -- is issued
@@ -560,23 +934,33 @@ int launch_fwd(const FaArgs& a, int grid) {
 
 // The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at
 // init so that no launch path touches function attributes (decode runs under capture).
-template <int D, int NQB, int TQ, bool PRECISE, bool DECODE, bool KDIRECT>
-hipError_t allow_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_kernel<D, NQB, TQ, PRECISE, DECODE, KDIRECT>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                               Geom<D, NQB, DECODE ? kDecodeWaves : kPrefillWaves, KDIRECT>::kLdsB);
+template <int D, int NQB, int TQ>
+int launch_prefill_kernel(const FaArgs& a, int grid) {
+    constexpr int lds = PGeom<D, NQB>::kLdsB;
+    hipLaunchKernelGGL((fa_prefill_kernel<D, NQB, TQ>), dim3(grid), dim3(kPrefillWaves * 64), lds, g_state.stream, a);
+    return hip_code(hipGetLastError());
+}
+
+// The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at
+// init so that no launch path touches function attributes (decode runs under capture).
+template <int D, int NQB, int TQ>
+hipError_t allow_lds_prefill() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_prefill_kernel<D, NQB, TQ>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, PGeom<D, NQB>::kLdsB);
 }
 
 template <int D>
 hipError_t allow_lds_all() {
     hipError_t e;
-    if ((e = allow_lds<D, 1, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 2, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 4, 16, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 8, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 4, 8, false, false, kPrefillKDirect>()) != hipSuccess) return e;
-    return allow_lds<D, 1, 1, true, true, kDecodeKDirect>();
+    if ((e = allow_lds_prefill<D, 1, 16>()) != hipSuccess) return e;
+    if ((e = allow_lds_prefill<D, 2, 16>()) != hipSuccess) return e;
+    if ((e = allow_lds_prefill<D, 3, 16>()) != hipSuccess) return e;
+    if ((e = allow_lds_prefill<D, 4, 16>()) != hipSuccess) return e;
+    if ((e = allow_lds_prefill<D, 3, 8>()) != hipSuccess) return e;
+    if ((e = allow_lds_prefill<D, 4, 8>()) != hipSuccess) return e;
+    return hipFuncSetAttribute(
+        reinterpret_cast<const void*>(fa_fwd_kernel<D, 1, 1, true, true, kDecodeKDirect>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, Geom<D, 1, kDecodeWaves, kDecodeKDirect>::kLdsB);
 }
 
 template <int D>
@@ -594,12 +978,12 @@ int launch_prefill(FaArgs a) {
     a.n_ttiles = (a.batch + tq - 1) / tq;
     const int grid = a.n_kv * a.n_hgroups * a.n_ttiles;
     switch (nqb * 100 + tq) {
-        case 116: return launch_fwd<D, 1, 16, false, false, kPrefillKDirect>(a, grid);
-        case 216: return launch_fwd<D, 2, 16, false, false, kPrefillKDirect>(a, grid);
-        case 316: return launch_fwd<D, 3, 16, false, false, kPrefillKDirect>(a, grid);
-        case 416: return launch_fwd<D, 4, 16, false, false, kPrefillKDirect>(a, grid);
-        case 308: return launch_fwd<D, 3, 8, false, false, kPrefillKDirect>(a, grid);
-        default:  return launch_fwd<D, 4, 8, false, false, kPrefillKDirect>(a, grid);
+        case 116: return launch_prefill_kernel<D, 1, 16>(a, grid);
+        case 216: return launch_prefill_kernel<D, 2, 16>(a, grid);
+        case 316: return launch_prefill_kernel<D, 3, 16>(a, grid);
+        case 416: return launch_prefill_kernel<D, 4, 16>(a, grid);
+        case 308: return launch_prefill_kernel<D, 3, 8>(a, grid);
+        default:  return launch_prefill_kernel<D, 4, 8>(a, grid);
     }
 }
 
