@@ -76,6 +76,7 @@ struct FaArgs {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+__device__ __forceinline__ float max2(float x, float y);
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
@@ -87,6 +88,12 @@ __device__ __forceinline__ float xor_max(float v) {
     v = fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
     s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+}
+__device__ __forceinline__ float xor_max_fast(float v) { // same, for inputs that are never NaN
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    float r = max2(__uint_as_float(s.x), __uint_as_float(s.y));
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(r), __float_as_uint(r), false, false);
+    return max2(__uint_as_float(s.x), __uint_as_float(s.y));
 }
 __device__ __forceinline__ float xor_sum(float v) {
     u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -471,12 +478,71 @@ struct PGeom {
     static constexpr int kVOff = 2 * kTileB;
     static constexpr int kOStride = D + 4;
     static constexpr int kMergeB = NQB * 16 * kOStride * 4;
-    static constexpr int kWaveB = (4 * kTileB > kMergeB) ? 4 * kTileB : kMergeB;
+    static constexpr int kScratchOff = 4 * kTileB;    // 1 KB per wave: 16 bytes per lane for the rare O rescale
+    static constexpr int kWaveB = (4 * kTileB + 1024 > kMergeB) ? 4 * kTileB + 1024 : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
     static constexpr int kLdsB = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4;
 };
 
 template <int N> struct IntC { static constexpr int value = N; };
+
+// Matrix instructions with the register file of each operand spelled out.  The prefill kernel
+// keeps its score accumulators in ordinary vector registers (the exponentials read them with no
+// copy) and its output accumulators in the accumulation-register file, and it fixes the issue
+// order of matrix and vector work by hand -- neither of which the builtin form allows.  The
+// price: the compiler knows nothing about the hazards of these.  (1) Result latency: every place
+// where a non-matrix instruction reads an accumulator is either a pipeline stage away or behind
+// settle().  (2) A matrix instruction must not read an operand in the two cycles after a vector
+// instruction wrote it, and the compiler is free to sink such a write (the fp16 conversion of P,
+// a register copy) right in front of the asm block: each block starts with the two wait states.
+__device__ __forceinline__ void mfma_v(f4& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "v"(b_op));
+}
+__device__ __forceinline__ void mfma_v_zero(f4& acc, h8 a_op, h8 b_op) { // acc = A B
+    // early clobber: the destination must not share registers with an operand that dies here
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "v"(b_op));
+}
+__device__ __forceinline__ void mfma_a(f4& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
+}
+// Lets the matrix pipe drain (32 wait states, more than any 16x16x32 result needs) and stops the
+// compiler from moving anything across.
+__device__ __forceinline__ void settle() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+// 16 bytes between LDS and the accumulation-register file, without a detour through vector
+// registers.  The output accumulators of the prefill kernel are only ever touched by these and
+// by mfma_a, which keeps them in that file for the whole kernel.
+__device__ __forceinline__ void lds_store_acc(unsigned lds_addr, const f4& acc) {
+    asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(lds_addr), "a"(acc) : "memory");
+}
+__device__ __forceinline__ void lds_load_acc(f4& acc, unsigned lds_addr) {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(acc) : "v"(lds_addr) : "memory");
+}
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(IntC<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// three-input maximum without the NaN-quieting moves the library fmaxf carries
+__device__ __forceinline__ float max3(float x, float y, float z) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
+    return r;
+}
+// (trailing wait state: the result may feed a lane-swap instruction, which must not read a
+// register in the cycle after a vector instruction wrote it, and the compiler cannot see that
+// this block is one)
+__device__ __forceinline__ float max2(float x, float y) {
+    float r;
+    asm("v_max_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
@@ -583,29 +649,39 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     f4 o[NQB][G::kDBlk];
     f4 s[2][2][NQB]; // [parity][sub-tile][query block]
     h8 pw[2][NQB];   // [parity][query block]
+    // Zero the slice once: a copy whose rows lie past the visible range fetches nothing, and must
+    // not expose stale bit patterns (their weights are zero, and 0 * NaN is not).  The output
+    // accumulators are cleared from the same zeros.
+#pragma unroll
+    for (int i = 0; i < (4 * G::kTileB + 1024) / 1024; ++i)
+        *reinterpret_cast<u32x4*>(ws + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the zero fill is done before the first copy can land
+    wave_lds_sync();
+    const unsigned scratch_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(ws + G::kScratchOff) + lane * 16;
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         m_ref[qb] = -INFINITY;
         l_run[qb] = 0.0f;
 #pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db) o[qb][db] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int db = 0; db < G::kDBlk; ++db) lds_load_acc(o[qb][db], scratch_addr);
     }
 
-    auto stage_a = [&](auto kpar, auto spar) { // S[spar] = K[kpar] Q^T
+    auto stage_a = [&](auto kpar, auto spar) { // S[spar] = K[kpar] Q^T (prologue form: not interleaved)
         constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
         const unsigned char* const kb = ws + G::kKOff + KP * G::kTileB;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) s[SP][t][qb] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < G::kSteps; ++kk)
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const h8 ka = *reinterpret_cast<const h8*>(kb + t * 16 * G::kRowB + k_rd[kk]);
 #pragma unroll
-                for (int qb = 0; qb < NQB; ++qb)
-                    s[SP][t][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, q[qb][kk], s[SP][t][qb], 0, 0, 0);
+                for (int qb = 0; qb < NQB; ++qb) {
+                    if (kk == 0) mfma_v_zero(s[SP][t][qb], ka, q[qb][kk]);
+                    else mfma_v(s[SP][t][qb], ka, q[qb][kk]);
+                    // With few query blocks the next k-step of the same accumulator is only a
+                    // couple of instructions away; give the result time to leave the pipe.
+                    if (2 * NQB < 8) asm volatile("s_nop 15");
+                }
             }
     };
 
@@ -630,10 +706,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                         if (row >= limit[qb]) v[t * 4 + i] = -INFINITY;
                     }
             }
-            float mx = fmaxf(fmaxf(v[0], v[1]), v[2]);
-            mx = fmaxf(fmaxf(mx, v[3]), v[4]);
-            mx = fmaxf(fmaxf(mx, v[5]), v[6]);
-            mx = xor_max(fmaxf(mx, v[7]));
+            float mx = max3(v[0], v[1], v[2]);
+            mx = max3(mx, v[3], v[4]);
+            mx = max3(mx, v[5], v[6]);
+            mx = xor_max_fast(max2(mx, v[7]));
             const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
             alpha[qb] = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f;
             if (move) m_ref[qb] = mx;
@@ -662,15 +738,25 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             const h4 v1 = lds_read_tr(vb + 16 * G::kRowB + v_rd[db]);
             const h8 va = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb)
-                o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pw[P][qb], o[qb][db], 0, 0, 0);
+            for (int qb = 0; qb < NQB; ++qb) mfma_a(o[qb][db], va, pw[P][qb]);
         }
     };
+    // Rare (a column's reference maximum moved): O *= alpha, one accumulator at a time through a
+    // 16-byte-per-lane LDS scratch so that O never becomes an operand of an ordinary vector instruction.
     auto rescale = [&]() {
+        settle(); // the last accumulation into O has left the matrix pipe
+        f4* const scratch = reinterpret_cast<f4*>(ws + G::kScratchOff) + lane;
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db) o[qb][db] *= alpha[qb];
+            for (int db = 0; db < G::kDBlk; ++db) {
+                lds_store_acc(scratch_addr, o[qb][db]);
+                f4 x = *scratch;
+                x *= alpha[qb];
+                *scratch = x;
+                lds_load_acc(o[qb][db], scratch_addr);
+            }
+        settle();
     };
     // The copies are tracked by the vector-memory counter and complete in issue order: waiting
     // until at most `newer` younger ones are outstanding guarantees a tile has landed.
@@ -682,14 +768,6 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     constexpr int kC = G::kCopies;
 
     if (n_mine > 0) {
-        // Zero the slice once: a copy whose rows lie past the visible range fetches nothing, and
-        // must not expose stale bit patterns (their weights are zero, and 0 * NaN is not).
-#pragma unroll
-        for (int i = 0; i < 4 * G::kTileB / 1024; ++i)
-            *reinterpret_cast<u32x4*>(ws + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the zero fill is done before the first copy can land
-        wave_lds_sync();
-
         fetch_k(IntC<0>{}, tile_of(0));
         fetch_v(IntC<0>{}, tile_of(0));
         fetch_k(IntC<1>{}, tile_of(1));
@@ -728,24 +806,112 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             wait_copies(IntC<2 * kC>{});           // K1 landed (V1 K2 may be in flight)
             stage_a(IntC<1>{}, IntC<1>{});         // S(1)
         }
+        settle();
         if (tile_of(0) * kTile + kTile > full_end) stage_b(IntC<0>{}, IntC<1>{}, tile_of(0));
         else stage_b(IntC<0>{}, IntC<0>{}, tile_of(0));
         // (O is still zero: no rescale)
 
-        // ---- steps t >= 1: issue A(t+1), B(t), C(t-1).  `newer` = copies issued after K(t+1):
-        //      K(t+2) only at t == 1 (step 0 issued no V), V(t) and K(t+2) afterwards. ----
+        // ---- steps t >= 1: A(t+1), B(t) and C(t-1) share one hand-ordered instruction stream.
+        // The 2 * kGroups/2 * NQB matrix instructions of A and C are cut into groups of NQB that
+        // share an LDS operand (A: one (k-step, sub-tile) of K; C: one 16-wide block of V^T),
+        // ordered A0 C0 A1 C1 ...; the vector work of B is cut into 16 sites per query block and
+        // each site is followed by its share of the matrix instructions, so the matrix pipe is
+        // fed while the exponentials run.  Operands are read from LDS two groups ahead.
+        // `newer` = copies issued after K(t+1): K(t+2) only at t == 1 (step 0 issued no V),
+        // V(t) and K(t+2) afterwards. ----
+        constexpr int kGroups = 2 * G::kSteps + G::kDBlk; // 2*kSteps == kDBlk
+        static_assert(2 * G::kSteps == G::kDBlk, "A and C groups alternate one to one");
         auto body = [&](auto tpar, auto has_next, auto newer, int t) {
             constexpr int TP = decltype(tpar)::value; // t & 1
+            constexpr bool HN = decltype(has_next)::value;
             __builtin_amdgcn_s_waitcnt(0xC07F);                         // A(t)'s LDS reads have returned
             fetch_k(IntC<TP>{}, tile_of(t + 2));                       // K(t+2) -> the buffer A(t) read
-            if (decltype(has_next)::value) {
-                wait_copies(newer);                                     // K(t+1) landed
-                stage_a(IntC<TP ^ 1>{}, IntC<TP ^ 1>{});                // S(t+1)
-            }
-            const bool moved = stage_b(IntC<TP>{}, IntC<0>{}, 0);       // P(t)
-            wait_copies(newer);                                         // V(t-1) is older than K(t+1)
-            stage_c(IntC<TP ^ 1>{});                                    // O += V(t-1)^T P(t-1)
-            __builtin_amdgcn_s_waitcnt(0xC07F);                         // its LDS reads have returned
+            wait_copies(newer);                                         // K(t+1) landed; V(t-1) is older
+            const unsigned char* const kb = ws + G::kKOff + (TP ^ 1) * G::kTileB;
+            const unsigned char* const vb = ws + G::kVOff + (TP ^ 1) * G::kTileB;
+            h8 gop[kGroups];
+            auto issue_read = [&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                if constexpr (g % 2 == 0) {
+                    constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
+                    if (HN) gop[g] = *reinterpret_cast<const h8*>(kb + tt * 16 * G::kRowB + k_rd[kk]);
+                } else {
+                    constexpr int db = g / 2;
+                    const h4 v0 = lds_read_tr(vb + v_rd[db]);
+                    const h4 v1 = lds_read_tr(vb + 16 * G::kRowB + v_rd[db]);
+                    gop[g] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+            };
+            auto ticket = [&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int g = i / NQB, m = i % NQB;
+                if constexpr (m == 0 && g + 2 < kGroups) issue_read(IntC<g + 2>{});
+                if constexpr (g % 2 == 0) {
+                    constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
+                    if (HN) {
+                        if constexpr (kk == 0) mfma_v_zero(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
+                        else mfma_v(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
+                    }
+                } else {
+                    mfma_a(o[m][g / 2], gop[g], pw[TP ^ 1][m]);
+                }
+            };
+            issue_read(IntC<0>{});
+            issue_read(IntC<1>{});
+            bool any_move = false;
+            static_for<0, NQB>([&](auto qbc) {
+                constexpr int qb = decltype(qbc)::value;
+                auto site = [&](auto jc) { // the matrix instructions that follow vector site j of this query block
+                    constexpr int j = decltype(jc)::value;
+                    constexpr int lo = qb * kGroups + j * kGroups / 16, hi = qb * kGroups + (j + 1) * kGroups / 16;
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<lo, hi>(ticket);
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+                float v[8];
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[tt * 4 + i] = s[TP][tt][qb][i];
+                float mx = max3(v[0], v[1], v[2]);
+                site(IntC<0>{});
+                mx = max3(mx, v[3], v[4]);
+                mx = max3(mx, v[5], v[6]);
+                site(IntC<1>{});
+                mx = max2(mx, v[7]);
+                {
+                    const u32x2 sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+                    mx = max2(__uint_as_float(sw.x), __uint_as_float(sw.y));
+                }
+                site(IntC<2>{});
+                {
+                    const u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+                    mx = max2(__uint_as_float(sw.x), __uint_as_float(sw.y));
+                }
+                site(IntC<3>{});
+                const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
+                site(IntC<4>{});
+                alpha[qb] = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f;
+                if (move) m_ref[qb] = mx;
+                any_move |= move;
+                const float nb = (m_ref[qb] == -INFINITY) ? kPShift : kPShift - m_ref[qb] * a.c;
+                site(IntC<5>{});
+                float sum = 0.0f;
+                h8 ph;
+                static_for<0, 8>([&](auto ec) {
+                    constexpr int e = decltype(ec)::value;
+                    const float pe = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
+                    sum += pe;
+                    ph[e] = (_Float16)pe;
+                    site(IntC<6 + e>{});
+                });
+                l_run[qb] = l_run[qb] * alpha[qb] + sum;
+                pw[TP][qb] = ph;
+                site(IntC<14>{});
+                site(IntC<15>{});
+            });
+            const bool moved = __builtin_amdgcn_ballot_w64(any_move) != 0;
+            __builtin_amdgcn_s_waitcnt(0xC07F);                         // C(t-1)'s LDS reads have returned
             fetch_v(IntC<TP ^ 1>{}, tile_of(t + 1));                   // V(t+1) -> the buffer C just read
             if (moved) rescale();
         };
@@ -767,15 +933,17 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         }
         // ---- drain: C(R) ----
         wait_copies(IntC<0>{});
+        settle(); // P(R) was converted just above
         if (R & 1) stage_c(IntC<1>{});
         else stage_c(IntC<0>{});
         __builtin_amdgcn_s_waitcnt(0xC07F); // every read of the tile buffers has returned: the merge reuses them
+        settle();                            // and O is out of the matrix pipe
         wave_lds_sync();
     }
 
     // ---- merge the four waves through LDS ----
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
-    float* const obuf = reinterpret_cast<float*>(smem + wave * G::kWaveB);
+    const unsigned obuf_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(smem + wave * G::kWaveB);
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const float l_tot = xor_sum(l_run[qb]);
@@ -785,7 +953,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         }
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db)
-            *reinterpret_cast<f4*>(obuf + (qb * 16 + col) * G::kOStride + db * 16 + grp * 4) = o[qb][db];
+            lds_store_acc(obuf_addr + ((qb * 16 + col) * G::kOStride + db * 16 + grp * 4) * 4, o[qb][db]);
     }
     __syncthreads();
 
