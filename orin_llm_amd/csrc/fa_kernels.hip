@@ -45,6 +45,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 // common factor cancels in O / l.
 constexpr float kLazy = 8.0f;
 constexpr float kPShift = 7.0f;
+constexpr float kUnsetRef = -1.0e30f; // prefill: reference maximum of a column that has seen no visible key yet
 constexpr size_t kWorkspaceBytes = 8u << 20;
 constexpr int kMaxSplits = 256;
 #ifndef FA_PREFILL_KDIRECT
@@ -660,7 +661,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const unsigned scratch_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(ws + G::kScratchOff) + lane * 16;
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        m_ref[qb] = -INFINITY;
+        m_ref[qb] = kUnsetRef;
         l_run[qb] = 0.0f;
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db) lds_load_acc(o[qb][db], scratch_addr);
@@ -710,11 +711,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             mx = max3(mx, v[3], v[4]);
             mx = max3(mx, v[5], v[6]);
             mx = xor_max_fast(max2(mx, v[7]));
-            const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
-            alpha[qb] = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f;
-            if (move) m_ref[qb] = mx;
+            const bool move = (mx - m_ref[qb]) * a.c > kLazy; // an unset reference is far below any score
+            alpha[qb] = fast_exp2(move ? (m_ref[qb] - mx) * a.c : 0.0f);
+            m_ref[qb] = move ? mx : m_ref[qb];
             any_move |= move;
-            const float nb = (m_ref[qb] == -INFINITY) ? kPShift : kPShift - m_ref[qb] * a.c;
+            const float nb = kPShift - m_ref[qb] * a.c;
             float sum = 0.0f;
             h8 ph;
 #pragma unroll
@@ -824,7 +825,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         auto body = [&](auto tpar, auto has_next, auto newer, int t) {
             constexpr int TP = decltype(tpar)::value; // t & 1
             constexpr bool HN = decltype(has_next)::value;
-            __builtin_amdgcn_s_waitcnt(0xC07F);                         // A(t)'s LDS reads have returned
+            // (Every LDS read of the previous step has been consumed by a matrix instruction that
+            // was issued before this point, so the K buffer A(t) read is free.)
             fetch_k(IntC<TP>{}, tile_of(t + 2));                       // K(t+2) -> the buffer A(t) read
             wait_copies(newer);                                         // K(t+1) landed; V(t-1) is older
             const unsigned char* const kb = ws + G::kKOff + (TP ^ 1) * G::kTileB;
@@ -858,61 +860,70 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             };
             issue_read(IntC<0>{});
             issue_read(IntC<1>{});
-            bool any_move = false;
+            // Matrix instruction tickets: NQB go to phase 0 (one per query block), the rest are
+            // spread over the 10 vector sites of each query block in phase 1.
+            constexpr int kPerQb = kGroups - 1;
+            auto tickets = [&](auto loc, auto hic) {
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<decltype(loc)::value, decltype(hic)::value>(ticket);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            // ---- phase 0: has any score outgrown its column's reference maximum?  Lane-local
+            // maxima only (no lane exchange, no execution-mask games: both stall the matrix pipe);
+            // the answer is "no" on all but the first few tiles.
+            float lmax[NQB];
+            float excess = -INFINITY;
             static_for<0, NQB>([&](auto qbc) {
                 constexpr int qb = decltype(qbc)::value;
-                auto site = [&](auto jc) { // the matrix instructions that follow vector site j of this query block
+                float mx = max3(s[TP][0][qb][0], s[TP][0][qb][1], s[TP][0][qb][2]);
+                mx = max3(mx, s[TP][0][qb][3], s[TP][1][qb][0]);
+                mx = max3(mx, s[TP][1][qb][1], s[TP][1][qb][2]);
+                mx = max2(mx, s[TP][1][qb][3]);
+                lmax[qb] = mx;
+                excess = max2(excess, (mx - m_ref[qb]) * a.c);
+                tickets(IntC<qb>{}, IntC<qb + 1>{});
+            });
+            bool moved = false;
+            if (__builtin_amdgcn_ballot_w64(excess > kLazy) != 0) {
+                moved = true;
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb) {
+                    const float mx = xor_max_fast(lmax[qb]);
+                    const bool move = (mx - m_ref[qb]) * a.c > kLazy;
+                    alpha[qb] = fast_exp2(move ? (m_ref[qb] - mx) * a.c : 0.0f);
+                    m_ref[qb] = move ? mx : m_ref[qb];
+                    l_run[qb] *= alpha[qb];
+                }
+            }
+            // ---- phase 1: P(t) = 2^(S*c - m_ref*c + shift), row sums, fp16 ----
+            static_for<0, NQB>([&](auto qbc) {
+                constexpr int qb = decltype(qbc)::value;
+                constexpr int base = NQB + qb * kPerQb;
+                auto site = [&](auto jc) {
                     constexpr int j = decltype(jc)::value;
-                    constexpr int lo = qb * kGroups + j * kGroups / 16, hi = qb * kGroups + (j + 1) * kGroups / 16;
-                    __builtin_amdgcn_sched_barrier(0);
-                    static_for<lo, hi>(ticket);
-                    __builtin_amdgcn_sched_barrier(0);
+                    tickets(IntC<base + j * kPerQb / 10>{}, IntC<base + (j + 1) * kPerQb / 10>{});
                 };
-                float v[8];
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) v[tt * 4 + i] = s[TP][tt][qb][i];
-                float mx = max3(v[0], v[1], v[2]);
-                site(IntC<0>{});
-                mx = max3(mx, v[3], v[4]);
-                mx = max3(mx, v[5], v[6]);
-                site(IntC<1>{});
-                mx = max2(mx, v[7]);
-                {
-                    const u32x2 sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-                    mx = max2(__uint_as_float(sw.x), __uint_as_float(sw.y));
-                }
-                site(IntC<2>{});
-                {
-                    const u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-                    mx = max2(__uint_as_float(sw.x), __uint_as_float(sw.y));
-                }
-                site(IntC<3>{});
-                const bool move = (mx - m_ref[qb]) * a.c > kLazy || (m_ref[qb] == -INFINITY && mx > -INFINITY);
-                site(IntC<4>{});
-                alpha[qb] = move ? fast_exp2((m_ref[qb] - mx) * a.c) : 1.0f;
-                if (move) m_ref[qb] = mx;
-                any_move |= move;
-                const float nb = (m_ref[qb] == -INFINITY) ? kPShift : kPShift - m_ref[qb] * a.c;
-                site(IntC<5>{});
+                const float nb = kPShift - m_ref[qb] * a.c;
                 float sum = 0.0f;
                 h8 ph;
                 static_for<0, 8>([&](auto ec) {
                     constexpr int e = decltype(ec)::value;
-                    const float pe = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
+                    float pe = fast_exp2(__builtin_fmaf(s[TP][e / 4][qb][e % 4], a.c, nb));
+                    // An empty volatile block that "rewrites" the value: it keeps its order among
+                    // the matrix instructions, so the exponential stays at this site instead of
+                    // being sunk into the next iteration next to its first use.
+                    asm volatile("" : "+v"(pe));
                     sum += pe;
                     ph[e] = (_Float16)pe;
-                    site(IntC<6 + e>{});
+                    site(IntC<e>{});
                 });
-                l_run[qb] = l_run[qb] * alpha[qb] + sum;
+                asm volatile("" : "+v"(ph));
+                l_run[qb] += sum;
                 pw[TP][qb] = ph;
-                site(IntC<14>{});
-                site(IntC<15>{});
+                site(IntC<8>{});
+                site(IntC<9>{});
             });
-            const bool moved = __builtin_amdgcn_ballot_w64(any_move) != 0;
-            __builtin_amdgcn_s_waitcnt(0xC07F);                         // C(t-1)'s LDS reads have returned
-            fetch_v(IntC<TP ^ 1>{}, tile_of(t + 1));                   // V(t+1) -> the buffer C just read
+            fetch_v(IntC<TP ^ 1>{}, tile_of(t + 1));                   // V(t+1) -> the buffer C(t-1) read (all consumed)
             if (moved) rescale();
         };
         if (R >= 1) {
@@ -948,7 +959,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     for (int qb = 0; qb < NQB; ++qb) {
         const float l_tot = xor_sum(l_run[qb]);
         if (grp == 0) {
-            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = (m_ref[qb] == -INFINITY) ? -INFINITY : m_ref[qb] * a.c;
+            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = m_ref[qb] * a.c; // unset: hugely negative, weight 0
             ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 1] = l_tot;
         }
 #pragma unroll
