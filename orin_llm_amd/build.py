@@ -1,25 +1,38 @@
 """Builds liborin_fa.so (HIP kernels + C ABI + llm::cuda shim) for gfx950, in-tree."""
 import os
 import subprocess
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "liborin_fa.so")
-SOURCES = [os.path.join(HERE, "csrc", "fa_kernels.hip"), os.path.join(HERE, "csrc", "llm_cuda_shim.cpp")]
+OBJ_DIR = os.path.join(HERE, "_obj")
+SOURCES = [os.path.join(HERE, "csrc", n)
+           for n in ("fa_prefill.hip", "fa_decode.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-exceptions",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-exceptions",
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
-def build(verbose=False):
-    cmd = [HIPCC] + FLAGS + SOURCES + ["-o", LIB]
+def _run(cmd):
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + res.stdout + res.stderr)
+    return " ".join(cmd)
+
+
+def build(verbose=False):
+    """Compiles every source (in parallel) and links the shared library.  Always recompiles."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in SOURCES]
+    cmds = [[HIPCC] + FLAGS + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
+        lines = list(pool.map(_run, cmds))
+    lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]))
     if verbose:
-        print(" ".join(cmd))
+        print("\n".join(lines))
     return LIB
 
 

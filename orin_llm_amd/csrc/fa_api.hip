@@ -1,0 +1,169 @@
+// Host side of liborin_fa.so: library state, argument checks, launch-shape choice and the
+// C ABI declared in include/orin_fa.h.  The kernels live in fa_prefill.hip and fa_decode.hip.
+//
+// Boundary: the reference's llm::cuda::flash_attention and flash_attention_decode_ind
+// (reference: src/kernels.h:97-109, launchers at src/kernels.cu:1944-2000).
+#include "fa_common.hpp"
+
+#include <stdio.h>
+
+#include "../../include/orin_fa.h"
+
+namespace orin_fa {
+namespace {
+
+struct State {
+    bool ready = false;
+    int device = 0;
+    int cu_count = 0;
+    hipStream_t stream = nullptr;
+    void* own_ws = nullptr; // allocated by init
+    void* ws = nullptr;     // active workspace
+    size_t ws_bytes = 0;
+};
+State g_state;
+
+inline int hip_code(hipError_t e) { return e == hipSuccess ? ORIN_FA_OK : ORIN_FA_E_HIP - (int)e; }
+
+// The kernels take maxima over raw scores and scale afterwards, which needs a positive
+// multiplier: the sign of `scale` moves into Q and a zero scale becomes a vanishing one.
+inline void set_scale(FaArgs& a, float scale) {
+    const float c = scale * kLog2e;
+    a.qsign = c < 0.0f ? -1.0f : 1.0f;
+    a.c = c < 0.0f ? -c : c;
+    if (!(a.c >= 1e-30f)) a.c = 1e-30f;
+}
+
+int decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
+    const int r = n_head / n_kv;
+    const int n_hgroups = (r + 15) / 16;
+    const int cus = g_state.cu_count > 0 ? g_state.cu_count : 256;
+    int s = cus / (n_kv * n_hgroups); // one 8-wave workgroup per CU
+    const int by_ctx = (n_ctx + kDecodeWaves * kTile - 1) / (kDecodeWaves * kTile);
+    if (s > by_ctx) s = by_ctx;
+    if (s > kMaxSplits) s = kMaxSplits;
+    const size_t per_split = (size_t)n_head * (head_dim + 2) * sizeof(float);
+    const size_t ws = g_state.ws ? g_state.ws_bytes : kWorkspaceBytes;
+    if ((size_t)s * per_split > ws) s = (int)(ws / per_split);
+    return s < 1 ? 1 : s;
+}
+
+int check_common(const void* q, const void* kc, const void* vc, const void* out,
+                 int n_head, int n_kv, int head_dim, int n_ctx) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!q || !kc || !vc || !out) return ORIN_FA_E_INVALID;
+    if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return ORIN_FA_E_INVALID;
+    if (head_dim != 64 && head_dim != 128) return ORIN_FA_E_HEAD_DIM;
+    if ((long long)n_ctx * head_dim * 2 >= (1ll << 31)) return ORIN_FA_E_INVALID; // 32-bit byte offsets per KV head
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kc) | reinterpret_cast<uintptr_t>(vc) |
+         reinterpret_cast<uintptr_t>(out)) & 15u)
+        return ORIN_FA_E_INVALID; // 128-bit loads and stores
+    return ORIN_FA_OK;
+}
+
+} // namespace
+} // namespace orin_fa
+
+using namespace orin_fa;
+
+extern "C" {
+
+int orin_fa_init(int device) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) {
+        fprintf(stderr, "[orin_fa] hipSetDevice(%d) failed: %s\n", device, hipGetErrorString(e));
+        return hip_code(e);
+    }
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_code(e);
+    g_state.device = device;
+    g_state.cu_count = prop.multiProcessorCount;
+    if ((e = prefill_allow_lds()) != hipSuccess) return hip_code(e);
+    if ((e = decode_allow_lds()) != hipSuccess) return hip_code(e);
+    if (!g_state.own_ws) {
+        e = hipMalloc(&g_state.own_ws, kWorkspaceBytes);
+        if (e != hipSuccess) return hip_code(e);
+    }
+    if (!g_state.ws) {
+        g_state.ws = g_state.own_ws;
+        g_state.ws_bytes = kWorkspaceBytes;
+    }
+    g_state.ready = true;
+    return ORIN_FA_OK;
+}
+
+void orin_fa_set_stream(void* stream) { g_state.stream = static_cast<hipStream_t>(stream); }
+
+size_t orin_fa_workspace_bytes(void) { return kWorkspaceBytes; }
+
+int orin_fa_set_workspace(void* dev_ptr, size_t bytes) {
+    if (!dev_ptr) { // back to the library's own block
+        g_state.ws = g_state.own_ws;
+        g_state.ws_bytes = g_state.own_ws ? kWorkspaceBytes : 0;
+        return ORIN_FA_OK;
+    }
+    if ((reinterpret_cast<uintptr_t>(dev_ptr) & 255u) != 0) return ORIN_FA_E_INVALID;
+    if (bytes < kWorkspaceBytes) return ORIN_FA_E_WORKSPACE;
+    g_state.ws = dev_ptr;
+    g_state.ws_bytes = bytes;
+    return ORIN_FA_OK;
+}
+
+int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                    int n_head, int n_kv, int head_dim, int n_ctx, int n_past, int batch, float scale) {
+    int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
+    if (rc != ORIN_FA_OK) return rc;
+    if (batch < 0 || n_past < 0 || (long long)n_past + batch > n_ctx) return ORIN_FA_E_INVALID;
+    if (batch == 0) return ORIN_FA_OK;
+    FaArgs a{};
+    a.q = q; a.kc = kc; a.vc = vc; a.out = out;
+    a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.n_past = n_past; a.batch = batch;
+    a.r = n_head / n_kv;
+    a.n_splits = 1;
+    set_scale(a, scale);
+    return hip_code(prefill_launch(a, head_dim, g_state.stream));
+}
+
+int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                       int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
+    int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
+    if (rc != ORIN_FA_OK) return rc;
+    if (!d_pos) return ORIN_FA_E_INVALID;
+    FaArgs a{};
+    a.q = q; a.kc = kc; a.vc = vc; a.out = out; a.d_pos = d_pos;
+    a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.batch = 1;
+    a.r = n_head / n_kv;
+    a.n_hgroups = (a.r + 15) / 16;
+    a.n_splits = decode_splits(n_head, n_kv, head_dim, n_ctx);
+    if (a.n_splits > 1) {
+        if (!g_state.ws) return ORIN_FA_E_WORKSPACE;
+        a.part_o = static_cast<float*>(g_state.ws);
+        a.part_ml = a.part_o + (size_t)a.n_splits * n_head * head_dim;
+    }
+    set_scale(a, scale);
+    return hip_code(decode_launch(a, head_dim, g_state.stream));
+}
+
+int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
+    if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return 0;
+    if (head_dim != 64 && head_dim != 128) return 0;
+    return decode_splits(n_head, n_kv, head_dim, n_ctx);
+}
+
+int orin_fa_cu_count(void) { return g_state.cu_count; }
+
+const char* orin_fa_error_string(int code) {
+    switch (code) {
+        case ORIN_FA_OK: return "ok";
+        case ORIN_FA_E_INVALID: return "invalid argument (shape, alignment or null pointer)";
+        case ORIN_FA_E_HEAD_DIM: return "unsupported head_dim (64 and 128 only)";
+        case ORIN_FA_E_WORKSPACE: return "split-KV workspace missing or too small";
+        case ORIN_FA_E_NOT_INIT: return "orin_fa_init has not been called";
+        default: break;
+    }
+    if (code <= ORIN_FA_E_HIP) return hipGetErrorString(static_cast<hipError_t>(ORIN_FA_E_HIP - code));
+    return "unknown error";
+}
+
+} // extern "C"

@@ -1,0 +1,118 @@
+// Shared pieces of the gfx950 flash-attention kernels: vector types, launch arguments,
+// wave-level helpers.  Included by fa_prefill.hip, fa_decode.hip and fa_api.hip only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace orin_fa {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef __fp16 fp16x4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kPrefillWaves = 4; // waves per prefill workgroup (one per SIMD: the kernel fills the register file)
+constexpr int kDecodeWaves = 8;  // waves per decode workgroup (two per SIMD, one workgroup per CU)
+constexpr int kTile = 32;        // KV rows per wave tile
+constexpr float kLog2e = 1.4426950408889634f;
+// Softmax weights are computed against a reference maximum that is only moved when a score
+// exceeds it by more than kLazy (log2 units), so the O accumulators are rescaled on a handful
+// of early tiles instead of every tile.  P = 2^(s - m_ref + kPShift) therefore lies in
+// (0, 2^(kLazy + kPShift)] = (0, 2^15], inside fp16 range and far enough above its subnormals
+// that small weights keep their 11 bits; the common factor cancels in O / l.
+constexpr float kLazy = 8.0f;
+constexpr float kPShift = 7.0f;
+constexpr int kMaxSplits = 256;                 // decode KV splits per KV head, at most
+constexpr size_t kWorkspaceBytes = 8u << 20;    // split-KV partial results
+
+struct FaArgs {
+    const float* q;
+    const uint16_t* kc;
+    const uint16_t* vc;
+    float* out;
+    float* part_o;    // decode: [split][n_head][D]
+    float* part_ml;   // decode: [split][n_head][2] = (reference maximum in log2 units, row sum)
+    const int* d_pos; // decode only
+    int n_head, n_kv, n_ctx;
+    int n_past, batch; // prefill only
+    int r;             // query heads per KV head
+    int n_hgroups;     // head groups per KV head
+    int n_ttiles;      // prefill: token tiles
+    int n_splits;      // decode: KV splits
+    float c;           // |scale| * log2(e), clamped away from zero
+    float qsign;       // sign of scale, folded into Q
+};
+
+// Launchers (defined next to their kernels).  All return hipError_t of the launch.
+hipError_t prefill_launch(const FaArgs& args, int head_dim, hipStream_t stream);
+hipError_t prefill_allow_lds();
+hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream);
+hipError_t decode_allow_lds();
+
+template <int N>
+struct IntC {
+    static constexpr int value = N;
+};
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(IntC<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// All-reduce over the four 16-lane groups of a wave (lanes l, l^16, l^32, l^48) with the
+// gfx950 lane-swap instructions: v_permlane32_swap exchanges the upper half of one register
+// with the lower half of the other, v_permlane16_swap does the same for odd/even 16-lane rows.
+__device__ __forceinline__ float xor_max(float v) {
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+}
+__device__ __forceinline__ float xor_sum(float v) {
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(s.x) + __uint_as_float(s.y);
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(s.x) + __uint_as_float(s.y);
+}
+
+// 16-byte load through a buffer descriptor: the hardware returns zeros for offsets at or
+// past the descriptor's byte count, so cache rows beyond the visible range (which may hold
+// anything, NaN patterns included) are never fetched and need no branch.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+// (The whole offset travels in the vector operand: the scalar offset operand is not range-checked.)
+// STREAM marks data that is read once (decode): the load carries the non-temporal hint so the
+// stream does not displace useful lines in L2 / Infinity Cache (measured 5-7% faster).
+template <bool STREAM>
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, STREAM ? 2 : 0);
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element (i % 4) of the
+// 8 bytes addressed by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 -- a 4x16 transpose on the way
+// out of LDS.  With lane i pointing at row (i / 4), 8-byte column (i % 4) of a row-major
+// fp16 tile, lane i ends up with rows 0..3 at column i: an MFMA operand whose k index runs
+// down the tile's rows.
+__device__ __forceinline__ h4 lds_read_tr(const unsigned char* p) {
+    const fp16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4f16((__attribute__((address_space(3))) fp16x4*)(p));
+    return __builtin_bit_cast(h4, t);
+}
+
+// Orders this wave's LDS writes before its later LDS reads (lanes of one wave exchange
+// data through the wave-private LDS slice).
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+} // namespace orin_fa

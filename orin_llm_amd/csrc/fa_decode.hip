@@ -1,0 +1,351 @@
+// Single-token GQA attention over the fp16 KV cache for gfx950 (MI355X): a split-KV kernel
+// spread over every CU plus a log-sum-exp combine kernel.
+//
+// Replaces the reference's flash_attention_decode_mma_k and its launcher (reference:
+// src/kernels.cu:1105-1345, 1983-2000), which runs one block per KV head.
+//
+//   * The visible cache rows [0, *d_pos] of one KV head are cut into 32-row tiles.  Workgroup
+//     (KV head, split s) is 8 wave64s; wave w takes tile s*8 + w and then every
+//     (8 * n_splits)-th tile after it, so at 32k context each wave streams one or two tiles and
+//     every byte of K and V is fetched exactly once, by 128-bit loads with the non-temporal hint.
+//   * K rows go straight from memory into MFMA A-operand order (lane (col, grp) takes row col,
+//     bytes (kk*4 + grp)*16): the score product needs no LDS round trip.  V rows are loaded
+//     coalesced, parked in the wave's LDS slice and read back transposed (ds_read_b64_tr_b16).
+//   * All query heads of the KV head's group (up to 16 per workgroup) are the 16 columns of
+//     S^T = K Q^T and O^T = V^T P on v_mfma_f32_16x16x32_f16, so the group shares one pass
+//     over K and V.  The matrix pipe is idle most of the time here, so Q and P are carried as
+//     fp16 hi + lo pairs and the result is accurate to fp32 rounding.
+//   * The position is read on the device; the launch shape depends only on by-value arguments,
+//     so the launch can be captured in a graph and replayed after the position changes.
+//   * Partials (reference maximum, row sum, O) of the 8 waves are merged through LDS and
+//     written per split; the combine kernel merges the splits that were active.
+#include "fa_common.hpp"
+
+namespace orin_fa {
+namespace {
+
+template <int D>
+struct DGeom {
+    static constexpr int kSteps = D / 32;                      // MFMA k-steps over head_dim
+    static constexpr int kDBlk = D / 16;                       // 16-wide output blocks over head_dim
+    static constexpr int kRowBV = D * 2 + 32;                  // bytes per V row in LDS (32 B pad spreads the transposing reads)
+    static constexpr int kChunksPerRow = D / 8;                // 16-byte chunks per KV row
+    static constexpr int kLoads = kTile * kChunksPerRow / 64;  // 16-byte V loads per lane per tile
+    static constexpr int kTileBV = kTile * kRowBV;             // one V tile in LDS
+    static constexpr int kOStride = D + 4;                     // floats per column in the merge buffer
+    static constexpr int kMergeB = 16 * kOStride * 4;
+    static constexpr int kWaveB = (kTileBV > kMergeB) ? kTileBV : kMergeB;
+    static constexpr int kMlOff = kDecodeWaves * kWaveB;       // (m, l) per wave per column follow the wave slices
+    static constexpr int kLdsB = kMlOff + kDecodeWaves * 16 * 2 * 4;
+};
+
+template <int D>
+__global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(const FaArgs a) {
+    using G = DGeom<D>;
+    constexpr int kWaves = kDecodeWaves;
+    constexpr int kThreads = kWaves * 64;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int col = lane & 15; // MFMA column (query head of the group) / row (KV row or head_dim index) of the lane
+    const int grp = lane >> 4; // lane-group: 8-wide k slice of an operand, 4-row slice of an accumulator
+
+    // Workgroup id -> (KV head, head group, split).  The KV head varies fastest.
+    int id = blockIdx.x;
+    const int kvh = id % a.n_kv;
+    id /= a.n_kv;
+    const int hg = id % a.n_hgroups;
+    id /= a.n_hgroups; // = split
+
+    int p = *a.d_pos;
+    p = p < 0 ? 0 : p;
+    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
+    const int n_tiles = (npos + kTile - 1) / kTile;
+    const int tile_first = id * kWaves + wave;
+    const int tile_step = kWaves * a.n_splits;
+    if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
+
+    unsigned char* const vs = smem + wave * G::kWaveB;
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)npos * D * 2);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)npos * D * 2);
+
+    u32x4 kreg[2 * G::kSteps], vreg[G::kLoads];
+    auto fetch_k = [&](int tile) {
+        const int soff = tile * kTile * D * 2;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kk = 0; kk < G::kSteps; ++kk)
+                kreg[t * G::kSteps + kk] = buf_load16<true>(krs, soff + (t * 16 + col) * D * 2 + (kk * 4 + grp) * 16);
+    };
+    auto fetch_v = [&](int tile) {
+        const int soff = tile * kTile * D * 2;
+#pragma unroll
+        for (int i = 0; i < G::kLoads; ++i) vreg[i] = buf_load16<true>(vrs, soff + (i * 64 + lane) * 16);
+    };
+    int tile = tile_first;
+    if (tile < n_tiles) { // in flight while the query heads are loaded and converted
+        fetch_k(tile);
+        fetch_v(tile);
+    }
+
+    // ---- query heads -> B operands, fp16 hi + lo ----
+    const int hl = hg * 16 + col;
+    const bool valid = hl < a.r;
+    const float* qp = a.q + (size_t)(valid ? kvh * a.r + hl : 0) * D;
+    const float qmul = valid ? a.qsign : 0.0f;
+    h8 qhi[G::kSteps], qlo[G::kSteps];
+#pragma unroll
+    for (int kk = 0; kk < G::kSteps; ++kk) {
+        const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
+        const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+        const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float xe = x[e] * qmul;
+            qhi[kk][e] = (_Float16)xe;
+            qlo[kk][e] = (_Float16)(xe - (float)qhi[kk][e]);
+        }
+    }
+
+    // m_ref: reference maximum of the raw scores (before the scale); l_run: this lane's share of
+    // the row sum; o: O^T accumulators, lane (col, grp) holds head_dim rows db*16 + grp*4 + i.
+    float m_ref = -INFINITY, l_run = 0.0f;
+    f4 o[G::kDBlk];
+#pragma unroll
+    for (int db = 0; db < G::kDBlk; ++db) o[db] = f4{0.f, 0.f, 0.f, 0.f};
+    const int v_rd = (grp * 4 + (col >> 2)) * G::kRowBV + (col & 3) * 8; // + h*16 rows, + db*32 bytes
+
+    for (; tile < n_tiles; tile += tile_step) {
+        const bool more = tile + tile_step < n_tiles;
+#pragma unroll
+        for (int i = 0; i < G::kLoads; ++i) {
+            const int c = i * 64 + lane;
+            *reinterpret_cast<u32x4*>(vs + (c / G::kChunksPerRow) * G::kRowBV + (c % G::kChunksPerRow) * 16) = vreg[i];
+        }
+        if (more) fetch_v(tile + tile_step);
+        wave_lds_sync();
+
+        // ---- S^T = K Q^T : rows = KV row (sub-tile t, row col), columns = query head ----
+        f4 s[2], s2[2]; // the Q-lo product runs as its own accumulation chain
+#pragma unroll
+        for (int t = 0; t < 2; ++t) s[t] = s2[t] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps; ++kk)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const h8 ka = __builtin_bit_cast(h8, kreg[t * G::kSteps + kk]);
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qhi[kk], s[t], 0, 0, 0);
+                s2[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qlo[kk], s2[t], 0, 0, 0);
+            }
+        s[0] += s2[0];
+        s[1] += s2[1];
+        if (more) fetch_k(tile + tile_step); // the operand registers are free again
+
+        // ---- softmax weights; lane (col, grp) holds rows t*16 + grp*4 + i of its column ----
+        float v[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[t * 4 + i] = s[t][i];
+        if (tile * kTile + kTile > npos) { // the last tile: rows past the position do not exist
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (tile * kTile + t * 16 + grp * 4 + i >= npos) v[t * 4 + i] = -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(v[0], v[1]), v[2]);
+        mx = fmaxf(fmaxf(mx, v[3]), v[4]);
+        mx = fmaxf(fmaxf(mx, v[5]), v[6]);
+        mx = xor_max(fmaxf(mx, v[7]));
+        // move the reference only when this tile's maximum is far above it (or it is unset)
+        const bool move = (mx - m_ref) * a.c > kLazy || (m_ref == -INFINITY && mx > -INFINITY);
+        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+            const float alpha = move ? fast_exp2((m_ref - mx) * a.c) : 1.0f; // unset reference -> 0
+            if (move) m_ref = mx;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db) o[db] *= alpha;
+        }
+        // exponent = s*c - m_ref*c + shift; a column that has seen no visible row keeps weight 0
+        const float nb = (m_ref == -INFINITY) ? kPShift : kPShift - m_ref * a.c;
+        h8 ph, pl;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float pe = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
+            l_run += pe;
+            ph[e] = (_Float16)pe;
+            pl[e] = (_Float16)(pe - (float)ph[e]);
+        }
+
+        // ---- O^T += V^T P : rows = head_dim index, columns = query head, k = the tile's 32 KV rows
+        //      in the order (grp, t, i) that matches the layout P already has ----
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db) {
+            const h4 v0 = lds_read_tr(vs + v_rd + db * 32);
+            const h4 v1 = lds_read_tr(vs + v_rd + 16 * G::kRowBV + db * 32);
+            const h8 va = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, ph, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pl, o[db], 0, 0, 0);
+        }
+        wave_lds_sync(); // the slice is overwritten at the top of the next iteration
+    }
+
+    // ---- merge the waves through LDS ----
+    float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
+    float* const obuf = reinterpret_cast<float*>(smem + wave * G::kWaveB);
+    const float l_tot = xor_sum(l_run);
+    if (grp == 0) {
+        ml[(wave * 16 + col) * 2 + 0] = (m_ref == -INFINITY) ? -INFINITY : m_ref * a.c; // log2 units
+        ml[(wave * 16 + col) * 2 + 1] = l_tot;
+    }
+#pragma unroll
+    for (int db = 0; db < G::kDBlk; ++db)
+        *reinterpret_cast<f4*>(obuf + col * G::kOStride + db * 16 + grp * 4) = o[db];
+    __syncthreads();
+
+    for (int idx = threadIdx.x; idx < 16 * (D / 4); idx += kThreads) {
+        const int c = idx / (D / 4);
+        const int d4 = (idx % (D / 4)) * 4;
+        const int h_local = hg * 16 + c;
+        if (h_local >= a.r) continue;
+        float mw[kWaves], lw[kWaves];
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mw[w] = ml[(w * 16 + c) * 2 + 0];
+            lw[w] = ml[(w * 16 + c) * 2 + 1];
+            m_all = fmaxf(m_all, mw[w]);
+        }
+        float l_all = 0.0f;
+        f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float wgt = fast_exp2(mw[w] - m_all); // a wave that had no tile has m = -inf -> weight 0
+            l_all += lw[w] * wgt;
+            acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4) * wgt;
+        }
+        const int head = kvh * a.r + h_local;
+        if (a.n_splits > 1) {
+            const size_t pi = (size_t)id * a.n_head + head;
+            *reinterpret_cast<f4*>(a.part_o + pi * D + d4) = acc;
+            if (d4 == 0) {
+                a.part_ml[pi * 2 + 0] = m_all;
+                a.part_ml[pi * 2 + 1] = l_all;
+            }
+        } else {
+            const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+            *reinterpret_cast<f4*>(a.out + (size_t)head * D + d4) = acc * inv;
+        }
+    }
+}
+
+// Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
+// head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the
+// position, the (m, l) pairs and this thread's share of the partial outputs -- is issued
+// before anything is waited on, so the kernel is one memory round trip deep.  Slots of
+// splits that were inactive for this position hold stale data and are masked after the load.
+template <int D>
+__global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) {
+    constexpr int kSlices = D / 32;
+    constexpr int kGroups = 8;
+    constexpr int kPer = kMaxSplits / kGroups; // partial-output loads per thread, at most
+    __shared__ float sh_w[kMaxSplits];
+    __shared__ float sh_red[kGroups][32];
+    __shared__ float sh_wave[4][2];
+    const int head = blockIdx.x / kSlices;
+    const int d = (blockIdx.x % kSlices) * 32 + (threadIdx.x & 31);
+    const int sg = threadIdx.x >> 5;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_splits = a.n_splits;
+
+    // loads first
+    const int s_mine = threadIdx.x; // kMaxSplits == 256 == blockDim.x
+    float m_s = -INFINITY, l_s = 0.0f;
+    if (s_mine < n_splits) {
+        const float2 ml = *reinterpret_cast<const float2*>(a.part_ml + ((size_t)s_mine * a.n_head + head) * 2);
+        m_s = ml.x;
+        l_s = ml.y;
+    }
+    float x[kPer];
+    const float* po = a.part_o + (size_t)head * D + d;
+    const size_t stride = (size_t)a.n_head * D;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int s = sg + j * kGroups;
+        x[j] = s < n_splits ? po[s * stride] : 0.0f;
+    }
+    int p = *a.d_pos;
+    p = p < 0 ? 0 : p;
+    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1;
+    const int n_tiles = (npos + kTile - 1) / kTile;
+    const int by_tiles = (n_tiles + kDecodeWaves - 1) / kDecodeWaves;
+    const int n_active = by_tiles < n_splits ? by_tiles : n_splits;
+
+    // weights w_s = 2^(m_s - max m) and the total row sum
+    if (s_mine >= n_active) {
+        m_s = -INFINITY;
+        l_s = 0.0f;
+    }
+    float m_all = m_s;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, off));
+    if (lane == 0) sh_wave[wave][0] = m_all;
+    __syncthreads();
+    m_all = fmaxf(fmaxf(sh_wave[0][0], sh_wave[1][0]), fmaxf(sh_wave[2][0], sh_wave[3][0]));
+    const float w = fast_exp2(m_s - m_all); // every active split has seen a visible row, so m_all is finite
+    sh_w[s_mine] = w;                       // 0 for inactive slots
+    float l_all = w * l_s;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) l_all += __shfl_xor(l_all, off);
+    if (lane == 0) sh_wave[wave][1] = l_all;
+    __syncthreads();
+    l_all = (sh_wave[0][1] + sh_wave[1][1]) + (sh_wave[2][1] + sh_wave[3][1]);
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int s = sg + j * kGroups;
+        if (s < n_active) acc = __builtin_fmaf(x[j], sh_w[s], acc);
+    }
+    sh_red[sg][threadIdx.x & 31] = acc;
+    __syncthreads();
+    if (sg == 0) {
+        float tot = 0.0f;
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) tot += sh_red[g][threadIdx.x];
+        a.out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
+    }
+}
+
+template <int D>
+hipError_t launch(const FaArgs& a, hipStream_t stream) {
+    const int grid = a.n_kv * a.n_hgroups * a.n_splits;
+    constexpr int lds = DGeom<D>::kLdsB;
+    hipLaunchKernelGGL(fa_decode_split_kernel<D>, dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || a.n_splits == 1) return e;
+    hipLaunchKernelGGL(fa_decode_combine_kernel<D>, dim3(a.n_head * (D / 32)), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+} // namespace
+
+hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream) {
+    return head_dim == 128 ? launch<128>(a, stream) : launch<64>(a, stream);
+}
+
+// The split kernel uses more than 64 KB of dynamic LDS; the opt-in is set once at init so
+// that no launch path touches function attributes (decode runs under stream capture).
+hipError_t decode_allow_lds() {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_decode_split_kernel<128>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, DGeom<128>::kLdsB);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_decode_split_kernel<64>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, DGeom<64>::kLdsB);
+}
+
+} // namespace orin_fa
