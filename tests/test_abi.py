@@ -1,0 +1,95 @@
+"""The C-ABI library loads and exports what the headers declare (no compute calls: runs without a GPU)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "orin_llm_amd", "liborin_fa.so")
+HDR = os.path.join(ROOT, "include", "orin_fa.h")
+SHIM_HDR = os.path.join(ROOT, "include", "orin_llm_amd", "kernels.h")
+REF_HDR = "/root/reference/src/kernels.h"
+
+
+def _strip_comments(text):
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    return re.sub(r"//[^\n]*", " ", text)
+
+
+def _declared_c_functions():
+    body = _strip_comments(open(HDR).read())
+    return sorted(set(re.findall(r"\b(orin_fa_[a-z_]+)\s*\(", body)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        pytest.fail("liborin_fa.so is not built: run `python orin_llm_amd/build.py`")
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_expected_entry_points():
+    assert _declared_c_functions() == sorted([
+        "orin_fa_init", "orin_fa_set_stream", "orin_fa_workspace_bytes", "orin_fa_set_workspace",
+        "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_splits", "orin_fa_cu_count",
+        "orin_fa_error_string"])
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in _declared_c_functions():
+        assert hasattr(lib, name), f"{name} declared in include/orin_fa.h but not exported"
+
+
+def test_calls_that_need_no_device(lib):
+    lib.orin_fa_workspace_bytes.restype = ctypes.c_size_t
+    assert lib.orin_fa_workspace_bytes() >= 256 * 32 * (128 + 2) * 4  # 256 splits of a 32-head model
+    lib.orin_fa_error_string.restype = ctypes.c_char_p
+    lib.orin_fa_error_string.argtypes = [ctypes.c_int]
+    assert lib.orin_fa_error_string(0) == b"ok"
+    assert b"head_dim" in lib.orin_fa_error_string(-2)
+    assert b"init" in lib.orin_fa_error_string(-4)
+    # shape screening happens before any device work
+    assert lib.orin_fa_decode_splits(12, 5, 128, 4096) == 0   # n_head % n_kv != 0
+    assert lib.orin_fa_decode_splits(12, 2, 96, 4096) == 0    # head_dim
+    assert lib.orin_fa_decode_splits(12, 2, 128, 32768) >= 1
+
+
+def test_launch_before_init_is_refused(lib):
+    """Every launch entry point checks the library state before it touches its arguments."""
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    if lib.orin_fa_cu_count() != 0:
+        pytest.skip("the library was initialised earlier in this process")
+    lib.orin_fa_prefill.argtypes = [vp] * 4 + [ci] * 6 + [ctypes.c_float]
+    lib.orin_fa_decode_ind.argtypes = [vp] * 4 + [ci] * 4 + [vp, ctypes.c_float]
+    assert lib.orin_fa_prefill(16, 16, 16, 16, 12, 2, 128, 4096, 0, 8, 0.1) == -4
+    assert lib.orin_fa_decode_ind(16, 16, 16, 16, 12, 2, 128, 4096, 16, 0.1) == -4
+
+
+def test_shim_symbols_have_the_reference_manglings():
+    """The C++ shim exports llm::cuda::flash_attention / flash_attention_decode_ind / init / set_stream
+    under exactly the names an engine compiled against the reference header links to."""
+    out = subprocess.run(["nm", "-D", "--defined-only", LIB], capture_output=True, text=True, check=True).stdout
+    syms = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    expected = [
+        "_ZN3llm4cuda15flash_attentionEPKfPKtS4_Pfiiiiiif",
+        "_ZN3llm4cuda26flash_attention_decode_indEPKfPKtS4_PfiiiiPKif",
+        "_ZN3llm4cuda4initEv",
+        "_ZN3llm4cuda10set_streamEPv",
+    ]
+    for s in expected:
+        assert s in syms, s
+
+
+def _decl(text, name):
+    m = re.search(r"void\s+" + name + r"\s*\([^)]*\)\s*;", _strip_comments(text))
+    assert m, name
+    return re.sub(r"\s+", " ", m.group(0)).replace("( ", "(").strip()
+
+
+@pytest.mark.skipif(not os.path.exists(REF_HDR), reason="reference tree not present on this machine")
+def test_shim_header_matches_reference_declarations():
+    ref, ours = open(REF_HDR).read(), open(SHIM_HDR).read()
+    for name in ("flash_attention", "flash_attention_decode_ind"):
+        assert _decl(ours, name) == _decl(ref, name)
