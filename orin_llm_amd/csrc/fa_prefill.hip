@@ -24,6 +24,11 @@
 namespace orin_fa {
 namespace {
 
+// Cycle-counter stamps for profiling builds (defined by a prefix header there); nothing otherwise.
+#ifndef FA_STAMP
+#define FA_STAMP(i)
+#endif
+
 constexpr float kUnsetRef = -1.0e30f; // reference maximum of a column that has seen no visible key yet
 
 __device__ __forceinline__ float max2(float x, float y);
@@ -137,6 +142,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     constexpr int kThreads = kWaves * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
+    FA_STAMP(0);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = lane & 15;
@@ -226,6 +232,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         for (int db = 0; db < G::kDBlk; ++db) lds_load_acc(o[qb][db], scratch_addr);
     }
 
+    FA_STAMP(1);
     auto stage_a = [&](auto kpar, auto spar) { // S[spar] = K[kpar] Q^T (prologue form: not interleaved)
         constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
         const unsigned char* const kb = ws + G::kKOff + KP * G::kTileB;
@@ -355,6 +362,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             }
         }
 
+        FA_STAMP(2);
         // Copy issue order: K0 V0 K1 V1 | K2 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
         // ---- step 0: the diagonal tile, the only one that can need the causal mask ----
         const int R = n_mine - 1; // steps after step 0
@@ -371,6 +379,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         else stage_b(IntC<0>{}, IntC<0>{}, tile_of(0));
         // (O is still zero: no rescale)
 
+        FA_STAMP(3);
         // ---- steps t >= 1: A(t+1), B(t) and C(t-1) share one hand-ordered instruction stream.
         // The 2 * kGroups/2 * NQB matrix instructions of A and C are cut into groups of NQB that
         // share an LDS operand (A: one (k-step, sub-tile) of K; C: one 16-wide block of V^T),
@@ -501,6 +510,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         } else if (t == R) {
             body(IntC<0>{}, IntC<0>{}, IntC<2 * kC>{}, t);
         }
+        FA_STAMP(4);
         // ---- drain: C(R) ----
         wait_copies(IntC<0>{});
         settle(); // P(R) was converted just above
@@ -511,6 +521,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         wave_lds_sync();
     }
 
+    FA_STAMP(5);
     // ---- merge the four waves through LDS ----
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
     const unsigned obuf_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(smem + wave * G::kWaveB);
@@ -525,7 +536,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         for (int db = 0; db < G::kDBlk; ++db)
             lds_store_acc(obuf_addr + ((qb * 16 + col) * G::kOStride + db * 16 + grp * 4) * 4, o[qb][db]);
     }
+    FA_STAMP(6);
     __syncthreads();
+    FA_STAMP(7);
 
     constexpr int kCols = NQB * 16;
     for (int idx = threadIdx.x; idx < kCols * (D / 4); idx += kThreads) {
@@ -554,6 +567,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
         *reinterpret_cast<f4*>(a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D + d4) = acc * inv;
     }
+    FA_STAMP(8);
 }
 
 template <int D, int NQB, int TQ>
