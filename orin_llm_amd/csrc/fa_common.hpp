@@ -48,7 +48,7 @@ struct FaArgs {
 };
 
 // Launchers (defined next to their kernels).  All return hipError_t of the launch.
-hipError_t prefill_launch(const FaArgs& args, int head_dim, hipStream_t stream);
+hipError_t prefill_launch(const FaArgs& args, int head_dim, int cu_count, hipStream_t stream);
 hipError_t prefill_allow_lds();
 hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream);
 hipError_t decode_allow_lds();

@@ -9,35 +9,34 @@
 // barrier.  S^T = K Q^T and O^T = V^T P run on v_mfma_f32_16x16x32_f16: the accumulator layout
 // of the first product (lane = query column, 4 KV rows per lane-group) is the B-operand layout
 // of the second once the 32 KV rows of a tile are numbered (lane-group, sub-tile, row), so P
-// needs no shuffle and every rescale factor is a per-lane scalar.
+// needs no shuffle and every per-column quantity is a per-lane scalar.
 //
 // The three stages of a tile
-//     A: S = K Q^T (MFMA)      B: P = 2^(S*c - m) (VALU)      C: O += V^T P (MFMA)
+//     A: S = K Q^T (MFMA)      B: P = 2^(S*c + b) (VALU)      C: O += V^T P, l += 1^T P (MFMA)
 // run skewed -- iteration t issues A(t+1), B(t) and C(t-1), which are independent of one
-// another, so the matrix pipe works while the vector pipe exponentiates.  K and V tiles are
-// copied global->LDS by the load unit itself (no staging registers, two buffers each per wave)
-// in an XOR-swizzled layout that both the 1 KB copy bursts and the operand reads hit
-// conflict-free.  Each wave walks its tiles from the diagonal backwards, so the only tile
+// another -- in one hand-ordered instruction stream, so the matrix pipe works while the vector
+// pipe exponentiates.  What keeps the vector share small:
+//   * B is one fused multiply-add (scale*log2(e) and the column's offset b = shift - reference
+//     maximum; Q itself stays unscaled, so fp16-representable inputs enter the products exactly),
+//     one v_exp_f32 per score and one v_cvt_pk_f16_f32 per pair.
+//   * Row sums are one more matrix instruction per query block (a ones operand times P).
+//   * The reference maximum is lazy: exponentials are computed optimistically while the largest
+//     exponent of the tile is tracked; only if it exceeds the fp16-safe bound (on a handful of
+//     early tiles) does a slow path move the reference, redo the tile's P and rescale O and l.
+// K and V tiles are copied global->LDS by the load unit itself (no staging registers, two
+// buffers each per wave, tile base in the scalar offset so the copies need no vector
+// arithmetic) in an XOR-swizzled layout that both the 1 KB copy bursts and the operand reads
+// hit conflict-free.  Each wave walks its tiles from the diagonal backwards, so the only tile
 // that can need the causal mask is handled in the prologue and the steady state is mask-free.
 #include "fa_common.hpp"
-
-namespace orin_fa {
-namespace {
 
 // Cycle-counter stamps for profiling builds (defined by a prefix header there); nothing otherwise.
 #ifndef FA_STAMP
 #define FA_STAMP(i)
 #endif
 
-constexpr float kUnsetRef = -1.0e30f; // reference maximum of a column that has seen no visible key yet
-
-__device__ __forceinline__ float max2(float x, float y);
-__device__ __forceinline__ float xor_max_fast(float v) { // all-reduce over lanes l, l^16, l^32, l^48; inputs never NaN
-    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    float r = max2(__uint_as_float(s.x), __uint_as_float(s.y));
-    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(r), __float_as_uint(r), false, false);
-    return max2(__uint_as_float(s.x), __uint_as_float(s.y));
-}
+namespace orin_fa {
+namespace {
 
 template <int D, int NQB>
 struct PGeom {
@@ -52,31 +51,47 @@ struct PGeom {
     static constexpr int kVOff = 2 * kTileB;
     static constexpr int kOStride = D + 4;
     static constexpr int kMergeB = NQB * 16 * kOStride * 4;
-    static constexpr int kScratchOff = 4 * kTileB;    // 1 KB per wave: 16 bytes per lane for the rare O rescale
+    static constexpr int kScratchOff = 4 * kTileB;    // 1 KB per wave: 16 bytes per lane for accumulator round trips
     static constexpr int kWaveB = (4 * kTileB + 1024 > kMergeB) ? 4 * kTileB + 1024 : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
     static constexpr int kLdsB = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4;
 };
 
-
-// Matrix instructions with the register file of each operand spelled out.  The prefill kernel
-// keeps its score accumulators in ordinary vector registers (the exponentials read them with no
-// copy) and its output accumulators in the accumulation-register file, and it fixes the issue
-// order of matrix and vector work by hand -- neither of which the builtin form allows.  The
-// price: the compiler knows nothing about the hazards of these.  (1) Result latency: every place
-// where a non-matrix instruction reads an accumulator is either a pipeline stage away or behind
-// settle().  (2) A matrix instruction must not read an operand in the two cycles after a vector
-// instruction wrote it, and the compiler is free to sink such a write (the fp16 conversion of P,
-// a register copy) right in front of the asm block: each block starts with the two wait states.
-__device__ __forceinline__ void mfma_v(f4& acc, h8 a_op, h8 b_op) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "v"(b_op));
+// ---------------------------------------------------------------------------------------------
+// Instructions with the register file of each operand spelled out.  The kernel keeps its score
+// accumulators in ordinary vector registers (the exponentials read them with no copy) and its
+// output accumulators and the query operands in the accumulation-register file, and it fixes the issue order of matrix
+// and vector work by hand -- neither of which the builtin forms allow.  The price: the compiler
+// knows nothing about the hazards of these blocks.
+//   (1) Result latency: a non-matrix instruction reads a matrix result only a pipeline stage
+//       (at least two later matrix instructions) after it was issued, or behind settle().
+//   (2) A matrix instruction must not read an operand in the two cycles after a vector
+//       instruction wrote it.  The forms with the _n suffix start with the two wait states and
+//       are used wherever compiler-generated vector code may sit right in front of the block
+//       (prologue, drain); the main loop uses the bare forms, where every operand was written
+//       a long way back (LDS reads, the previous iteration's conversions, loop invariants).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void mfma_v_n(f4& acc, h8 a_op, h8 b_acc) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
 }
-__device__ __forceinline__ void mfma_v_zero(f4& acc, h8 a_op, h8 b_op) { // acc = A B
+__device__ __forceinline__ void mfma_v_zero_n(f4& acc, h8 a_op, h8 b_acc) { // acc = A B
     // early clobber: the destination must not share registers with an operand that dies here
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "v"(b_op));
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
+}
+__device__ __forceinline__ void mfma_a_n(f4& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
+}
+__device__ __forceinline__ void mfma_a_zero_n(f4& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&a"(acc) : "v"(a_op), "v"(b_op));
+}
+__device__ __forceinline__ void mfma_v(f4& acc, h8 a_op, h8 b_acc) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
+}
+__device__ __forceinline__ void mfma_v_zero(f4& acc, h8 a_op, h8 b_acc) { // acc = A B
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
 }
 __device__ __forceinline__ void mfma_a(f4& acc, h8 a_op, h8 b_op) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
 }
 // Lets the matrix pipe drain (32 wait states, more than any 16x16x32 result needs) and stops the
 // compiler from moving anything across.
@@ -86,52 +101,84 @@ __device__ __forceinline__ void settle() {
     __builtin_amdgcn_sched_barrier(0);
 }
 // 16 bytes between LDS and the accumulation-register file, without a detour through vector
-// registers.  The output accumulators of the prefill kernel are only ever touched by these and
-// by mfma_a, which keeps them in that file for the whole kernel.
+// registers.  The output accumulators are only ever touched by these and by the matrix
+// instructions, which keeps them in that file for the whole kernel.
 __device__ __forceinline__ void lds_store_acc(unsigned lds_addr, const f4& acc) {
     asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(lds_addr), "a"(acc) : "memory");
 }
-__device__ __forceinline__ void lds_load_acc(f4& acc, unsigned lds_addr) {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=a"(acc) : "v"(lds_addr) : "memory");
+template <int OFF>
+__device__ __forceinline__ void lds_store_acc_nowait(unsigned lds_addr, const f4& acc) { // caller waits
+    asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(lds_addr), "a"(acc), "n"(OFF) : "memory");
 }
+// (The accumulator is declared read-write although its old value is dead: a tied operand keeps it in
+// the same registers, where a fresh definition on a rarely taken path costs a copy of the whole set.)
+__device__ __forceinline__ void lds_load_acc(f4& acc, unsigned lds_addr) {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "+a"(acc) : "v"(lds_addr) : "memory");
+}
+// The vector side of the main loop, as volatile blocks so that it stays where it is written,
+// interleaved with the matrix instructions.
+__device__ __forceinline__ void v_fma(float& r, float x, float y, float z) { asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z)); }
+__device__ __forceinline__ void v_exp2(float& r) { asm volatile("v_exp_f32 %0, %0" : "+v"(r)); }
+__device__ __forceinline__ void v_cvt_pk(unsigned& r, float lo, float hi) { // two fp32 -> packed fp16, round to nearest even
+    asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+}
+__device__ __forceinline__ void v_max2(float& r, float x, float y) { asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y)); }
+__device__ __forceinline__ void v_max3_acc(float& r, float x, float y) { asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(r) : "v"(x), "v"(y)); }
 
-// three-input maximum without the NaN-quieting moves the library fmaxf carries
+// maxima without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
+// for results that feed a lane-swap instruction, which must not read a register in the cycle
+// after a vector instruction wrote it (the compiler cannot see that this block is one)
 __device__ __forceinline__ float max3(float x, float y, float z) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
     return r;
 }
-// (trailing wait state: the result may feed a lane-swap instruction, which must not read a
-// register in the cycle after a vector instruction wrote it, and the compiler cannot see that
-// this block is one)
 __device__ __forceinline__ float max2(float x, float y) {
     float r;
     asm("v_max_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(x), "v"(y));
     return r;
 }
-
+__device__ __forceinline__ float xor_max_fast(float v) { // all-reduce over lanes l, l^16, l^32, l^48; inputs never NaN
+    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    float r = max2(__uint_as_float(s.x), __uint_as_float(s.y));
+    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(r), __float_as_uint(r), false, false);
+    return max2(__uint_as_float(s.x), __uint_as_float(s.y));
+}
 
 // Buffer descriptor words for the global->LDS copies below: base address, stride 0, byte
-// count, raw 32-bit format.  Offsets at or past the byte count are not fetched.
+// count, raw 32-bit format.  Vector offsets at or past the byte count are not fetched.
 __device__ __forceinline__ i32x4 make_desc(const void* base, unsigned bytes) {
     const unsigned long long b = reinterpret_cast<unsigned long long>(base);
     return i32x4{(int)(unsigned)b, (int)((unsigned)(b >> 32) & 0xffffu), (int)bytes, 0x00020000};
 }
 
 // Four 1 KB global->LDS copies (buffer_load ... lds): lane l of copy i fetches 16 bytes at
-// global offset off_i + i*1024 and the load unit writes them to LDS byte lds_base + i*1024 +
-// l*16 (the immediate offset advances both addresses).  They count on the vector-memory
-// counter and complete in issue order; callers wait with s_waitcnt vmcnt(n).  Written as one
-// asm block so that M0 (the LDS base) cannot change between the copies.
-__device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int off_even, int off_odd) {
+// global offset soff + off_i + i*1024 and the load unit writes them to LDS byte lds_base +
+// i*1024 + l*16 (the immediate offset advances both addresses).  soff is a scalar and is not
+// part of the range check.  The copies count on the vector-memory counter and complete in
+// issue order; callers wait with s_waitcnt vmcnt(n).  One asm block, so that M0 (the LDS base)
+// cannot change between the copies.
+__device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int off_even, int off_odd, int soff) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
-        "buffer_load_dwordx4 %1, %3, 0 offen lds\n\t"
-        "buffer_load_dwordx4 %2, %3, 0 offen offset:1024 lds\n\t"
-        "buffer_load_dwordx4 %1, %3, 0 offen offset:2048 lds\n\t"
-        "buffer_load_dwordx4 %2, %3, 0 offen offset:3072 lds"
+        "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
+        "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds\n\t"
+        "buffer_load_dwordx4 %1, %3, %4 offen offset:2048 lds\n\t"
+        "buffer_load_dwordx4 %2, %3, %4 offen offset:3072 lds"
         :
-        : "s"(lds_base), "v"(off_even), "v"(off_odd), "s"(desc)
+        : "s"(lds_base), "v"(off_even), "v"(off_odd), "s"(desc), "s"(soff)
+        : "memory", "m0");
+}
+
+// One such copy, for the main loop, which deals them out between the matrix instructions so
+// that the vector-memory issue queue never backs up.
+template <int IMM>
+__device__ __forceinline__ void lds_copy_1k(i32x4 desc, unsigned lds_base, int off, int soff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
+        :
+        : "s"(lds_base), "v"(off), "s"(desc), "s"(soff), "n"(IMM)
         : "memory", "m0");
 }
 
@@ -139,12 +186,11 @@ template <int D, int NQB, int TQ>
 __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const FaArgs a) {
     using G = PGeom<D, NQB>;
     constexpr int kWaves = kPrefillWaves;
-    constexpr int kThreads = kWaves * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
     FA_STAMP(0);
+
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: tile indices live in scalar registers
     const int col = lane & 15;
     const int grp = lane >> 4;
 
@@ -158,16 +204,15 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     constexpr int kHeadsPerGroup = NQB * 16 / TQ;
     const int head_lo = hg * kHeadsPerGroup;
     const int tok_hi = (t0 + TQ < batch) ? t0 + TQ : batch;
-    const int kv_end = n_past + tok_hi;
-    const int full_end = n_past + t0 + 1;
+    const int kv_end = n_past + tok_hi;   // the workgroup's columns see rows [0, kv_end) at most
+    const int full_end = n_past + t0 + 1; // rows below this are visible to every column
     const int n_tiles = (kv_end + kTile - 1) / kTile;
     // Wave w owns tiles w, w+4, ...; step j visits them from the highest down.  Steps past the
-    // end map to negative tiles, whose copies fall outside the buffer descriptor and fetch nothing.
+    // end map to negative tiles, whose copies fetch nothing.
     const int n_mine = n_tiles > wave ? (n_tiles - 1 - wave) / kWaves + 1 : 0;
     auto tile_of = [&](int j) { return wave + kWaves * (n_mine - 1 - j); };
 
     unsigned char* const ws = smem + wave * G::kWaveB; // this wave's LDS slice
-    // wave-uniform by construction; readfirstlane tells the compiler so (it has to live in a scalar register)
     const unsigned ws_addr = __builtin_amdgcn_readfirstlane(
         (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ws);
     const i32x4 kdesc = make_desc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
@@ -186,145 +231,119 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         }
     }
     constexpr int kOdd = (G::kRowsPerCopy == 4) ? 1 : 0;
-    // K operand read: lane (col, grp) takes row t*16 + col, logical chunk kk*4 + grp.
-    int k_rd[G::kSteps];
+    // K operand read: lane (col, grp) takes row t*16 + col, logical chunk kk*4 + grp.  The
+    // pointers carry every per-lane term; buffer parity and sub-tile are immediate offsets.
+    const unsigned char* kp[G::kSteps];
 #pragma unroll
-    for (int kk = 0; kk < G::kSteps; ++kk) k_rd[kk] = col * G::kRowB + (((kk * 4 + grp) ^ (col & 7)) * 16);
+    for (int kk = 0; kk < G::kSteps; ++kk) kp[kk] = ws + G::kKOff + col * G::kRowB + (((kk * 4 + grp) ^ (col & 7)) * 16);
     // V transposing read: lane (col, grp) addresses row grp*4 + col/4 (+16 for the second half),
     // 8-byte column db*4 + col%4.
-    int v_rd[G::kDBlk];
+    const unsigned char* vp[G::kDBlk];
     {
         const int r0 = grp * 4 + (col >> 2), sw = r0 & 7;
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db)
-            v_rd[db] = r0 * G::kRowB + (((db * 2 + ((col & 3) >> 1)) ^ sw) * 16) + (col & 1) * 8;
+            vp[db] = ws + G::kVOff + r0 * G::kRowB + (((db * 2 + ((col & 3) >> 1)) ^ sw) * 16) + (col & 1) * 8;
     }
 
-    auto copy_tile = [&](i32x4 desc, unsigned lds_dst, int tile) { // kCopies (4 or 8) copies
+    // Prologue copies: the whole offset is in the (range-checked) vector operand, so rows at or
+    // past kv_end of the diagonal tile, and tiles below zero, are not fetched.
+    auto copy_checked = [&](const i32x4& desc, unsigned lds_dst, int tile) {
         const int base = tile * G::kTileB;
-        lds_copy_4k(desc, lds_dst, base + g_off[0], base + g_off[kOdd]);
-        if (G::kCopies > 4) lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[kOdd]);
+        lds_copy_4k(desc, lds_dst, base + g_off[0], base + g_off[kOdd], 0);
+        if (G::kCopies > 4) lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[kOdd], 0);
     };
-    auto fetch_k = [&](auto par, int tile) { copy_tile(kdesc, ws_addr + G::kKOff + decltype(par)::value * G::kTileB, tile); };
-    auto fetch_v = [&](auto par, int tile) { copy_tile(vdesc, ws_addr + G::kVOff + decltype(par)::value * G::kTileB, tile); };
+    // Main-loop copies: every tile they name is either wholly inside the visible range, and its
+    // base travels as the scalar offset, or below zero, and then the descriptor is emptied.
+    auto copy_fast = [&](const i32x4& desc, unsigned lds_dst, int tile) {
+        const bool live = tile >= 0;
+        const i32x4 d = i32x4{desc[0], desc[1], live ? desc[2] : 0, desc[3]};
+        const int soff = live ? tile * G::kTileB : 0;
+        lds_copy_4k(d, lds_dst, g_off[0], g_off[kOdd], soff);
+        if (G::kCopies > 4) lds_copy_4k(d, lds_dst + 4096, g_off[0], g_off[kOdd], soff + 4096);
+    };
+    // Copy number i (of kCopies) of a main-loop tile; desc and soff as prepared by live_desc / tile_soff.
+    auto live_desc = [&](const i32x4& desc, int tile) { return i32x4{desc[0], desc[1], tile >= 0 ? desc[2] : 0, desc[3]}; };
+    auto tile_soff = [&](int tile) { return tile >= 0 ? tile * G::kTileB : 0; };
+    auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int half = i / 4, sub = i % 4;
+        lds_copy_1k<sub * 1024>(d, lds_dst + half * 4096, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
+    };
+    auto k_buf = [&](int par) { return ws_addr + G::kKOff + par * G::kTileB; };
+    auto v_buf = [&](int par) { return ws_addr + G::kVOff + par * G::kTileB; };
 
     // ---- state ----
-    h8 q[NQB][G::kSteps];
-    int limit[NQB];
-    float m_ref[NQB], l_run[NQB];
-    f4 o[NQB][G::kDBlk];
-    f4 s[2][2][NQB]; // [parity][sub-tile][query block]
-    h8 pw[2][NQB];   // [parity][query block]
-    // Zero the slice once: a copy whose rows lie past the visible range fetches nothing, and must
-    // not expose stale bit patterns (their weights are zero, and 0 * NaN is not).  The output
-    // accumulators are cleared from the same zeros.
+    h8 q[NQB][G::kSteps]; // B operands of A: the query columns, fp16
+    float nb[NQB];        // each column's exponent offset: shift - reference maximum * c (log2 units)
+    f4 o[NQB][G::kDBlk];  // O^T accumulators (accumulation registers)
+    f4 lacc[NQB];         // row sums: every element of a lane's four holds the column's sum
+    f4 s[2][2][NQB];      // scores: [parity][sub-tile][query block]
+    u32x4 pw[2][NQB];     // P as packed fp16: [parity][query block]
+    h8 ones;
 #pragma unroll
-    for (int i = 0; i < (4 * G::kTileB + 1024) / 1024; ++i)
-        *reinterpret_cast<u32x4*>(ws + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the zero fill is done before the first copy can land
-    wave_lds_sync();
-    const unsigned scratch_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(ws + G::kScratchOff) + lane * 16;
+    for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
+    asm volatile("" : "+v"(ones)); // stays in registers; never rematerialised in front of a matrix instruction
+
+    const unsigned scratch_addr = ws_addr + G::kScratchOff + lane * 16;
+    float* const scratch = reinterpret_cast<float*>(ws + G::kScratchOff) + lane * 4;
+
+    if (n_mine > 0) {
+        // V buffer 0 receives the diagonal tile, whose rows at or past kv_end are not fetched:
+        // clear it first, so that no stale bit pattern meets a zero weight (0 * NaN is not 0).
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-        m_ref[qb] = kUnsetRef;
-        l_run[qb] = 0.0f;
-#pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db) lds_load_acc(o[qb][db], scratch_addr);
+        for (int i = 0; i < G::kCopies; ++i)
+            *reinterpret_cast<u32x4*>(ws + G::kVOff + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the fill is done before the first copy can land
+        wave_lds_sync();
+        copy_checked(kdesc, k_buf(0), tile_of(0));
+        copy_checked(vdesc, v_buf(0), tile_of(0));
+        copy_checked(kdesc, k_buf(1), tile_of(1));
+        copy_checked(vdesc, v_buf(1), tile_of(1));
     }
 
-    FA_STAMP(1);
-    auto stage_a = [&](auto kpar, auto spar) { // S[spar] = K[kpar] Q^T (prologue form: not interleaved)
-        constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
-        const unsigned char* const kb = ws + G::kKOff + KP * G::kTileB;
-#pragma unroll
-        for (int kk = 0; kk < G::kSteps; ++kk)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const h8 ka = *reinterpret_cast<const h8*>(kb + t * 16 * G::kRowB + k_rd[kk]);
-#pragma unroll
-                for (int qb = 0; qb < NQB; ++qb) {
-                    if (kk == 0) mfma_v_zero(s[SP][t][qb], ka, q[qb][kk]);
-                    else mfma_v(s[SP][t][qb], ka, q[qb][kk]);
-                    // With few query blocks the next k-step of the same accumulator is only a
-                    // couple of instructions away; give the result time to leave the pipe.
-                    if (2 * NQB < 8) asm volatile("s_nop 15");
-                }
-            }
-    };
-
-    float alpha[NQB];
-    // P[par] = 2^(S[par]*c - m_ref*c + shift); returns whether any column moved its reference
-    auto stage_b = [&](auto par, auto masked, int tile) -> bool {
-        constexpr int P = decltype(par)::value;
-        bool any_move = false;
+    FA_STAMP(9);
+    // ---- query columns -> B operands ----
+    int limit[NQB];
+    {
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
-            float v[8];
+            const int c = qb * 16 + col;
+            const int tok = t0 + c % TQ;
+            const int hl = head_lo + c / TQ;
+            const bool valid = (hl < a.r) && (tok < batch);
+            limit[qb] = valid ? n_past + tok + 1 : 0x7fffffff;
+            const float* qp = a.q + ((size_t)(valid ? tok : 0) * a.n_head + (size_t)(valid ? kvh * a.r + hl : 0)) * D;
+            const float qmul = valid ? a.qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int kk = 0; kk < G::kSteps; ++kk) {
+                const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
+                const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                h8 hv;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) v[t * 4 + i] = s[P][t][qb][i];
-            if (decltype(masked)::value) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int row = tile * kTile + t * 16 + grp * 4 + i;
-                        if (row >= limit[qb]) v[t * 4 + i] = -INFINITY;
-                    }
+                for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(x[e] * qmul);
+                asm volatile("" : "=a"(q[qb][kk]) : "0"(hv)); // parked in the accumulation-register file for good
             }
-            float mx = max3(v[0], v[1], v[2]);
-            mx = max3(mx, v[3], v[4]);
-            mx = max3(mx, v[5], v[6]);
-            mx = xor_max_fast(max2(mx, v[7]));
-            const bool move = (mx - m_ref[qb]) * a.c > kLazy; // an unset reference is far below any score
-            alpha[qb] = fast_exp2(move ? (m_ref[qb] - mx) * a.c : 0.0f);
-            m_ref[qb] = move ? mx : m_ref[qb];
-            any_move |= move;
-            const float nb = kPShift - m_ref[qb] * a.c;
-            float sum = 0.0f;
-            h8 ph;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float p = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
-                sum += p;
-                ph[e] = (_Float16)p;
-            }
-            l_run[qb] = l_run[qb] * alpha[qb] + sum;
-            pw[P][qb] = ph;
         }
-        return __builtin_amdgcn_ballot_w64(any_move) != 0;
-    };
+    }
+    FA_STAMP(10);
+    // O = 0, l = 0: a matrix instruction with a zero addend writes the accumulation registers
+    // without touching memory (0 * Q is 0 for finite Q; a non-finite Q spoils its column anyway).
+    {
+        h8 zero;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) zero[e] = (_Float16)0.0f;
+        asm volatile("" : "+v"(zero));
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db) mfma_a_zero_n(o[qb][db], zero, zero);
+            mfma_a_zero_n(lacc[qb], zero, zero);
+        }
+    }
+    FA_STAMP(1);
 
-    auto stage_c = [&](auto par) { // O += V[par]^T P[par]
-        constexpr int P = decltype(par)::value;
-        const unsigned char* const vb = ws + G::kVOff + P * G::kTileB;
-#pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db) {
-            const h4 v0 = lds_read_tr(vb + v_rd[db]);
-            const h4 v1 = lds_read_tr(vb + 16 * G::kRowB + v_rd[db]);
-            const h8 va = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) mfma_a(o[qb][db], va, pw[P][qb]);
-        }
-    };
-    // Rare (a column's reference maximum moved): O *= alpha, one accumulator at a time through a
-    // 16-byte-per-lane LDS scratch so that O never becomes an operand of an ordinary vector instruction.
-    auto rescale = [&]() {
-        settle(); // the last accumulation into O has left the matrix pipe
-        f4* const scratch = reinterpret_cast<f4*>(ws + G::kScratchOff) + lane;
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db) {
-                lds_store_acc(scratch_addr, o[qb][db]);
-                f4 x = *scratch;
-                x *= alpha[qb];
-                *scratch = x;
-                lds_load_acc(o[qb][db], scratch_addr);
-            }
-        settle();
-    };
     // The copies are tracked by the vector-memory counter and complete in issue order: waiting
     // until at most `newer` younger ones are outstanding guarantees a tile has landed.
     auto wait_copies = [&](auto newer) {
@@ -335,237 +354,317 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     constexpr int kC = G::kCopies;
 
     if (n_mine > 0) {
-        fetch_k(IntC<0>{}, tile_of(0));
-        fetch_v(IntC<0>{}, tile_of(0));
-        fetch_k(IntC<1>{}, tile_of(1));
-        fetch_v(IntC<1>{}, tile_of(1));
-
-        // ---- query columns -> B operands ----
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
-            const int c = qb * 16 + col;
-            const int tok = t0 + c % TQ;
-            const int hl = head_lo + c / TQ;
-            const bool valid = (hl < a.r) && (tok < batch);
-            limit[qb] = valid ? n_past + tok + 1 : 0x7fffffff;
-            const float* qp = a.q + ((size_t)(valid ? tok : 0) * a.n_head + (size_t)(valid ? kvh * a.r + hl : 0)) * D;
-            const float qmul = valid ? a.qsign : 0.0f;
-#pragma unroll
-            for (int kk = 0; kk < G::kSteps; ++kk) {
-                const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
-                const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
-                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                h8 hv;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(x[e] * qmul);
-                q[qb][kk] = hv;
-            }
-        }
-
-        FA_STAMP(2);
-        // Copy issue order: K0 V0 K1 V1 | K2 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
-        // ---- step 0: the diagonal tile, the only one that can need the causal mask ----
         const int R = n_mine - 1; // steps after step 0
-        wait_copies(IntC<3 * kC>{});               // K0 landed (V0 K1 V1 may be in flight)
-        stage_a(IntC<0>{}, IntC<0>{});             // S(0)
-        __builtin_amdgcn_s_waitcnt(0xC07F);        // its LDS reads have returned: K buffer 0 is free
-        fetch_k(IntC<0>{}, tile_of(2));
+        // Prologue form of A: S[spar] = K[kpar] Q^T with a zero addend, operands read up front.
+        auto stage_a0 = [&](auto kpar, auto spar) {
+            constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
+            h8 ka[G::kSteps][2];
+#pragma unroll
+            for (int kk = 0; kk < G::kSteps; ++kk)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    ka[kk][t] = *reinterpret_cast<const h8*>(kp[kk] + KP * G::kTileB + t * 16 * G::kRowB);
+#pragma unroll
+            for (int kk = 0; kk < G::kSteps; ++kk)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int qb = 0; qb < NQB; ++qb) {
+                        if (kk == 0) mfma_v_zero_n(s[SP][t][qb], ka[kk][t], q[qb][kk]);
+                        else mfma_v_n(s[SP][t][qb], ka[kk][t], q[qb][kk]);
+                        // With few query blocks the next k-step of the same accumulator is only a
+                        // couple of instructions away; give the result time to leave the pipe.
+                        if (2 * NQB < 8) asm volatile("s_nop 15");
+                    }
+        };
+        // Copy issue order: K0 V0 K1 V1 | K2 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
+        // (within a step, K goes out over the first tickets and V over the last)
+        // ---- step 0: the diagonal tile, the only one that can need the causal mask ----
+        wait_copies(IntC<3 * kC>{});        // K0 landed (V0 K1 V1 may be in flight)
+        stage_a0(IntC<0>{}, IntC<0>{});     // S(0)
+        __builtin_amdgcn_s_waitcnt(0xC07F); // its LDS reads have returned: K buffer 0 is free
+        copy_fast(kdesc, k_buf(0), tile_of(2));
         if (R > 0) {
-            wait_copies(IntC<2 * kC>{});           // K1 landed (V1 K2 may be in flight)
-            stage_a(IntC<1>{}, IntC<1>{});         // S(1)
+            wait_copies(IntC<2 * kC>{});    // K1 landed (V1 K2 may be in flight)
+            stage_a0(IntC<1>{}, IntC<1>{}); // S(1)
         }
         settle();
-        if (tile_of(0) * kTile + kTile > full_end) stage_b(IntC<0>{}, IntC<1>{}, tile_of(0));
-        else stage_b(IntC<0>{}, IntC<0>{}, tile_of(0));
-        // (O is still zero: no rescale)
-
+        FA_STAMP(2);
+        // Reference maximum of each column: over its visible scores of tile 0 and, when there is
+        // one, tile 1 (every row of which is visible to every column).  A column with no visible
+        // row in this wave keeps weight zero whatever the reference.
+        {
+            const int row0 = tile_of(0) * kTile + grp * 4;
+            const bool masked = tile_of(0) * kTile + kTile > full_end;
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                float v[8];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        v[t * 4 + i] = s[0][t][qb][i];
+                        if (masked && row0 + t * 16 + i >= limit[qb]) v[t * 4 + i] = -INFINITY;
+                    }
+                float mx = max3(v[0], v[1], v[2]);
+                mx = max3(mx, v[3], v[4]);
+                mx = max3(mx, v[5], v[6]);
+                mx = max2(mx, v[7]);
+                if (R > 0) {
+                    mx = max3(mx, s[1][0][qb][0], s[1][0][qb][1]);
+                    mx = max3(mx, s[1][0][qb][2], s[1][0][qb][3]);
+                    mx = max3(mx, s[1][1][qb][0], s[1][1][qb][1]);
+                    mx = max3(mx, s[1][1][qb][2], s[1][1][qb][3]);
+                    mx = max2(mx, mx);
+                }
+                mx = xor_max_fast(mx);
+                nb[qb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
+                h8 ph;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ph[e] = (_Float16)fast_exp2(__builtin_fmaf(v[e], a.c, nb[qb]));
+                pw[0][qb] = __builtin_bit_cast(u32x4, ph);
+            }
+        }
+        settle(); // (the vector writes of P are well clear of the next matrix instruction)
         FA_STAMP(3);
-        // ---- steps t >= 1: A(t+1), B(t) and C(t-1) share one hand-ordered instruction stream.
-        // The 2 * kGroups/2 * NQB matrix instructions of A and C are cut into groups of NQB that
-        // share an LDS operand (A: one (k-step, sub-tile) of K; C: one 16-wide block of V^T),
-        // ordered A0 C0 A1 C1 ...; the vector work of B is cut into 16 sites per query block and
-        // each site is followed by its share of the matrix instructions, so the matrix pipe is
-        // fed while the exponentials run.  Operands are read from LDS two groups ahead.
-        // `newer` = copies issued after K(t+1): K(t+2) only at t == 1 (step 0 issued no V),
-        // V(t) and K(t+2) afterwards. ----
-        constexpr int kGroups = 2 * G::kSteps + G::kDBlk; // 2*kSteps == kDBlk
+
+        // ---- steps t >= 1: A(t+1), B(t) and C(t-1) in one instruction stream.  The matrix
+        // instructions are cut into groups of NQB that share an LDS operand (A: one (k-step,
+        // sub-tile) of K; C: one 16-wide block of V^T; last, the row sums), ordered A0 C0 A1 C1
+        // ... L; the 24 vector instructions per query block of B are dealt out evenly between
+        // them.  Operands are read from LDS kAhead groups ahead of their use.
+        // `newer` = copies issued after K(t+1) and before the wait: none at t == 1 (step 0 issued
+        // K(2) last), V(t) afterwards. ----
         static_assert(2 * G::kSteps == G::kDBlk, "A and C groups alternate one to one");
-        auto body = [&](auto tpar, auto has_next, auto newer, int t) {
+        constexpr int kGroups = 2 * G::kSteps + G::kDBlk; // groups with an LDS operand
+        constexpr int kTickets = (kGroups + 1) * NQB;     // matrix instructions per step
+        constexpr int kItems = 24 * NQB;                  // vector instructions of B per step
+        constexpr int kAhead = 3;
+        constexpr float kBound = kLazy + kPShift;         // largest exponent P may be built from
+        constexpr float kBoundP = 32768.0f;               // = 2^kBound
+        // (The last step has no tile t+1: its A stage multiplies whatever the K buffer holds and
+        // nobody reads the result -- cheaper than a second copy of the loop body without it.)
+        float c = a.c;
+        asm volatile("" : "+v"(c)); // a vector register for the whole loop, not a move per step
+        auto body = [&](auto tpar, auto newer, int t) {
             constexpr int TP = decltype(tpar)::value; // t & 1
-            constexpr bool HN = decltype(has_next)::value;
             // (Every LDS read of the previous step has been consumed by a matrix instruction that
             // was issued before this point, so the K buffer A(t) read is free.)
-            fetch_k(IntC<TP>{}, tile_of(t + 2));                       // K(t+2) -> the buffer A(t) read
-            wait_copies(newer);                                         // K(t+1) landed; V(t-1) is older
-            const unsigned char* const kb = ws + G::kKOff + (TP ^ 1) * G::kTileB;
-            const unsigned char* const vb = ws + G::kVOff + (TP ^ 1) * G::kTileB;
+            // K(t+2) goes to the buffer A(t) read; its copies are dealt out over the first tickets.
+            // (Issued after this step's wait, they are not among the `newer` copies any more.)
+            const i32x4 kd = live_desc(kdesc, tile_of(t + 2));
+            const int ksoff = tile_soff(tile_of(t + 2));
+            const i32x4 vd = live_desc(vdesc, tile_of(t + 1));
+            const int vsoff = tile_soff(tile_of(t + 1));
+            wait_copies(newer);                          // K(t+1) landed; V(t-1) is older
             h8 gop[kGroups];
             auto issue_read = [&](auto gc) {
                 constexpr int g = decltype(gc)::value;
+                __builtin_amdgcn_sched_barrier(0);
                 if constexpr (g % 2 == 0) {
                     constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
-                    if (HN) gop[g] = *reinterpret_cast<const h8*>(kb + tt * 16 * G::kRowB + k_rd[kk]);
+                    gop[g] = *reinterpret_cast<const h8*>(kp[kk] + (TP ^ 1) * G::kTileB + tt * 16 * G::kRowB);
                 } else {
                     constexpr int db = g / 2;
-                    const h4 v0 = lds_read_tr(vb + v_rd[db]);
-                    const h4 v1 = lds_read_tr(vb + 16 * G::kRowB + v_rd[db]);
+                    const h4 v0 = lds_read_tr(vp[db] + (TP ^ 1) * G::kTileB);
+                    const h4 v1 = lds_read_tr(vp[db] + (TP ^ 1) * G::kTileB + 16 * G::kRowB);
                     gop[g] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             };
-            auto ticket = [&](auto ic) {
+            float pe[NQB][8];
+            float amax;
+            // Vector instruction j of B(t).  Per query block and pair of scores: two multiply-adds
+            // (the exponents), two exponentials, the running maximum of the weights, the conversion;
+            // no instruction reads the result of the one right before it.
+            auto item = [&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                constexpr int qb = j / 24, r = j % 24;
+                // 0 multiply-add, 1 maximum, 2 exponential, 3 conversion
+                constexpr int kind[24] = {0, 0, 2, 2, 0, 0, 1, 2, 2, 3, 0, 0, 1, 2, 2, 3, 0, 0, 1, 2, 2, 3, 1, 3};
+                constexpr int arg[24] = {0, 1, 0, 1, 2, 3, 0, 2, 3, 0, 4, 5, 1, 4, 5, 1, 6, 7, 2, 6, 7, 2, 3, 3};
+                constexpr int x = arg[r];
+                if constexpr (kind[r] == 0) {
+                    v_fma(pe[qb][x], s[TP][x / 4][qb][x % 4], c, nb[qb]);
+                } else if constexpr (kind[r] == 2) {
+                    v_exp2(pe[qb][x]);
+                } else if constexpr (kind[r] == 3) {
+                    unsigned packed;
+                    v_cvt_pk(packed, pe[qb][2 * x], pe[qb][2 * x + 1]);
+                    pw[TP][qb][x] = packed;
+                } else {
+                    if constexpr (j == 6) v_max2(amax, pe[qb][2 * x], pe[qb][2 * x + 1]);
+                    else v_max3_acc(amax, pe[qb][2 * x], pe[qb][2 * x + 1]);
+                }
+            };
+            static_for<0, kAhead>(issue_read);
+            static_for<0, kTickets>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 constexpr int g = i / NQB, m = i % NQB;
-                if constexpr (m == 0 && g + 2 < kGroups) issue_read(IntC<g + 2>{});
-                if constexpr (g % 2 == 0) {
+                if constexpr (m == 0 && g + kAhead < kGroups) issue_read(IntC<g + kAhead>{});
+                if constexpr (g == kGroups) {
+                    mfma_a(lacc[m], ones, __builtin_bit_cast(h8, pw[TP ^ 1][m]));
+                } else if constexpr (g % 2 == 0) {
                     constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
-                    if (HN) {
-                        if constexpr (kk == 0) mfma_v_zero(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
-                        else mfma_v(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
-                    }
+                    if constexpr (kk == 0) mfma_v_zero(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
+                    else mfma_v(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
                 } else {
-                    mfma_a(o[m][g / 2], gop[g], pw[TP ^ 1][m]);
+                    mfma_a(o[m][g / 2], gop[g], __builtin_bit_cast(h8, pw[TP ^ 1][m]));
                 }
-            };
-            issue_read(IntC<0>{});
-            issue_read(IntC<1>{});
-            // Matrix instruction tickets: NQB go to phase 0 (one per query block), the rest are
-            // spread over the 10 vector sites of each query block in phase 1.
-            constexpr int kPerQb = kGroups - 1;
-            auto tickets = [&](auto loc, auto hic) {
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<decltype(loc)::value, decltype(hic)::value>(ticket);
-                __builtin_amdgcn_sched_barrier(0);
-            };
-            // ---- phase 0: has any score outgrown its column's reference maximum?  Lane-local
-            // maxima only (no lane exchange, no execution-mask games: both stall the matrix pipe);
-            // the answer is "no" on all but the first few tiles.
-            float lmax[NQB];
-            float excess = -INFINITY;
-            static_for<0, NQB>([&](auto qbc) {
-                constexpr int qb = decltype(qbc)::value;
-                float mx = max3(s[TP][0][qb][0], s[TP][0][qb][1], s[TP][0][qb][2]);
-                mx = max3(mx, s[TP][0][qb][3], s[TP][1][qb][0]);
-                mx = max3(mx, s[TP][1][qb][1], s[TP][1][qb][2]);
-                mx = max2(mx, s[TP][1][qb][3]);
-                lmax[qb] = mx;
-                excess = max2(excess, (mx - m_ref[qb]) * a.c);
-                tickets(IntC<qb>{}, IntC<qb + 1>{});
+                static_for<(i * kItems) / kTickets, ((i + 1) * kItems) / kTickets>(item);
+                if constexpr (i % 2 == 1 && i / 2 < kC) copy_one(IntC<i / 2>{}, kd, k_buf(TP), ksoff);
+                // V(t+1) goes to the buffer C(t-1) reads: its copies wait for the last of those reads
+                // to be consumed, which the row-sum group (no LDS operand) marks.
+                if constexpr (g == kGroups) {
+                    constexpr int per = (kC + NQB - 1) / NQB;
+                    static_for<m * per, (m + 1) * per < kC ? (m + 1) * per : kC>([&](auto cc) { copy_one(cc, vd, v_buf(TP ^ 1), vsoff); });
+                }
             });
-            bool moved = false;
-            if (__builtin_amdgcn_ballot_w64(excess > kLazy) != 0) {
-                moved = true;
+            // S(t+1) is alive to the end of the step even when nobody reads it (last step): its
+            // registers must not be handed out while the matrix instructions that write them are in flight.
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                asm volatile("" : : "v"(s[TP ^ 1][0][qb]));
+                asm volatile("" : : "v"(s[TP ^ 1][1][qb]));
+            }
+            // ---- slow path: some exponent of this tile is above the bound.  Move the reference of
+            // the columns concerned to their new maximum, redo P(t) and rescale O and l -- one
+            // accumulator at a time through a 16-byte-per-lane LDS scratch, so that they never
+            // become operands of a vector instruction. ----
+            if (__builtin_amdgcn_ballot_w64(amax > kBoundP) != 0) {
+                settle(); // C(t-1) has left the matrix pipe
+                float alpha[NQB];
 #pragma unroll
                 for (int qb = 0; qb < NQB; ++qb) {
-                    const float mx = xor_max_fast(lmax[qb]);
-                    const bool move = (mx - m_ref[qb]) * a.c > kLazy;
-                    alpha[qb] = fast_exp2(move ? (m_ref[qb] - mx) * a.c : 0.0f);
-                    m_ref[qb] = move ? mx : m_ref[qb];
-                    l_run[qb] *= alpha[qb];
+                    float mx = max3(s[TP][0][qb][0], s[TP][0][qb][1], s[TP][0][qb][2]);
+                    mx = max3(mx, s[TP][0][qb][3], s[TP][1][qb][0]);
+                    mx = max3(mx, s[TP][1][qb][1], s[TP][1][qb][2]);
+                    mx = xor_max_fast(max2(mx, s[TP][1][qb][3]));
+                    const float top = __builtin_fmaf(mx, c, nb[qb]); // the column's largest exponent
+                    const float delta = top > kBound ? top - kPShift : 0.0f;
+                    alpha[qb] = fast_exp2(-delta);
+                    nb[qb] -= delta;
+                    h8 ph;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ph[e] = (_Float16)fast_exp2(__builtin_fmaf(s[TP][e / 4][qb][e % 4], c, nb[qb]));
+                    pw[TP][qb] = __builtin_bit_cast(u32x4, ph);
                 }
-            }
-            // ---- phase 1: P(t) = 2^(S*c - m_ref*c + shift), row sums, fp16 ----
-            static_for<0, NQB>([&](auto qbc) {
-                constexpr int qb = decltype(qbc)::value;
-                constexpr int base = NQB + qb * kPerQb;
-                auto site = [&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    tickets(IntC<base + j * kPerQb / 10>{}, IntC<base + (j + 1) * kPerQb / 10>{});
+                auto scale_acc = [&](f4& acc, float al) {
+                    lds_store_acc(scratch_addr, acc);
+                    f4 x = *reinterpret_cast<f4*>(scratch);
+                    x *= al;
+                    *reinterpret_cast<f4*>(scratch) = x;
+                    lds_load_acc(acc, scratch_addr);
                 };
-                const float nb = kPShift - m_ref[qb] * a.c;
-                float sum = 0.0f;
-                h8 ph;
-                static_for<0, 8>([&](auto ec) {
-                    constexpr int e = decltype(ec)::value;
-                    float pe = fast_exp2(__builtin_fmaf(s[TP][e / 4][qb][e % 4], a.c, nb));
-                    // An empty volatile block that "rewrites" the value: it keeps its order among
-                    // the matrix instructions, so the exponential stays at this site instead of
-                    // being sunk into the next iteration next to its first use.
-                    asm volatile("" : "+v"(pe));
-                    sum += pe;
-                    ph[e] = (_Float16)pe;
-                    site(IntC<e>{});
+                static_for<0, NQB>([&](auto qbc) {
+                    constexpr int qb = decltype(qbc)::value;
+                    static_for<0, G::kDBlk>([&](auto dbc) { scale_acc(o[qb][decltype(dbc)::value], alpha[qb]); });
+                    scale_acc(lacc[qb], alpha[qb]);
                 });
-                asm volatile("" : "+v"(ph));
-                l_run[qb] += sum;
-                pw[TP][qb] = ph;
-                site(IntC<8>{});
-                site(IntC<9>{});
-            });
-            fetch_v(IntC<TP ^ 1>{}, tile_of(t + 1));                   // V(t+1) -> the buffer C(t-1) read (all consumed)
-            if (moved) rescale();
+                settle();
+            }
         };
-        if (R >= 1) {
-            if (R == 1) body(IntC<1>{}, IntC<0>{}, IntC<kC>{}, 1);
-            else body(IntC<1>{}, IntC<1>{}, IntC<kC>{}, 1);
-        }
+        if (R >= 1) body(IntC<1>{}, IntC<0>{}, 1);
         int t = 2;
-        while (t + 1 < R) { // t even
-            body(IntC<0>{}, IntC<1>{}, IntC<2 * kC>{}, t);
-            body(IntC<1>{}, IntC<1>{}, IntC<2 * kC>{}, t + 1);
-            t += 2;
+        for (; t + 1 <= R; t += 2) {
+            body(IntC<0>{}, IntC<kC>{}, t);
+            body(IntC<1>{}, IntC<kC>{}, t + 1);
         }
-        if (t < R) { // steps t (even) and t + 1 == R
-            body(IntC<0>{}, IntC<1>{}, IntC<2 * kC>{}, t);
-            body(IntC<1>{}, IntC<0>{}, IntC<2 * kC>{}, t + 1);
-        } else if (t == R) {
-            body(IntC<0>{}, IntC<0>{}, IntC<2 * kC>{}, t);
-        }
+        if (t == R) body(IntC<0>{}, IntC<kC>{}, t);
         FA_STAMP(4);
         // ---- drain: C(R) ----
         wait_copies(IntC<0>{});
         settle(); // P(R) was converted just above
-        if (R & 1) stage_c(IntC<1>{});
-        else stage_c(IntC<0>{});
+        {   // O += V(R)^T P(R), l += 1^T P(R); both live in the buffers of parity R & 1
+            const bool odd = (R & 1) != 0;
+            const int v_par = odd ? G::kTileB : 0;
+            h8 va[G::kDBlk], pl[NQB];
+            if (odd) {
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb) pw[0][qb] = pw[1][qb];
+            }
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db) {
+                const h4 v0 = lds_read_tr(vp[db] + v_par);
+                const h4 v1 = lds_read_tr(vp[db] + v_par + 16 * G::kRowB);
+                va[db] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) pl[qb] = __builtin_bit_cast(h8, pw[0][qb]);
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db)
+#pragma unroll
+                for (int qb = 0; qb < NQB; ++qb) mfma_a_n(o[qb][db], va[db], pl[qb]);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) mfma_a_n(lacc[qb], ones, pl[qb]);
+        }
         __builtin_amdgcn_s_waitcnt(0xC07F); // every read of the tile buffers has returned: the merge reuses them
-        settle();                            // and O is out of the matrix pipe
-        wave_lds_sync();
+    } else {
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) nb[qb] = 0.0f;
     }
-
+    settle(); // O and l are out of the matrix pipe
+    wave_lds_sync();
     FA_STAMP(5);
+
     // ---- merge the four waves through LDS ----
+    // (m, l) per wave and column, m = the reference in log2 units (the common shift cancels);
+    // a wave that saw no visible row of a column has l = 0 and is given m = -inf (weight 0).
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
-    const unsigned obuf_addr = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)(smem + wave * G::kWaveB);
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        const float l_tot = xor_sum(l_run[qb]);
+        lds_store_acc(scratch_addr, lacc[qb]);
+        const float l_tot = scratch[0];
         if (grp == 0) {
-            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = m_ref[qb] * a.c; // unset: hugely negative, weight 0
+            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = l_tot > 0.0f ? -nb[qb] : -INFINITY;
             ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 1] = l_tot;
         }
-#pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db)
-            lds_store_acc(obuf_addr + ((qb * 16 + col) * G::kOStride + db * 16 + grp * 4) * 4, o[qb][db]);
     }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    wave_lds_sync(); // the scratch lies inside the merge buffer when the tile is small
+    const unsigned obuf_addr = ws_addr + (col * G::kOStride + grp * 4) * 4;
+    static_for<0, NQB>([&](auto qbc) {
+        static_for<0, G::kDBlk>([&](auto dbc) {
+            constexpr int qb = decltype(qbc)::value, db = decltype(dbc)::value;
+            lds_store_acc_nowait<(qb * 16 * G::kOStride + db * 16) * 4>(obuf_addr, o[qb][db]);
+        });
+    });
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     FA_STAMP(6);
     __syncthreads();
     FA_STAMP(7);
 
+    // Four threads per column: the weights are computed once, then each thread merges and stores
+    // a quarter of the column's head_dim in 16-byte pieces (the four pieces of a step are one
+    // contiguous 64 bytes of the output row).
     constexpr int kCols = NQB * 16;
-    for (int idx = threadIdx.x; idx < kCols * (D / 4); idx += kThreads) {
-        const int c = idx / (D / 4);
-        const int d4 = (idx % (D / 4)) * 4;
-        const int tok = t0 + c % TQ;
-        const int hl = head_lo + c / TQ;
-        if (hl >= a.r || tok >= batch) continue;
-        float mw[kWaves], lw[kWaves];
-        float m_all = -INFINITY;
+    const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
+    const int tok = t0 + c % TQ;
+    const int hl = head_lo + c / TQ;
+    if (c < kCols && hl < a.r && tok < batch) {
+        float wgt[kWaves];
+        float m_all = -INFINITY, l_all = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            mw[w] = ml[(w * kCols + c) * 2 + 0];
-            lw[w] = ml[(w * kCols + c) * 2 + 1];
-            m_all = fmaxf(m_all, mw[w]);
+            wgt[w] = ml[(w * kCols + c) * 2 + 0];
+            m_all = fmaxf(m_all, wgt[w]);
         }
-        float l_all = 0.0f;
-        f4 acc = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            const float wgt = fast_exp2(mw[w] - m_all); // a wave that saw no visible row has m = -inf -> weight 0
-            l_all += lw[w] * wgt;
-            const f4 ow = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4);
-            acc += ow * wgt;
+            wgt[w] = fast_exp2(wgt[w] - m_all); // the wave that holds the column's diagonal has a finite m
+            l_all += ml[(w * kCols + c) * 2 + 1] * wgt[w];
         }
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
-        *reinterpret_cast<f4*>(a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D + d4) = acc * inv;
+        float* const dst = a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D;
+#pragma unroll
+        for (int j = 0; j < D / 16; ++j) {
+            const int d4 = (j * 4 + part) * 4;
+            f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w)
+                acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4) * wgt[w];
+            *reinterpret_cast<f4*>(dst + d4) = acc * inv;
+        }
     }
     FA_STAMP(8);
 }
@@ -591,11 +690,12 @@ hipError_t allow_lds_all() {
     if ((e = allow_lds<D, 3, 16>()) != hipSuccess) return e;
     if ((e = allow_lds<D, 4, 16>()) != hipSuccess) return e;
     if ((e = allow_lds<D, 3, 8>()) != hipSuccess) return e;
+    if ((e = allow_lds<D, 2, 4>()) != hipSuccess) return e;
     return allow_lds<D, 4, 8>();
 }
 
 template <int D>
-hipError_t launch(FaArgs a, hipStream_t stream) {
+hipError_t launch(FaArgs a, int cu_count, hipStream_t stream) {
     // Column packing per GQA ratio: (16-column blocks, tokens per workgroup).
     // r <= 4: 16 tokens x r heads; r in 5..8: 8 tokens x up to 8 heads; larger ratios
     // are cut into groups of 8 heads that each re-read the KV head.
@@ -604,11 +704,19 @@ hipError_t launch(FaArgs a, hipStream_t stream) {
     if (r <= 4) { nqb = r; tq = 16; }
     else if (r <= 6) { nqb = 3; tq = 8; }
     else { nqb = 4; tq = 8; }
+    // A workgroup occupies a whole CU and the kernel lasts as long as its longest workgroup, so
+    // a grid that leaves half the CUs idle is better cut finer: 4 tokens x up to 8 heads, which
+    // halves the columns (and the time) per workgroup for r = 5..8.
+    if (r > 4 && 2 * a.n_kv * ((r + nqb * 16 / tq - 1) / (nqb * 16 / tq)) * ((a.batch + tq - 1) / tq) <= cu_count) {
+        nqb = 2;
+        tq = 4;
+    }
     const int heads_per_group = nqb * 16 / tq;
     a.n_hgroups = (r + heads_per_group - 1) / heads_per_group;
     a.n_ttiles = (a.batch + tq - 1) / tq;
     const int grid = a.n_kv * a.n_hgroups * a.n_ttiles;
     switch (nqb * 100 + tq) {
+        case 204: return launch_kernel<D, 2, 4>(a, grid, stream);
         case 116: return launch_kernel<D, 1, 16>(a, grid, stream);
         case 216: return launch_kernel<D, 2, 16>(a, grid, stream);
         case 316: return launch_kernel<D, 3, 16>(a, grid, stream);
@@ -620,8 +728,8 @@ hipError_t launch(FaArgs a, hipStream_t stream) {
 
 } // namespace
 
-hipError_t prefill_launch(const FaArgs& a, int head_dim, hipStream_t stream) {
-    return head_dim == 128 ? launch<128>(a, stream) : launch<64>(a, stream);
+hipError_t prefill_launch(const FaArgs& a, int head_dim, int cu_count, hipStream_t stream) {
+    return head_dim == 128 ? launch<128>(a, cu_count, stream) : launch<64>(a, cu_count, stream);
 }
 
 // The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at init.

@@ -154,10 +154,12 @@ def test_prefill_row_equals_decode_and_chunk_split(fa):
     whole = gpu_prefill(fa, q, kc, vc, H, G, d, n_ctx, n_past, batch, scale)
     a = gpu_prefill(fa, q[:77], kc, vc, H, G, d, n_ctx, n_past, 77, scale)
     b = gpu_prefill(fa, q[77:], kc, vc, H, G, d, n_ctx, n_past + 77, batch - 77, scale)
-    check(np.concatenate([a, b]), whole, "chunk split", tol=2e-4)
+    # (the weights are rounded to fp16 relative to a reference that depends on how the rows fall
+    # into tiles, so two chunkings agree to the size of that rounding, not bit for bit)
+    check(np.concatenate([a, b]), whole, "chunk split", tol=1e-3)
     for t in (0, 76, 199):
         dec = gpu_decode(fa, q[t], kc, vc, H, G, d, n_ctx, n_past + t, scale)
-        check(dec, whole[t], f"prefill row {t} vs decode", tol=5e-4)
+        check(dec, whole[t], f"prefill row {t} vs decode", tol=1e-3)
 
 
 def test_decode_ignores_cache_tail_and_position_is_read_on_device(fa):
