@@ -84,8 +84,8 @@ __device__ __forceinline__ float xor_sum(float v) {
 }
 
 // 16-byte load through a buffer descriptor: the hardware returns zeros for offsets at or
-// past the descriptor's byte count, so cache rows beyond the visible range (which may hold
-// anything, NaN patterns included) are never fetched and need no branch.
+// past the descriptor's byte count, so rows beyond the bound are never fetched and need no
+// branch.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }

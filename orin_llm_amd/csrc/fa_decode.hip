@@ -16,10 +16,18 @@
 //     over K and V.  The matrix pipe is idle most of the time here, so Q and P are carried as
 //     fp16 hi + lo pairs and the result is accurate to fp32 rounding.
 //   * The position is read on the device; the launch shape depends only on by-value arguments,
-//     so the launch can be captured in a graph and replayed after the position changes.
+//     so the launch can be captured in a graph and replayed after the position changes.  Every
+//     wave requests its first tile before the position has arrived (one memory round trip less
+//     on the critical path): the loads are bounded by n_ctx, which is always safe, and rows at
+//     or past the position are masked (K) or zeroed on their way into LDS (V) afterwards.
 //   * Partials (reference maximum, row sum, O) of the 8 waves are merged through LDS and
 //     written per split; the combine kernel merges the splits that were active.
 #include "fa_common.hpp"
+
+// Cycle-counter stamps for profiling builds (defined by a prefix header there); nothing otherwise.
+#ifndef FA_STAMP
+#define FA_STAMP(i)
+#endif
 
 namespace orin_fa {
 namespace {
@@ -45,6 +53,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     constexpr int kWaves = kDecodeWaves;
     constexpr int kThreads = kWaves * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    FA_STAMP(0);
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -58,17 +67,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     const int hg = id % a.n_hgroups;
     id /= a.n_hgroups; // = split
 
-    int p = *a.d_pos;
-    p = p < 0 ? 0 : p;
-    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
-    const int n_tiles = (npos + kTile - 1) / kTile;
     const int tile_first = id * kWaves + wave;
     const int tile_step = kWaves * a.n_splits;
-    if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
-
     unsigned char* const vs = smem + wave * G::kWaveB;
-    const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)npos * D * 2);
-    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)npos * D * 2);
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
 
     u32x4 kreg[2 * G::kSteps], vreg[G::kLoads];
     auto fetch_k = [&](int tile) {
@@ -85,11 +88,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         for (int i = 0; i < G::kLoads; ++i) vreg[i] = buf_load16<true>(vrs, soff + (i * 64 + lane) * 16);
     };
     int tile = tile_first;
-    if (tile < n_tiles) { // in flight while the query heads are loaded and converted
-        fetch_k(tile);
-        fetch_v(tile);
-    }
+    fetch_k(tile); // in flight while the position and the query heads are loaded
+    fetch_v(tile);
 
+    int p = *a.d_pos;
+    p = p < 0 ? 0 : p;
+    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
+    const int n_tiles = (npos + kTile - 1) / kTile;
+    if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
+
+    FA_STAMP(1);
     // ---- query heads -> B operands, fp16 hi + lo ----
     const int hl = hg * 16 + col;
     const bool valid = hl < a.r;
@@ -109,6 +117,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         }
     }
 
+    FA_STAMP(2);
     // m_ref: reference maximum of the raw scores (before the scale); l_run: this lane's share of
     // the row sum; o: O^T accumulators, lane (col, grp) holds head_dim rows db*16 + grp*4 + i.
     float m_ref = -INFINITY, l_run = 0.0f;
@@ -119,14 +128,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 
     for (; tile < n_tiles; tile += tile_step) {
         const bool more = tile + tile_step < n_tiles;
-#pragma unroll
-        for (int i = 0; i < G::kLoads; ++i) {
-            const int c = i * 64 + lane;
-            *reinterpret_cast<u32x4*>(vs + (c / G::kChunksPerRow) * G::kRowBV + (c % G::kChunksPerRow) * 16) = vreg[i];
-        }
-        if (more) fetch_v(tile + tile_step);
-        wave_lds_sync();
-
         // ---- S^T = K Q^T : rows = KV row (sub-tile t, row col), columns = query head ----
         f4 s[2], s2[2]; // the Q-lo product runs as its own accumulation chain
 #pragma unroll
@@ -142,6 +143,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         s[0] += s2[0];
         s[1] += s2[1];
         if (more) fetch_k(tile + tile_step); // the operand registers are free again
+        FA_STAMP(3);
 
         // ---- softmax weights; lane (col, grp) holds rows t*16 + grp*4 + i of its column ----
         float v[8];
@@ -180,6 +182,18 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
             pl[e] = (_Float16)(pe - (float)ph[e]);
         }
 
+        // ---- V: registers -> this wave's LDS slice (K was needed first and arrives first) ----
+        const int rows_left = npos - tile * kTile; // rows of this tile below the position (>= 32: all)
+#pragma unroll
+        for (int i = 0; i < G::kLoads; ++i) {
+            const int c = i * 64 + lane;
+            // rows at or past the position may hold anything; their weights are zero, and 0 * NaN is not
+            const u32x4 x = (c / G::kChunksPerRow) < rows_left ? vreg[i] : u32x4{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4*>(vs + (c / G::kChunksPerRow) * G::kRowBV + (c % G::kChunksPerRow) * 16) = x;
+        }
+        if (more) fetch_v(tile + tile_step);
+        wave_lds_sync();
+
         // ---- O^T += V^T P : rows = head_dim index, columns = query head, k = the tile's 32 KV rows
         //      in the order (grp, t, i) that matches the layout P already has ----
 #pragma unroll
@@ -193,6 +207,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         wave_lds_sync(); // the slice is overwritten at the top of the next iteration
     }
 
+    FA_STAMP(4);
     // ---- merge the waves through LDS ----
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
     float* const obuf = reinterpret_cast<float*>(smem + wave * G::kWaveB);
@@ -204,7 +219,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 #pragma unroll
     for (int db = 0; db < G::kDBlk; ++db)
         *reinterpret_cast<f4*>(obuf + col * G::kOStride + db * 16 + grp * 4) = o[db];
+    FA_STAMP(5);
     __syncthreads();
+    FA_STAMP(6);
 
     for (int idx = threadIdx.x; idx < 16 * (D / 4); idx += kThreads) {
         const int c = idx / (D / 4);
@@ -240,6 +257,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
             *reinterpret_cast<f4*>(a.out + (size_t)head * D + d4) = acc * inv;
         }
     }
+    FA_STAMP(7);
 }
 
 // Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
