@@ -116,6 +116,7 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
     if (rc != ORIN_FA_OK) return rc;
     if (batch < 0 || n_past < 0 || (long long)n_past + batch > n_ctx) return ORIN_FA_E_INVALID;
     if (batch == 0) return ORIN_FA_OK;
+    if ((long long)batch * n_head * head_dim * 4 >= (1ll << 31)) return ORIN_FA_E_INVALID; // 32-bit byte offsets into q
     FaArgs a{};
     a.q = q; a.kc = kc; a.vc = vc; a.out = out;
     a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.n_past = n_past; a.batch = batch;

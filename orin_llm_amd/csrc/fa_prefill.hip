@@ -54,7 +54,9 @@ struct PGeom {
     static constexpr int kScratchOff = 4 * kTileB;    // 1 KB per wave: 16 bytes per lane for accumulator round trips
     static constexpr int kWaveB = (4 * kTileB + 1024 > kMergeB) ? 4 * kTileB + 1024 : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
-    static constexpr int kLdsB = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4;
+    static constexpr int kQOff = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4; // the query block as fp16, [column][head_dim]
+    static constexpr int kQStride = D * 2 + 16;       // (padded: 16 columns read 16 bytes each without bank conflicts)
+    static constexpr int kLdsB = kQOff + NQB * 16 * kQStride;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -168,6 +170,17 @@ __device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int o
         :
         : "s"(lds_base), "v"(off_even), "v"(off_odd), "s"(desc), "s"(soff)
         : "memory", "m0");
+}
+
+// 16 bytes per lane from global memory into vector registers, same addressing.  Counts on the
+// vector-memory counter like the copies; the consumer waits with s_waitcnt vmcnt(n) (the
+// compiler does not know that the registers are filled late).
+template <int IMM>
+__device__ __forceinline__ void reg_load16(u32x4& dst, i32x4 desc, int off, int soff) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4"
+                 : "=&v"(dst)
+                 : "v"(off), "s"(desc), "s"(soff), "n"(IMM)
+                 : "memory");
 }
 
 // One such copy, for the main loop, which deals them out between the matrix instructions so
@@ -288,48 +301,36 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const unsigned scratch_addr = ws_addr + G::kScratchOff + lane * 16;
     float* const scratch = reinterpret_cast<float*>(ws + G::kScratchOff) + lane * 4;
 
-    if (n_mine > 0) {
-        // V buffer 0 receives the diagonal tile, whose rows at or past kv_end are not fetched:
-        // clear it first, so that no stale bit pattern meets a zero weight (0 * NaN is not 0).
-#pragma unroll
-        for (int i = 0; i < G::kCopies; ++i)
-            *reinterpret_cast<u32x4*>(ws + G::kVOff + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
-        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the fill is done before the first copy can land
-        wave_lds_sync();
-        copy_checked(kdesc, k_buf(0), tile_of(0));
-        copy_checked(vdesc, v_buf(0), tile_of(0));
-        copy_checked(kdesc, k_buf(1), tile_of(1));
-        copy_checked(vdesc, v_buf(1), tile_of(1));
-    }
-
-    FA_STAMP(9);
-    // ---- query columns -> B operands ----
-    int limit[NQB];
+    // ---- prologue loads, most urgent first: the query block, then the first K tile; the rest of
+    // the first two tiles follows once the queries are on their way into LDS.  All of them are
+    // issued by hand and counted on the vector-memory counter, so that no wait has to sit out
+    // the loads behind the one it needs.
+    // The query block is loaded once per workgroup: wave w takes a quarter of the columns with
+    // coalesced 16-byte loads (a column is D/4 lanes wide), converts to fp16 and leaves it in LDS;
+    // after the barrier every wave picks up its B operands from there. ----
+    constexpr int kColsPerLoad = 256 / D;              // columns one load instruction covers
+    constexpr int kQLoads = NQB * 4 / kColsPerLoad;    // load instructions per wave
+    u32x4 qraw[kQLoads];
+    float qmul[kQLoads];
+    int qcol[kQLoads];
     {
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
-            const int c = qb * 16 + col;
+        const i32x4 qdesc = make_desc(a.q, (unsigned)batch * a.n_head * D * 4);
+        static_for<0, kQLoads>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int c = wave * (NQB * 4) + j * kColsPerLoad + lane / (D / 4);
             const int tok = t0 + c % TQ;
             const int hl = head_lo + c / TQ;
             const bool valid = (hl < a.r) && (tok < batch);
-            limit[qb] = valid ? n_past + tok + 1 : 0x7fffffff;
-            const float* qp = a.q + ((size_t)(valid ? tok : 0) * a.n_head + (size_t)(valid ? kvh * a.r + hl : 0)) * D;
-            const float qmul = valid ? a.qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
-#pragma unroll
-            for (int kk = 0; kk < G::kSteps; ++kk) {
-                const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
-                const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
-                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                h8 hv;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) hv[e] = (_Float16)(x[e] * qmul);
-                asm volatile("" : "=a"(q[qb][kk]) : "0"(hv)); // parked in the accumulation-register file for good
-            }
-        }
+            qcol[j] = c;
+            qmul[j] = valid ? a.qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
+            const int q_off = valid ? ((tok * a.n_head + kvh * a.r + hl) * D + (lane % (D / 4)) * 4) * 4 : 0;
+            reg_load16<0>(qraw[j], qdesc, q_off, 0);
+        });
     }
-    FA_STAMP(10);
+    if (n_mine > 0) copy_checked(kdesc, k_buf(0), tile_of(0));
+    FA_STAMP(9);
     // O = 0, l = 0: a matrix instruction with a zero addend writes the accumulation registers
-    // without touching memory (0 * Q is 0 for finite Q; a non-finite Q spoils its column anyway).
+    // without touching memory.
     {
         h8 zero;
 #pragma unroll
@@ -340,6 +341,43 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
 #pragma unroll
             for (int db = 0; db < G::kDBlk; ++db) mfma_a_zero_n(o[qb][db], zero, zero);
             mfma_a_zero_n(lacc[qb], zero, zero);
+        }
+    }
+    if (n_mine > 0) {
+        // V buffer 0 receives the diagonal tile, whose rows at or past kv_end are not fetched:
+        // clear it first, so that no stale bit pattern meets a zero weight (0 * NaN is not 0).
+#pragma unroll
+        for (int i = 0; i < G::kCopies; ++i)
+            *reinterpret_cast<u32x4*>(ws + G::kVOff + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    }
+    FA_STAMP(10);
+    // ---- query block -> LDS (fp16) ----
+    if (n_mine > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (G::kCopies & 15) | ((G::kCopies >> 4) << 14)); // vmcnt: the queries are in, K(0) may be in flight
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+    for (int j = 0; j < kQLoads; ++j) {
+        h4 hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] = (_Float16)(__uint_as_float(qraw[j][e]) * qmul[j]);
+        *reinterpret_cast<h4*>(smem + G::kQOff + qcol[j] * G::kQStride + (lane % (D / 4)) * 8) = hv;
+    }
+    __syncthreads(); // (also orders the clearing of V buffer 0 before the copy into it)
+    if (n_mine > 0) {
+        copy_checked(vdesc, v_buf(0), tile_of(0));
+        copy_checked(kdesc, k_buf(1), tile_of(1));
+        copy_checked(vdesc, v_buf(1), tile_of(1));
+    }
+    int limit[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int c = qb * 16 + col;
+        const int tok = t0 + c % TQ;
+        const int hl = head_lo + c / TQ;
+        limit[qb] = (hl < a.r) && (tok < batch) ? n_past + tok + 1 : 0x7fffffff;
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps; ++kk) {
+            const h8 hv = *reinterpret_cast<const h8*>(smem + G::kQOff + c * G::kQStride + (kk * 32 + grp * 8) * 2);
+            asm volatile("" : "=a"(q[qb][kk]) : "0"(hv)); // parked in the accumulation-register file for good
         }
     }
     FA_STAMP(1);
