@@ -50,6 +50,9 @@ WORKLOADS = {
     "qwen1.5b-decode-32k": ("qwen1.5b", "decode", 32768, 32768),
     "llama8b-decode-8k": ("llama8b", "decode", 8192, 8192),
     "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
+    # not part of the path: a plain device copy of known size, the yardstick that the HBM
+    # counters (FETCH_SIZE / WRITE_SIZE) and the achievable streaming rate are scaled by
+    "hbm-copy-256MiB": (None, "copy", 0, 256 << 20),
 }
 ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k"]
 
@@ -91,21 +94,27 @@ def parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, n_past, batch
     return rel_err(got, want)
 
 
-def cpu_baseline_prefill(ref, q, k, v, H, G, d, n_ctx, P, B, scale, budget_s=12.0):
-    """The oracle's reference-order loop (fp32 cache, one thread) on a bounded token sample."""
-    kf = ref.fp16_to_fp32(k)
-    vf = ref.fp16_to_fp32(v)
-    toks = [int(t) for t in np.linspace(0, B - 1, 64).round()]
-    done, flops, t0 = 0, 0.0, time.perf_counter()
-    for t in toks:
-        ref.attention_token_f32(q[t], kf, vf, H, G, d, n_ctx, P + t + 1, np.float32(scale))
-        flops += 4.0 * d * H * (P + t + 1)
-        done += 1
-        if time.perf_counter() - t0 > budget_s:
+def cpu_baseline_prefill(ref, layers_qkv, H, G, d, n_ctx, P, B, scale, budget_s=15.0):
+    """The oracle's reference-order loop (fp32 cache, one thread) on a bounded sample of the same
+    workload: the query tokens of the first layers' chunk, in a fixed shuffled order, until the
+    time budget is used."""
+    done, flops, dt, used = 0, 0.0, 0.0, 0
+    for q, k, v in layers_qkv:
+        kf = ref.fp16_to_fp32(k)  # (the conversion of the cache is not timed: the CPU backend stores fp32)
+        vf = ref.fp16_to_fp32(v)
+        used += 1
+        t0 = time.perf_counter()
+        for t in (int(t) for t in np.random.default_rng(1).permutation(B)):
+            ref.attention_token_f32(q[t], kf, vf, H, G, d, n_ctx, P + t + 1, np.float32(scale))
+            flops += 4.0 * d * H * (P + t + 1)
+            done += 1
+            if dt + time.perf_counter() - t0 > budget_s:
+                break
+        dt += time.perf_counter() - t0
+        if dt > budget_s:
             break
-    dt = time.perf_counter() - t0
     return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=1, kind="port",
-                sample=f"{done} query tokens x {H} heads at depth {P} of layer 0 "
+                sample=f"{done} query tokens x {H} heads at depth {P} from the first {used} layer(s) "
                        f"({flops / 1e9:.2f} GFLOP in {dt:.1f} s), reference loop order, fp32 cache")
 
 
@@ -160,6 +169,18 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
+    # Per-launch duration of the dominant kernel: one event pair around every single launch of
+    # one pass over the stack (the events sit on the stream the kernels are launched on).
+    dom = max(range(len(chunks)), key=lambda ci: prefill_flops(H, d, *chunks[ci]))
+    P, B = chunks[dom]
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in stacks[dom]]
+    for (q, k, v, out), (a0, a1) in zip(stacks[dom], pairs):
+        a0.record()
+        kernels.flash_attention(q, k, v, out, H, G, d, n_ctx, P, B, scale)
+        a1.record()
+    torch.cuda.synchronize()
+    single_us = float(np.median([a0.elapsed_time(a1) for a0, a1 in pairs])) * 1e3
+
     flops_step = sum(prefill_flops(H, d, P, B) for P, B in chunks) * layers
     per_chunk = []
     for ci, (P, B) in enumerate(chunks):
@@ -167,24 +188,27 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
         f = prefill_flops(H, d, P, B)
         per_chunk.append(dict(P=P, B=B, launch_us=ms * 1e3, tflops=f / (ms * 1e-3) / 1e12,
                               frac=f / (ms * 1e-3) / PEAK_FLOPS))
-    dom = max(range(len(chunks)), key=lambda ci: prefill_flops(H, d, *chunks[ci]))
-    P, B = chunks[dom]
     q, k, v, out = stacks[dom][0]
     err = parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, P, B, scale)
     res = dict(
         value=flops_step * steps / wall / 1e12, unit="TFLOP/s", ms_per_step=wall / steps * 1e3,
         config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_ctx=n_ctx,
                     chunks=[list(c) for c in chunks], flops_per_step=flops_step),
-        roofline=dict(bound="mfma", achieved=per_chunk[dom]["tflops"], peak=PEAK_FLOPS / 1e12, unit="TFLOP/s",
-                      frac=per_chunk[dom]["frac"], traffic=None,
-                      kernel=f"fa_fwd_kernel prefill P={P} B={B}", launch_us=per_chunk[dom]["launch_us"],
-                      flops_per_launch=prefill_flops(H, d, P, B)),
+        roofline=dict(bound="mfma", achieved=prefill_flops(H, d, P, B) / (single_us * 1e-6) / 1e12,
+                      peak=PEAK_FLOPS / 1e12, unit="TFLOP/s",
+                      frac=prefill_flops(H, d, P, B) / (single_us * 1e-6) / PEAK_FLOPS, traffic=None,
+                      kernel=f"fa_prefill_kernel<{d}, ...> at P={P} B={B}", launch_us=single_us,
+                      launch_us_back_to_back=per_chunk[dom]["launch_us"],
+                      flops_per_launch=prefill_flops(H, d, P, B),
+                      note="launch_us: median of event pairs around single launches; "
+                           "launch_us_back_to_back: stack average including launch gaps"),
         per_chunk=per_chunk,
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="sampled, layer 0, vs CPU oracle"),
     )
     if with_cpu:
-        res["cpu_baseline"] = cpu_baseline_prefill(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
-                                                   v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, P, B, scale)
+        sample = ((ql.cpu().numpy(), kl.view(torch.uint16).cpu().numpy(), vl.view(torch.uint16).cpu().numpy())
+                  for ql, kl, vl, _ in stacks[dom][:6])
+        res["cpu_baseline"] = cpu_baseline_prefill(ref, sample, H, G, d, n_ctx, P, B, scale)
     return res
 
 
@@ -250,6 +274,15 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     wall_graph = time.perf_counter() - t0
     dev_graph_ms = e0.elapsed_time(e1)
 
+    # Duration of each of the two kernels: events between them, recorded by the library on its stream.
+    split_us, combine_us = [], []
+    for si in range(n_stacks):
+        for q, k, v, out in stacks[si]:
+            a, b = kernels.flash_attention_decode_ind_timed(q, k, v, out, H, G, d, n_ctx, dpos, scale)
+            split_us.append(a)
+            combine_us.append(b)
+    split_us, combine_us = float(np.median(split_us)), float(np.median(combine_us))
+
     q, k, v, out = stacks[(steps - 1) % n_stacks][0]
     rows = np.array([(0, h) for h in range(H)], np.int32)
     want = ref.flash_attention_rows(q.cpu().numpy()[None], k.view(torch.uint16).cpu().numpy(),
@@ -265,8 +298,12 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
                     splits=kernels.decode_splits(H, G, d, n_ctx)),
         roofline=dict(bound="hbm", achieved=bytes_layer / (launch_us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9,
                       unit="GB/s", frac=bytes_layer / (launch_us * 1e-6) / PEAK_BYTES, traffic=None,
-                      kernel="fa_fwd_kernel decode split + fa_decode_combine_kernel (per layer, incl. launch gaps)",
-                      launch_us=launch_us, bytes_per_launch=bytes_layer),
+                      kernel=f"fa_decode_split_kernel<{d}> + fa_decode_combine_kernel<{d}> (one layer)",
+                      launch_us=launch_us, split_kernel_us_events=split_us, combine_kernel_us_events=combine_us,
+                      bytes_per_launch=bytes_layer,
+                      note="launch_us: both kernels of a layer, back to back in the timed loop, launch gaps "
+                           "included (the conservative figure); *_events: median of event pairs around each "
+                           "kernel alone, which include about 2 us of dispatch latency each"),
         eager=dict(ms_per_step=wall_eager / steps * 1e3, device_ms_per_step=dev_eager_ms / steps),
         graph=dict(ms_per_step=wall_graph / steps * 1e3, device_ms_per_step=dev_graph_ms / steps),
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="all heads, layer 0, vs CPU oracle"),
@@ -279,9 +316,34 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     return res
 
 
+def run_copy(torch, kernels, name, steps, warmup, with_cpu):
+    """dst.copy_(src) over rotating buffer pairs larger than the last-level cache."""
+    nbytes = WORKLOADS[name][3]
+    pairs = [(torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(i + 1),
+              torch.empty(nbytes, dtype=torch.uint8, device="cuda")) for i in range(3)]
+    for i in range(warmup):
+        pairs[i % 3][1].copy_(pairs[i % 3][0])
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        pairs[i % 3][1].copy_(pairs[i % 3][0])
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = e0.elapsed_time(e1) * 1e3 / steps
+    return dict(value=2.0 * nbytes * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+                config=dict(workload=name, bytes_read_per_step=nbytes, bytes_written_per_step=nbytes),
+                roofline=dict(bound="hbm", achieved=2.0 * nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=2.0 * nbytes / (us * 1e-6) / PEAK_BYTES, traffic=2.0 * nbytes,
+                              kernel="torch copy kernel (read + write)", launch_us=us),
+                parity=None)
+
+
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = run_prefill if kind == "prefill" else run_decode
+    fn = {"prefill": run_prefill, "decode": run_decode, "copy": run_copy}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
 

@@ -74,6 +74,14 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
 
+/* Measurement aid with no counterpart in the reference: orin_fa_decode_ind with HIP events
+ * recorded before, between and after its two kernels on the library's stream.  Synchronises
+ * on the last event and returns the elapsed time of the split kernel and of the combine
+ * kernel in microseconds (the latter 0 when the shape needs no split).  Not capture-safe. */
+int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                             int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
+                             float* us_split, float* us_combine);
+
 /* Introspection for tests and benchmarks: the number of KV splits a decode launch
  * with these shapes uses (0 if the shape is rejected), and the CU count seen at init. */
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx);

@@ -126,8 +126,40 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
     return hip_code(prefill_launch(a, head_dim, g_state.cu_count, g_state.stream));
 }
 
+namespace {
+int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
+                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid);
+}
+
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr);
+}
+
+int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                             int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
+                             float* us_split, float* us_combine) {
+    static hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+    hipError_t e = hipSuccess;
+    for (int i = 0; i < 3 && e == hipSuccess; ++i)
+        if (!ev[i]) e = hipEventCreate(&ev[i]);
+    if (e != hipSuccess) return hip_code(e);
+    if ((e = hipEventRecord(ev[0], g_state.stream)) != hipSuccess) return hip_code(e);
+    const int rc = decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, ev[1]);
+    if (rc != ORIN_FA_OK) return rc;
+    if ((e = hipEventRecord(ev[2], g_state.stream)) != hipSuccess) return hip_code(e);
+    if ((e = hipEventSynchronize(ev[2])) != hipSuccess) return hip_code(e);
+    float ms_split = 0.0f, ms_combine = 0.0f;
+    if ((e = hipEventElapsedTime(&ms_split, ev[0], ev[1])) != hipSuccess) return hip_code(e);
+    if ((e = hipEventElapsedTime(&ms_combine, ev[1], ev[2])) != hipSuccess) return hip_code(e);
+    if (us_split) *us_split = ms_split * 1e3f;
+    if (us_combine) *us_combine = ms_combine * 1e3f;
+    return ORIN_FA_OK;
+}
+
+namespace {
+int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
+                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid) {
     int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
     if (rc != ORIN_FA_OK) return rc;
     if (!d_pos) return ORIN_FA_E_INVALID;
@@ -143,8 +175,9 @@ int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, f
         a.part_ml = a.part_o + (size_t)a.n_splits * n_head * head_dim;
     }
     set_scale(a, scale);
-    return hip_code(decode_launch(a, head_dim, g_state.stream));
+    return hip_code(decode_launch(a, head_dim, g_state.stream, mid));
 }
+} // namespace
 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return 0;

@@ -50,7 +50,8 @@ struct FaArgs {
 // Launchers (defined next to their kernels).  All return hipError_t of the launch.
 hipError_t prefill_launch(const FaArgs& args, int head_dim, int cu_count, hipStream_t stream);
 hipError_t prefill_allow_lds();
-hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream);
+// mid, when not null, is recorded between the split kernel and the combine kernel (timing only).
+hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream, hipEvent_t mid = nullptr);
 hipError_t decode_allow_lds();
 
 template <int N>

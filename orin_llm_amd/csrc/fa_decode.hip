@@ -340,11 +340,12 @@ __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) 
 }
 
 template <int D>
-hipError_t launch(const FaArgs& a, hipStream_t stream) {
+hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     const int grid = a.n_kv * a.n_hgroups * a.n_splits;
     constexpr int lds = DGeom<D>::kLdsB;
     hipLaunchKernelGGL(fa_decode_split_kernel<D>, dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
     hipError_t e = hipGetLastError();
+    if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
     hipLaunchKernelGGL(fa_decode_combine_kernel<D>, dim3(a.n_head * (D / 32)), dim3(256), 0, stream, a);
     return hipGetLastError();
@@ -352,8 +353,8 @@ hipError_t launch(const FaArgs& a, hipStream_t stream) {
 
 } // namespace
 
-hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream) {
-    return head_dim == 128 ? launch<128>(a, stream) : launch<64>(a, stream);
+hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream, hipEvent_t mid) {
+    return head_dim == 128 ? launch<128>(a, stream, mid) : launch<64>(a, stream, mid);
 }
 
 // The split kernel uses more than 64 KB of dynamic LDS; the opt-in is set once at init so

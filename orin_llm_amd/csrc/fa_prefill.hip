@@ -651,15 +651,13 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
-        lds_store_acc(scratch_addr, lacc[qb]);
-        const float l_tot = scratch[0];
+        asm volatile("" : "+a"(lacc[qb])); // pins the read below behind the settled pipe
+        const float l_tot = lacc[qb][0];
         if (grp == 0) {
             ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = l_tot > 0.0f ? -nb[qb] : -INFINITY;
             ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 1] = l_tot;
         }
     }
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    wave_lds_sync(); // the scratch lies inside the merge buffer when the tile is small
     const unsigned obuf_addr = ws_addr + (col * G::kOStride + grp * 4) * 4;
     static_for<0, NQB>([&](auto qbc) {
         static_for<0, G::kDBlk>([&](auto dbc) {

@@ -43,6 +43,9 @@ def lib():
         L.orin_fa_prefill.restype = _int
         L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_decode_ind_timed.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
+                                               ctypes.POINTER(_flt), ctypes.POINTER(_flt)]
+        L.orin_fa_decode_ind_timed.restype = _int
         L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
         L.orin_fa_decode_splits.restype = _int
         L.orin_fa_cu_count.argtypes = []
@@ -99,6 +102,17 @@ def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_
                                   _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def flash_attention_decode_ind_timed(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):
+    """Measurement aid: the same launch with HIP events around its two kernels; synchronises and
+    returns (microseconds of the split kernel, microseconds of the combine kernel)."""
+    us_split, us_combine = _flt(0.0), _flt(0.0)
+    rc = lib().orin_fa_decode_ind_timed(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), n_head, n_kv, head_dim, n_ctx,
+                                        _ptr(d_pos), scale, ctypes.byref(us_split), ctypes.byref(us_combine))
+    if rc != 0:
+        raise OrinFaError("flash_attention_decode_ind_timed", rc)
+    return us_split.value, us_combine.value
 
 
 def decode_splits(n_head, n_kv, head_dim, n_ctx):
