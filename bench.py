@@ -54,6 +54,14 @@ WORKLOADS = {
     # counters (FETCH_SIZE / WRITE_SIZE) and the achievable streaming rate are scaled by
     "hbm-copy-256MiB": (None, "copy", 0, 256 << 20),
 }
+# HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
+# WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy.  These are
+# recorded measurements (a counter pass cannot run inside the timed benchmark); None where not taken.
+TRAFFIC = {
+    "llama8b-prefill512-d4096": 27.60e6 + 8.39e6,
+    "qwen1.5b-decode-32k": 33.68e6 + 0.80e6 + 0.97e6 + 0.006e6,
+    "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
+}
 ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k"]
 
 
@@ -196,7 +204,7 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
                     chunks=[list(c) for c in chunks], flops_per_step=flops_step),
         roofline=dict(bound="mfma", achieved=prefill_flops(H, d, P, B) / (single_us * 1e-6) / 1e12,
                       peak=PEAK_FLOPS / 1e12, unit="TFLOP/s",
-                      frac=prefill_flops(H, d, P, B) / (single_us * 1e-6) / PEAK_FLOPS, traffic=None,
+                      frac=prefill_flops(H, d, P, B) / (single_us * 1e-6) / PEAK_FLOPS, traffic=TRAFFIC.get(name),
                       kernel=f"fa_prefill_kernel<{d}, ...> at P={P} B={B}", launch_us=single_us,
                       launch_us_back_to_back=per_chunk[dom]["launch_us"],
                       flops_per_launch=prefill_flops(H, d, P, B),
@@ -297,7 +305,7 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
                     bytes_per_step=bytes_layer * layers, stacks_rotated=n_stacks,
                     splits=kernels.decode_splits(H, G, d, n_ctx)),
         roofline=dict(bound="hbm", achieved=bytes_layer / (launch_us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9,
-                      unit="GB/s", frac=bytes_layer / (launch_us * 1e-6) / PEAK_BYTES, traffic=None,
+                      unit="GB/s", frac=bytes_layer / (launch_us * 1e-6) / PEAK_BYTES, traffic=TRAFFIC.get(name),
                       kernel=f"fa_decode_split_kernel<{d}> + fa_decode_combine_kernel<{d}> (one layer)",
                       launch_us=launch_us, split_kernel_us_events=split_us, combine_kernel_us_events=combine_us,
                       bytes_per_launch=bytes_layer,
