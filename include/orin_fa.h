@@ -74,6 +74,26 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
 
+/* Replaces llm::cuda::kv_store_batch (reference: src/kernels.h:66-67, src/kernels.cu:1659-1678,
+ * 2079-2083; CPU statement src/model_cpu.cpp:276-279): rounds the fp32 K and V rows of `batch`
+ * tokens (k, v: [batch][heads][head_dim]) to binary16, nearest-even, into cache positions
+ * [pos_base, pos_base + batch) of one layer's caches.  This is the step that runs right before
+ * orin_fa_prefill at the call site (src/model_gpu.cu:378-384).  Any head_dim is accepted. */
+int orin_fa_kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                           int heads, int head_dim, int n_ctx, int pos_base, int batch);
+
+/* Replaces llm::cuda::kv_store_ind (reference: src/kernels.h:69-70, src/kernels.cu:2085-2088):
+ * the same for one token whose position is read from device memory (capture-safe; call site
+ * src/model_gpu.cu:276-282).  A position outside [0, n_ctx) stores nothing. */
+int orin_fa_kv_store_ind(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                         int heads, int head_dim, int n_ctx, const int* d_pos);
+
+/* Replaces llm::cuda::kv_shift (reference: src/kernels.h:72-73, src/kernels.cu:1682-1700, 2090-2093;
+ * CPU statement src/model_cpu.cpp:321-338; policy src/engine.cpp:231-235): over the WHOLE cache
+ * (kc, vc: [n_layer][n_kv][n_ctx][head_dim] each), per layer and head, rows [n_keep + shift, n_ctx)
+ * move to [n_keep, n_ctx - shift) and the last `shift` rows are cleared, in place. */
+int orin_fa_kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep, int shift);
+
 /* Measurement aid with no counterpart in the reference: orin_fa_decode_ind with HIP events
  * recorded before, between and after its two kernels on the library's stream.  Synchronises
  * on the last event and returns the elapsed time of the split kernel and of the combine

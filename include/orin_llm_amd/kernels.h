@@ -1,5 +1,5 @@
-// The attention slice of the orin_llm operator API, with the reference's own
-// signatures (reference: src/kernels.h:8-10 and :77-81), implemented for MI355X by
+// The attention and KV-cache slice of the orin_llm operator API, with the reference's own
+// signatures (reference: src/kernels.h:8-10, :66-73 and :77-81), implemented for MI355X by
 // liborin_fa.so.  An engine built against the reference header links these symbols
 // unchanged; each forwards to the C ABI in include/orin_fa.h and, like the
 // reference's CUDA_CHECK (src/common.h:14-22), prints and abort()s on failure.
@@ -20,6 +20,14 @@ namespace llm::cuda {
 int init();
 void set_stream(void* stream);
 #endif
+
+void kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                    int heads, int head_dim, int n_ctx, int pos_base, int batch);
+
+void kv_store_ind(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                  int heads, int head_dim, int n_ctx, const int* d_pos);
+
+void kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep, int shift);
 
 void flash_attention(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                     int n_head, int n_kv, int head_dim, int n_ctx, int n_past, int batch, float scale);

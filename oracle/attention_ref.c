@@ -11,6 +11,7 @@
  *   orc_attention_token_f16, _row_f16     bit-equal to _f32 on fp16-representable caches + float64 closed form
  *   orc_flash_attention*, _rows           composition of the above, checked against the same fixtures
  *   orc_kv_store_*                        exact against numpy astype(float16) at the documented offset
+ *   orc_kv_shift_u16                      exact against the slice statement new[keep:n-s] = old[keep+s:], tail 0
  */
 #include "attention_ref.h"
 
@@ -107,6 +108,25 @@ void orc_kv_store_f16(uint16_t* kc, uint16_t* vc, const float* k, const float* v
             const size_t src = ((size_t)b * n_kv + h) * head_dim;
             orc_fp32_to_fp16_n(k + src, kc + dst, (size_t)head_dim);
             orc_fp32_to_fp16_n(v + src, vc + dst, (size_t)head_dim);
+        }
+}
+
+/* Rolling-window shift of the whole cache (reference: src/model_cpu.cpp:321-338, which
+ * states it on the CPU backend's fp32 cache; the device cache holds 16-bit elements,
+ * src/kernels.cu:1682-1700): per layer and head, rows [n_keep + shift, n_ctx) move to
+ * [n_keep, n_ctx - shift) and the last `shift` rows are cleared. */
+void orc_kv_shift_u16(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx,
+                      int n_keep, int shift) {
+    const size_t d = (size_t)head_dim;
+    const size_t per_layer = (size_t)n_kv * n_ctx * d;
+    for (int l = 0; l < n_layer; ++l)
+        for (int h = 0; h < n_kv; ++h) {
+            uint16_t* kh = kc + l * per_layer + (size_t)h * n_ctx * d;
+            uint16_t* vh = vc + l * per_layer + (size_t)h * n_ctx * d;
+            memmove(kh + n_keep * d, kh + (n_keep + shift) * d, (size_t)(n_ctx - n_keep - shift) * d * sizeof(uint16_t));
+            memmove(vh + n_keep * d, vh + (n_keep + shift) * d, (size_t)(n_ctx - n_keep - shift) * d * sizeof(uint16_t));
+            memset(kh + (size_t)(n_ctx - shift) * d, 0, (size_t)shift * d * sizeof(uint16_t));
+            memset(vh + (size_t)(n_ctx - shift) * d, 0, (size_t)shift * d * sizeof(uint16_t));
         }
 }
 

@@ -41,6 +41,11 @@ void orc_kv_store_f32(float* kc, float* vc, const float* k, const float* v,
 void orc_kv_store_f16(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
                       int n_kv, int head_dim, int n_ctx, int pos_base, int batch);
 
+/* Rolling-window shift (reference: src/model_cpu.cpp:321-338, src/kernels.cu:1682-1700).
+ * kc, vc: the whole cache, [n_layer][n_kv][n_ctx][head_dim] 16-bit elements each. */
+void orc_kv_shift_u16(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx,
+                      int n_keep, int shift);
+
 /* One query token against the first npos cache positions
  * (reference: src/model_cpu.cpp:281-295, softmax :20-30, dot :32-36).
  * q, out: [n_head][head_dim].  score: caller scratch of >= npos floats.

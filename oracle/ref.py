@@ -32,6 +32,7 @@ def _load():
     lib.orc_fp32_to_fp16_n.argtypes = [_f32p, _u16p, ctypes.c_size_t]
     lib.orc_kv_store_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int]
     lib.orc_kv_store_f16.argtypes = [_u16p, _u16p, _f32p, _f32p, _int, _int, _int, _int, _int]
+    lib.orc_kv_shift_u16.argtypes = [_u16p, _u16p, _int, _int, _int, _int, _int, _int]
     lib.orc_attention_token_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
     lib.orc_attention_token_f16.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
     lib.orc_attention_row_f16.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _flt, _f32p]
@@ -85,6 +86,14 @@ def kv_store_f16(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch):
     k, v = _c(k, np.float32), _c(v, np.float32)
     assert kc.dtype == np.uint16 and kc.flags.c_contiguous and kc.size == n_kv * n_ctx * d
     lib().orc_kv_store_f16(_p(kc, _u16p), _p(vc, _u16p), _p(k, _f32p), _p(v, _f32p), n_kv, d, n_ctx, pos_base, batch)
+
+
+def kv_shift_u16(kc, vc, n_layer, n_kv, d, n_ctx, n_keep, shift):
+    """kc, vc: uint16 arrays [n_layer][n_kv][n_ctx][d], modified in place."""
+    assert kc.dtype == np.uint16 and kc.flags.c_contiguous and kc.size == n_layer * n_kv * n_ctx * d
+    assert vc.dtype == np.uint16 and vc.flags.c_contiguous and vc.size == kc.size
+    assert 0 <= n_keep and 0 <= shift and n_keep + shift <= n_ctx
+    lib().orc_kv_shift_u16(_p(kc, _u16p), _p(vc, _u16p), n_layer, n_kv, d, n_ctx, n_keep, shift)
 
 
 def kv_store_f32(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch):

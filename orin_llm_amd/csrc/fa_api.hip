@@ -2,7 +2,8 @@
 // C ABI declared in include/orin_fa.h.  The kernels live in fa_prefill.hip and fa_decode.hip.
 //
 // Boundary: the reference's llm::cuda::flash_attention and flash_attention_decode_ind
-// (reference: src/kernels.h:97-109, launchers at src/kernels.cu:1944-2000).
+// (reference: src/kernels.h:77-81, launchers at src/kernels.cu:1944-2000) and its KV-cache
+// mutators kv_store_batch / kv_store_ind / kv_shift (src/kernels.h:66-73, src/kernels.cu:2079-2093).
 #include "fa_common.hpp"
 
 #include <stdio.h>
@@ -178,6 +179,33 @@ int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* o
     return hip_code(decode_launch(a, head_dim, g_state.stream, mid));
 }
 } // namespace
+
+int orin_fa_kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                           int heads, int head_dim, int n_ctx, int pos_base, int batch) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!kc || !vc || !k || !v) return ORIN_FA_E_INVALID;
+    if (heads <= 0 || head_dim <= 0 || n_ctx <= 0 || batch < 0 || pos_base < 0) return ORIN_FA_E_INVALID;
+    if ((long long)pos_base + batch > n_ctx) return ORIN_FA_E_INVALID;
+    if (batch == 0) return ORIN_FA_OK;
+    return hip_code(kv_store_launch(kc, vc, k, v, heads, head_dim, n_ctx, pos_base, batch, nullptr, g_state.stream));
+}
+
+int orin_fa_kv_store_ind(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                         int heads, int head_dim, int n_ctx, const int* d_pos) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!kc || !vc || !k || !v || !d_pos) return ORIN_FA_E_INVALID;
+    if (heads <= 0 || head_dim <= 0 || n_ctx <= 0) return ORIN_FA_E_INVALID;
+    return hip_code(kv_store_launch(kc, vc, k, v, heads, head_dim, n_ctx, 0, 1, d_pos, g_state.stream));
+}
+
+int orin_fa_kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep, int shift) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!kc || !vc) return ORIN_FA_E_INVALID;
+    if (n_layer <= 0 || n_kv <= 0 || head_dim <= 0 || n_ctx <= 0) return ORIN_FA_E_INVALID;
+    if (n_keep < 0 || shift < 0 || (long long)n_keep + shift > n_ctx) return ORIN_FA_E_INVALID;
+    if (shift == 0) return ORIN_FA_OK;
+    return hip_code(kv_shift_launch(kc, vc, n_layer, n_kv, head_dim, n_ctx, n_keep, shift, g_state.stream));
+}
 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return 0;

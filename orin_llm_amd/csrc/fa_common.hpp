@@ -54,6 +54,13 @@ hipError_t prefill_allow_lds();
 hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream, hipEvent_t mid = nullptr);
 hipError_t decode_allow_lds();
 
+// KV-cache mutators (kv_cache.hip).  d_pos not null selects the single-token form that reads
+// the position on the device.
+hipError_t kv_store_launch(uint16_t* kc, uint16_t* vc, const float* k, const float* v, int heads, int head_dim,
+                           int n_ctx, int pos_base, int batch, const int* d_pos, hipStream_t stream);
+hipError_t kv_shift_launch(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep,
+                           int shift, hipStream_t stream);
+
 template <int N>
 struct IntC {
     static constexpr int value = N;

@@ -1,5 +1,5 @@
 // llm::cuda::* entry points with the reference's signatures (reference:
-// src/kernels.h:8-10,77-81; definitions src/kernels.cu:1728-1737,1974-2000),
+// src/kernels.h:8-10,66-73,77-81; definitions src/kernels.cu:1728-1737,1974-2000,2079-2093),
 // forwarding to the C ABI.  Plain C++: no HIP headers, no device code.
 #include "../../include/orin_llm_amd/kernels.h"
 
@@ -33,6 +33,23 @@ int init() {
 
 void set_stream(void* stream) { orin_fa_set_stream(stream); }
 #endif
+
+void kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                    int heads, int head_dim, int n_ctx, int pos_base, int batch) {
+    const int rc = orin_fa_kv_store_batch(kc, vc, k, v, heads, head_dim, n_ctx, pos_base, batch);
+    if (rc != ORIN_FA_OK) die("kv_store_batch", rc);
+}
+
+void kv_store_ind(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
+                  int heads, int head_dim, int n_ctx, const int* d_pos) {
+    const int rc = orin_fa_kv_store_ind(kc, vc, k, v, heads, head_dim, n_ctx, d_pos);
+    if (rc != ORIN_FA_OK) die("kv_store_ind", rc);
+}
+
+void kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep, int shift) {
+    const int rc = orin_fa_kv_shift(kc, vc, n_layer, n_kv, head_dim, n_ctx, n_keep, shift);
+    if (rc != ORIN_FA_OK) die("kv_shift", rc);
+}
 
 void flash_attention(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                      int n_head, int n_kv, int head_dim, int n_ctx, int n_past, int batch, float scale) {

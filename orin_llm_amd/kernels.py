@@ -43,6 +43,12 @@ def lib():
         L.orin_fa_prefill.restype = _int
         L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_kv_store_batch.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int]
+        L.orin_fa_kv_store_batch.restype = _int
+        L.orin_fa_kv_store_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]
+        L.orin_fa_kv_store_ind.restype = _int
+        L.orin_fa_kv_shift.argtypes = [_vp, _vp, _int, _int, _int, _int, _int, _int]
+        L.orin_fa_kv_shift.restype = _int
         L.orin_fa_decode_ind_timed.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
                                                ctypes.POINTER(_flt), ctypes.POINTER(_flt)]
         L.orin_fa_decode_ind_timed.restype = _int
@@ -102,6 +108,24 @@ def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_
                                   _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def kv_store_batch(kc, vc, k, v, heads, head_dim, n_ctx, pos_base, batch):
+    rc = lib().orin_fa_kv_store_batch(_ptr(kc), _ptr(vc), _ptr(k), _ptr(v), heads, head_dim, n_ctx, pos_base, batch)
+    if rc != 0:
+        raise OrinFaError("kv_store_batch", rc)
+
+
+def kv_store_ind(kc, vc, k, v, heads, head_dim, n_ctx, d_pos):
+    rc = lib().orin_fa_kv_store_ind(_ptr(kc), _ptr(vc), _ptr(k), _ptr(v), heads, head_dim, n_ctx, _ptr(d_pos))
+    if rc != 0:
+        raise OrinFaError("kv_store_ind", rc)
+
+
+def kv_shift(kc, vc, n_layer, n_kv, head_dim, n_ctx, n_keep, shift):
+    rc = lib().orin_fa_kv_shift(_ptr(kc), _ptr(vc), n_layer, n_kv, head_dim, n_ctx, n_keep, shift)
+    if rc != 0:
+        raise OrinFaError("kv_shift", rc)
 
 
 def flash_attention_decode_ind_timed(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):

@@ -1,0 +1,186 @@
+"""KV-cache mutators: the oracle pinned on the CPU, the HIP path bit-exact against it on the GPU
+(reference: src/kernels.cu:1659-1700, 2079-2093; src/model_cpu.cpp:276-279, 321-338)."""
+import numpy as np
+import pytest
+
+from oracle import ref
+
+
+def _cache(rng, n_layer, n_kv, n_ctx, d):
+    return (rng.integers(1, 65535, size=(n_layer, n_kv, n_ctx, d), dtype=np.uint16),
+            rng.integers(1, 65535, size=(n_layer, n_kv, n_ctx, d), dtype=np.uint16))
+
+
+SHIFT_CASES = [  # n_layer, n_kv, d, n_ctx, n_keep, shift
+    (2, 2, 128, 64, 4, 30),      # the engine's policy: half of what lies past n_keep
+    (1, 3, 128, 97, 0, 1),       # one row, long chains
+    (2, 1, 64, 50, 7, 43),       # shift == n_ctx - n_keep: everything past n_keep is cleared
+    (1, 2, 128, 40, 40, 0),      # nothing to do
+    (1, 2, 128, 33, 5, 5),
+    (3, 2, 72, 31, 3, 9),        # 144-byte rows
+    (1, 1, 20, 17, 2, 6),        # rows that are no multiple of 16 bytes
+]
+
+
+@pytest.mark.parametrize("case", SHIFT_CASES)
+def test_oracle_kv_shift_is_the_slice_statement(case):
+    n_layer, n_kv, d, n_ctx, n_keep, shift = case
+    rng = np.random.default_rng(5)
+    kc, vc = _cache(rng, n_layer, n_kv, n_ctx, d)
+    k2, v2 = kc.copy(), vc.copy()
+    ref.kv_shift_u16(k2, v2, n_layer, n_kv, d, n_ctx, n_keep, shift)
+    for new, old in ((k2, kc), (v2, vc)):
+        want = old.copy()
+        want[:, :, n_keep:n_ctx - shift] = old[:, :, n_keep + shift:]
+        want[:, :, n_ctx - shift:] = 0
+        assert np.array_equal(new, want)
+
+
+def test_oracle_kv_store_matches_numpy_float16():
+    rng = np.random.default_rng(6)
+    n_kv, d, n_ctx, pos_base, batch = 3, 128, 40, 11, 7
+    k = rng.standard_normal((batch, n_kv, d)).astype(np.float32) * np.float32(100.0)
+    v = rng.standard_normal((batch, n_kv, d)).astype(np.float32) * np.float32(1e-6)  # subnormal halves
+    k[0, 0, :6] = [65504.0, 65519.99, 65520.0, 1e9, -np.inf, 2.0 ** -25]
+    kc = np.full((n_kv, n_ctx, d), 0x1234, np.uint16)
+    vc = np.full((n_kv, n_ctx, d), 0x4321, np.uint16)
+    ref.kv_store_f16(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch)
+    with np.errstate(over="ignore"):
+        wk = k.astype(np.float16).view(np.uint16).transpose(1, 0, 2)
+        wv = v.astype(np.float16).view(np.uint16).transpose(1, 0, 2)
+    assert np.array_equal(kc[:, pos_base:pos_base + batch], wk)
+    assert np.array_equal(vc[:, pos_base:pos_base + batch], wv)
+    assert (kc[:, :pos_base] == 0x1234).all() and (kc[:, pos_base + batch:] == 0x1234).all()
+    assert (vc[:, :pos_base] == 0x4321).all() and (vc[:, pos_base + batch:] == 0x4321).all()
+
+
+# ---------------------------------------------------------------------------------------- GPU
+
+@pytest.fixture(scope="module")
+def fa():
+    import torch
+    from orin_llm_amd import kernels
+    assert torch.cuda.is_available()
+    kernels.init(0)
+    kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+    return kernels
+
+
+def _dev_u16(torch, a):
+    return torch.from_numpy(a.view(np.int16).copy()).cuda()
+
+
+def _host_u16(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_kv,d,n_ctx,pos_base,batch", [
+    (2, 128, 4096, 0, 512), (8, 128, 600, 88, 512), (4, 128, 300, 299, 1), (2, 64, 100, 3, 45),
+    (3, 72, 50, 1, 9), (1, 20, 17, 5, 12)])
+def test_kv_store_batch_bit_exact(fa, n_kv, d, n_ctx, pos_base, batch):
+    import torch
+    rng = np.random.default_rng(batch + d)
+    k = (rng.standard_normal((batch, n_kv, d)) * 30).astype(np.float32)
+    v = (rng.standard_normal((batch, n_kv, d)) * 3e-6).astype(np.float32)   # many subnormal halves
+    k.reshape(-1)[:8] = [65504.0, 65519.99, 65520.0, 1e9, -np.inf, 2.0 ** -25, -0.0, 6.1e-5]
+    kc0, vc0 = _cache(rng, 1, n_kv, n_ctx, d)
+    kc0, vc0 = kc0[0], vc0[0]
+    wk, wv = kc0.copy(), vc0.copy()
+    ref.kv_store_f16(wk, wv, k, v, n_kv, d, n_ctx, pos_base, batch)
+    dk, dv = _dev_u16(torch, kc0), _dev_u16(torch, vc0)
+    fa.kv_store_batch(dk, dv, torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), n_kv, d, n_ctx, pos_base, batch)
+    torch.cuda.synchronize()
+    assert np.array_equal(_host_u16(dk), wk)   # rows outside [pos_base, pos_base + batch) untouched as well
+    assert np.array_equal(_host_u16(dv), wv)
+
+
+@pytest.mark.gpu
+def test_kv_store_ind_reads_the_position_on_the_device_and_replays(fa):
+    import torch
+    n_kv, d, n_ctx = 4, 128, 256
+    rng = np.random.default_rng(9)
+    kc0, vc0 = _cache(rng, 1, n_kv, n_ctx, d)
+    dk, dv = _dev_u16(torch, kc0[0]), _dev_u16(torch, vc0[0])
+    wk, wv = kc0[0].copy(), vc0[0].copy()
+    k = torch.zeros((n_kv, d), device="cuda")
+    v = torch.zeros((n_kv, d), device="cuda")
+    dpos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            fa.set_stream(torch.cuda.current_stream().cuda_stream)
+            fa.kv_store_ind(dk, dv, k, v, n_kv, d, n_ctx, dpos)
+    finally:
+        fa.set_stream(torch.cuda.current_stream().cuda_stream)
+    for pos in (0, 17, 255, 256, -1):     # the last two are out of range: nothing may be written
+        hk = rng.standard_normal((1, n_kv, d)).astype(np.float32)
+        hv = rng.standard_normal((1, n_kv, d)).astype(np.float32)
+        k.copy_(torch.from_numpy(hk[0]))
+        v.copy_(torch.from_numpy(hv[0]))
+        dpos.fill_(pos)
+        g.replay()
+        torch.cuda.synchronize()
+        if 0 <= pos < n_ctx:
+            ref.kv_store_f16(wk, wv, hk, hv, n_kv, d, n_ctx, pos, 1)
+        assert np.array_equal(_host_u16(dk), wk), pos
+        assert np.array_equal(_host_u16(dv), wv), pos
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", SHIFT_CASES + [(4, 2, 128, 4096, 16, 2040), (2, 8, 128, 1024, 0, 512)])
+def test_kv_shift_bit_exact(fa, case):
+    import torch
+    n_layer, n_kv, d, n_ctx, n_keep, shift = case
+    rng = np.random.default_rng(n_ctx + shift)
+    kc, vc = _cache(rng, n_layer, n_kv, n_ctx, d)
+    dk, dv = _dev_u16(torch, kc), _dev_u16(torch, vc)
+    ref.kv_shift_u16(kc, vc, n_layer, n_kv, d, n_ctx, n_keep, shift)
+    fa.kv_shift(dk, dv, n_layer, n_kv, d, n_ctx, n_keep, shift)
+    torch.cuda.synchronize()
+    assert np.array_equal(_host_u16(dk), kc)
+    assert np.array_equal(_host_u16(dv), vc)
+
+
+@pytest.mark.gpu
+def test_store_then_attend_equals_attending_a_prebuilt_cache(fa):
+    """The call-site order (reference: src/model_gpu.cu:378-384): append the chunk's K/V, then attend."""
+    import torch
+    H, G, d, n_ctx, n_past, batch = 12, 2, 128, 512, 100, 77
+    scale = float(1.0 / np.sqrt(d))
+    rng = np.random.default_rng(3)
+    k_all = rng.standard_normal((n_past + batch, G, d)).astype(np.float32)
+    v_all = rng.standard_normal((n_past + batch, G, d)).astype(np.float32)
+    q = rng.standard_normal((batch, H, d)).astype(np.float32)
+    kc = np.zeros((G, n_ctx, d), np.uint16)
+    vc = np.zeros((G, n_ctx, d), np.uint16)
+    ref.kv_store_f16(kc, vc, k_all, v_all, G, d, n_ctx, 0, n_past + batch)
+    want = ref.flash_attention(q, kc, vc, H, G, d, n_ctx, n_past, batch, np.float32(scale))
+    dk = torch.full((G, n_ctx, d), 0x7e00, dtype=torch.int16, device="cuda")   # NaN everywhere
+    dv = torch.full((G, n_ctx, d), 0x7e00, dtype=torch.int16, device="cuda")
+    fa.kv_store_batch(dk, dv, torch.from_numpy(k_all[:n_past]).cuda(), torch.from_numpy(v_all[:n_past]).cuda(),
+                      G, d, n_ctx, 0, n_past)
+    fa.kv_store_batch(dk, dv, torch.from_numpy(k_all[n_past:]).cuda(), torch.from_numpy(v_all[n_past:]).cuda(),
+                      G, d, n_ctx, n_past, batch)
+    out = torch.empty((batch, H, d), device="cuda")
+    fa.flash_attention(torch.from_numpy(q).cuda(), dk, dv, out, H, G, d, n_ctx, n_past, batch, scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    err = np.max(np.abs(got - want).max(axis=2) / np.abs(want).max(axis=2))
+    assert np.isfinite(got).all() and err < 2e-3, err
+
+
+@pytest.mark.gpu
+def test_kv_mutators_reject_bad_arguments(fa):
+    import torch
+    from orin_llm_amd.kernels import OrinFaError
+    t16 = torch.zeros(2 * 64 * 128, dtype=torch.int16, device="cuda")
+    t32 = torch.zeros(8 * 2 * 128, device="cuda")
+    with pytest.raises(OrinFaError):
+        fa.kv_store_batch(t16, t16, t32, t32, 2, 128, 64, 60, 8)      # runs past n_ctx
+    with pytest.raises(OrinFaError):
+        fa.kv_store_batch(t16, t16, t32, t32, 2, 128, 64, -1, 8)
+    with pytest.raises(OrinFaError):
+        fa.kv_shift(t16, t16, 1, 2, 128, 64, 40, 30)                  # n_keep + shift > n_ctx
+    with pytest.raises(OrinFaError):
+        fa.kv_store_ind(t16, t16, t32, t32, 2, 128, 64, None)
