@@ -50,6 +50,9 @@ WORKLOADS = {
     "qwen1.5b-decode-32k": ("qwen1.5b", "decode", 32768, 32768),
     "llama8b-decode-8k": ("llama8b", "decode", 8192, 8192),
     "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
+    # the two mutators of the cache (byte movers; value = bytes read + written per second)
+    "llama8b-kv-store-512": ("llama8b", "kv_store", 8192, (4096, 512)),
+    "qwen1.5b-kv-shift-32k": ("qwen1.5b", "kv_shift", 32768, (4, 16382)),
     # not part of the path: a plain device copy of known size, the yardstick that the HBM
     # counters (FETCH_SIZE / WRITE_SIZE) and the achievable streaming rate are scaled by
     "hbm-copy-256MiB": (None, "copy", 0, 256 << 20),
@@ -62,7 +65,8 @@ TRAFFIC = {
     "qwen1.5b-decode-32k": 33.68e6 + 0.80e6 + 0.97e6 + 0.006e6,
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
-ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k"]
+ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k",
+        "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
 
 
 def prefill_flops(H, d, P, B):
@@ -324,6 +328,91 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     return res
 
 
+def run_kv_store(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = kv_store_batch of a 512-token chunk into every layer's cache (fp32 in, fp16 out)."""
+    from oracle import ref
+    shape_name, _, n_ctx, (P, B) = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    G, d, layers = s["G"], s["d"], s["layers"]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(77)
+    stack = [(torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda"),
+              torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda"),
+              torch.randn((B, G, d), generator=g, device="cuda"), torch.randn((B, G, d), generator=g, device="cuda"))
+             for _ in range(layers)]
+
+    def one_step():
+        for kc, vc, k, v in stack:
+            kernels.kv_store_batch(kc, vc, k, v, G, d, n_ctx, P, B)
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        one_step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+    nbytes = 2.0 * B * G * d * (4 + 2)  # K and V: fp32 read, fp16 written
+    kc, vc, k, v = stack[0]
+    wk = np.zeros((G, n_ctx, d), np.uint16)
+    wv = np.zeros((G, n_ctx, d), np.uint16)
+    ref.kv_store_f16(wk, wv, k.cpu().numpy(), v.cpu().numpy(), G, d, n_ctx, P, B)
+    exact = bool(np.array_equal(kc.cpu().numpy().view(np.uint16), wk) and np.array_equal(vc.cpu().numpy().view(np.uint16), wv))
+    return dict(value=nbytes * layers * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+                config=dict(workload=name, shape=f"G{G} d{d}", layers=layers, n_ctx=n_ctx, pos_base=P, batch=B,
+                            bytes_per_step=nbytes * layers),
+                roofline=dict(bound="hbm", achieved=nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None, kernel="kv_store_kernel<8, false>",
+                              launch_us=us, bytes_per_launch=nbytes,
+                              note="3 MB per launch: bound by the launch, not by HBM"),
+                parity=dict(bit_exact=exact, rows="layer 0, whole cache, vs CPU oracle"))
+
+
+def run_kv_shift(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = kv_shift over the whole cache (all layers, K and V), in place."""
+    from oracle import ref
+    shape_name, _, n_ctx, (n_keep, shift) = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    G, d, layers = s["G"], s["d"], s["layers"]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(78)
+    kc = torch.randint(1, 30000, (layers, G, n_ctx, d), generator=g, device="cuda", dtype=torch.int16)
+    vc = torch.randint(1, 30000, (layers, G, n_ctx, d), generator=g, device="cuda", dtype=torch.int16)
+    # parity on the first launch, against the oracle on two layers' worth of the same data
+    hk, hv = kc[:2].cpu().numpy().view(np.uint16).copy(), vc[:2].cpu().numpy().view(np.uint16).copy()
+    ref.kv_shift_u16(hk, hv, 2, G, d, n_ctx, n_keep, shift)
+    kernels.kv_shift(kc, vc, layers, G, d, n_ctx, n_keep, shift)
+    torch.cuda.synchronize()
+    exact = bool(np.array_equal(kc[:2].cpu().numpy().view(np.uint16), hk) and
+                 np.array_equal(vc[:2].cpu().numpy().view(np.uint16), hv))
+    for _ in range(warmup):
+        kernels.kv_shift(kc, vc, layers, G, d, n_ctx, n_keep, shift)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        kernels.kv_shift(kc, vc, layers, G, d, n_ctx, n_keep, shift)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = e0.elapsed_time(e1) * 1e3 / steps
+    moved = n_ctx - n_keep - shift
+    nbytes = 2.0 * layers * G * d * 2 * (moved + moved + shift)  # rows read + rows written + rows cleared, K and V
+    return dict(value=nbytes * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+                config=dict(workload=name, shape=f"G{G} d{d}", layers=layers, n_ctx=n_ctx, n_keep=n_keep, shift=shift,
+                            bytes_per_step=nbytes),
+                roofline=dict(bound="hbm", achieved=nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None, kernel="kv_shift_kernel<16>",
+                              launch_us=us, bytes_per_launch=nbytes),
+                parity=dict(bit_exact=exact, rows="layers 0-1, whole strips, vs CPU oracle"))
+
+
 def run_copy(torch, kernels, name, steps, warmup, with_cpu):
     """dst.copy_(src) over rotating buffer pairs larger than the last-level cache."""
     nbytes = WORKLOADS[name][3]
@@ -351,7 +440,8 @@ def run_copy(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "copy": run_copy}[kind]
+    fn = {"prefill": run_prefill, "decode": run_decode, "copy": run_copy, "kv_store": run_kv_store,
+          "kv_shift": run_kv_shift}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
 
