@@ -53,6 +53,8 @@ WORKLOADS = {
     # the two mutators of the cache (byte movers; value = bytes read + written per second)
     "llama8b-kv-store-512": ("llama8b", "kv_store", 8192, (4096, 512)),
     "qwen1.5b-kv-shift-32k": ("qwen1.5b", "kv_shift", 32768, (4, 16382)),
+    # rotary embedding of a 512-token chunk's Q and K rows (value = bytes read + written per second)
+    "llama8b-rope-512": ("llama8b", "rope", 8192, (4096, 512)),
     # not part of the path: a plain device copy of known size, the yardstick that the HBM
     # counters (FETCH_SIZE / WRITE_SIZE) and the achievable streaming rate are scaled by
     "hbm-copy-256MiB": (None, "copy", 0, 256 << 20),
@@ -66,7 +68,7 @@ TRAFFIC = {
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
 ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k",
-        "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
+        "llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
 
 
 def prefill_flops(H, d, P, B):
@@ -373,6 +375,54 @@ def run_kv_store(torch, kernels, name, steps, warmup, with_cpu):
                 parity=dict(bit_exact=exact, rows="layer 0, whole cache, vs CPU oracle"))
 
 
+def run_rope(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = rope_normal_batch on the Q rows and on the K rows of a 512-token chunk, per layer."""
+    from oracle import ref
+    shape_name, _, n_ctx, (P, B) = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    H, G, d, layers = s["H"], s["G"], s["d"], s["layers"]
+    theta = 500000.0
+    g = torch.Generator(device="cuda")
+    g.manual_seed(79)
+    q0 = torch.randn((B * H, d), generator=g, device="cuda")
+    k0 = torch.randn((B * G, d), generator=g, device="cuda")
+    stack = [(q0.clone(), k0.clone()) for _ in range(layers)]
+    kernels.rope_normal_batch(stack[0][0], B * H, d, d, theta, P, H)
+    kernels.rope_normal_batch(stack[0][1], B * G, d, d, theta, P, G)
+    torch.cuda.synchronize()
+    wq = ref.rope_batch(q0.cpu().numpy(), d, d, theta, P, H, None, False)
+    wk = ref.rope_batch(k0.cpu().numpy(), d, d, theta, P, G, None, False)
+    err = max(float(np.abs(stack[0][0].cpu().numpy() - wq).max() / np.abs(wq).max()),
+              float(np.abs(stack[0][1].cpu().numpy() - wk).max() / np.abs(wk).max()))
+
+    def one_step():
+        for q, k in stack:
+            kernels.rope_normal_batch(q, B * H, d, d, theta, P, H)
+            kernels.rope_normal_batch(k, B * G, d, d, theta, P, G)
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        one_step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+    nbytes = 2.0 * B * (H + G) * d * 4
+    return dict(value=nbytes * layers * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+                config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_past=P, batch=B, n_rot=d,
+                            bytes_per_step=nbytes * layers),
+                roofline=dict(bound="hbm", achieved=nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None,
+                              kernel="rope_kernel<false, false>, Q rows then K rows", launch_us=us,
+                              bytes_per_launch=nbytes, note="launch_us and bytes cover the two launches of a layer"),
+                parity=dict(max_rel_to_tensor_max=err, rows="layer 0, all rows, vs CPU oracle"))
+
+
 def run_kv_shift(torch, kernels, name, steps, warmup, with_cpu):
     """One step = kv_shift over the whole cache (all layers, K and V), in place."""
     from oracle import ref
@@ -441,7 +491,7 @@ def run_copy(torch, kernels, name, steps, warmup, with_cpu):
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
     fn = {"prefill": run_prefill, "decode": run_decode, "copy": run_copy, "kv_store": run_kv_store,
-          "kv_shift": run_kv_shift}[kind]
+          "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
 

@@ -74,6 +74,19 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
 
+/* Replace llm::cuda::rope_neox_batch / rope_normal_batch (neox != 0 / == 0) and rope_neox_ind /
+ * rope_normal_ind (reference: src/kernels.h:55-62, src/kernels.cu:1619-1657, 2059-2075; CPU statement
+ * src/model_cpu.cpp:179-203): rotary position embedding in place on fp32 rows x[rows][head_dim].
+ * Pair i of a row turns by pos * theta^(-2i/n_rot) (divided by freq_factors[i] when freq_factors is
+ * not NULL; n_rot/2 floats on the device); elements at or past n_rot are untouched.
+ * Batch form: row = token * heads + head, pos = n_past + token (call site src/model_gpu.cu:379-381).
+ * Single-token form: every row is a head of the one token whose position is read from device
+ * memory (capture-safe; call site src/model_gpu.cu:277-279). */
+int orin_fa_rope_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                       const float* freq_factors, int neox);
+int orin_fa_rope_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos,
+                     const float* freq_factors, int neox);
+
 /* Replaces llm::cuda::kv_store_batch (reference: src/kernels.h:66-67, src/kernels.cu:1659-1678,
  * 2079-2083; CPU statement src/model_cpu.cpp:276-279): rounds the fp32 K and V rows of `batch`
  * tokens (k, v: [batch][heads][head_dim]) to binary16, nearest-even, into cache positions

@@ -1,5 +1,5 @@
-// The attention and KV-cache slice of the orin_llm operator API, with the reference's own
-// signatures (reference: src/kernels.h:8-10, :66-73 and :77-81), implemented for MI355X by
+// The attention, KV-cache and rotary-embedding slice of the orin_llm operator API, with the reference's own
+// signatures (reference: src/kernels.h:8-10, :55-62, :66-73 and :77-81), implemented for MI355X by
 // liborin_fa.so.  An engine built against the reference header links these symbols
 // unchanged; each forwards to the C ABI in include/orin_fa.h and, like the
 // reference's CUDA_CHECK (src/common.h:14-22), prints and abort()s on failure.
@@ -20,6 +20,14 @@ namespace llm::cuda {
 int init();
 void set_stream(void* stream);
 #endif
+
+void rope_neox_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors = nullptr);
+
+void rope_normal_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors = nullptr);
+
+void rope_neox_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos, const float* freq_factors = nullptr);
+
+void rope_normal_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos, const float* freq_factors = nullptr);
 
 void kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
                     int heads, int head_dim, int n_ctx, int pos_base, int batch);

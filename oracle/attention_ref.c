@@ -12,6 +12,8 @@
  *   orc_flash_attention*, _rows           composition of the above, checked against the same fixtures
  *   orc_kv_store_*                        exact against numpy astype(float16) at the documented offset
  *   orc_kv_shift_u16                      exact against the slice statement new[keep:n-s] = old[keep+s:], tail 0
+ *   orc_rope_*                            float64 rotation by the same fp32 angle; neox == permuted normal, bit for bit;
+ *                                         position 0 is the identity; elements past n_rot untouched
  */
 #include "attention_ref.h"
 
@@ -128,6 +130,46 @@ void orc_kv_shift_u16(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int hea
             memset(kh + (size_t)(n_ctx - shift) * d, 0, (size_t)shift * d * sizeof(uint16_t));
             memset(vh + (size_t)(n_ctx - shift) * d, 0, (size_t)shift * d * sizeof(uint16_t));
         }
+}
+
+/* ---- rotary position embedding ------------------------------------------------ */
+
+/* One head row (reference: src/model_cpu.cpp:179-190 and :193-203).  std::pow, std::cos and
+ * std::sin on float arguments are the float overloads. */
+void orc_rope_neox_row(float* x, int n_rot, float theta, int pos, const float* freq_factors) {
+    const int half = n_rot / 2;
+    for (int i = 0; i < half; ++i) {
+        float freq = powf(theta, -2.0f * i / n_rot);
+        if (freq_factors) freq /= freq_factors[i];
+        const float ang = (float)pos * freq;
+        const float c = cosf(ang), s = sinf(ang);
+        const float x0 = x[i], x1 = x[i + half];
+        x[i] = x0 * c - x1 * s;
+        x[i + half] = x0 * s + x1 * c;
+    }
+}
+
+void orc_rope_normal_row(float* x, int n_rot, float theta, int pos, const float* freq_factors) {
+    for (int i = 0; i < n_rot; i += 2) {
+        float freq = powf(theta, -1.0f * i / n_rot);
+        if (freq_factors) freq /= freq_factors[i / 2];
+        const float ang = (float)pos * freq;
+        const float c = cosf(ang), s = sinf(ang);
+        const float x0 = x[i], x1 = x[i + 1];
+        x[i] = x0 * c - x1 * s;
+        x[i + 1] = x0 * s + x1 * c;
+    }
+}
+
+/* All rows of a chunk: row = token * heads + head, position n_past + token (the loop of
+ * src/model_cpu.cpp:264-275 over heads, run token by token as :314-319 does). */
+void orc_rope_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                    const float* freq_factors, int neox) {
+    for (int r = 0; r < rows; ++r) {
+        const int pos = n_past + r / heads;
+        if (neox) orc_rope_neox_row(x + (size_t)r * head_dim, n_rot, theta, pos, freq_factors);
+        else orc_rope_normal_row(x + (size_t)r * head_dim, n_rot, theta, pos, freq_factors);
+    }
 }
 
 /* ---- attention -------------------------------------------------------------- */

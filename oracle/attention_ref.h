@@ -46,6 +46,13 @@ void orc_kv_store_f16(uint16_t* kc, uint16_t* vc, const float* k, const float* v
 void orc_kv_shift_u16(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx,
                       int n_keep, int shift);
 
+/* Rotary position embedding, in place (reference: src/model_cpu.cpp:179-203, call site :264-275).
+ * x: [rows][head_dim] with row = token * heads + head; position of a row = n_past + token. */
+void orc_rope_neox_row(float* x, int n_rot, float theta, int pos, const float* freq_factors);
+void orc_rope_normal_row(float* x, int n_rot, float theta, int pos, const float* freq_factors);
+void orc_rope_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                    const float* freq_factors, int neox);
+
 /* One query token against the first npos cache positions
  * (reference: src/model_cpu.cpp:281-295, softmax :20-30, dot :32-36).
  * q, out: [n_head][head_dim].  score: caller scratch of >= npos floats.

@@ -32,6 +32,7 @@ def _load():
     lib.orc_fp32_to_fp16_n.argtypes = [_f32p, _u16p, ctypes.c_size_t]
     lib.orc_kv_store_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int]
     lib.orc_kv_store_f16.argtypes = [_u16p, _u16p, _f32p, _f32p, _int, _int, _int, _int, _int]
+    lib.orc_rope_batch.argtypes = [_f32p, _int, _int, _int, _flt, _int, _int, _f32p, _int]
     lib.orc_kv_shift_u16.argtypes = [_u16p, _u16p, _int, _int, _int, _int, _int, _int]
     lib.orc_attention_token_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
     lib.orc_attention_token_f16.argtypes = [_f32p, _u16p, _u16p, _f32p, _int, _int, _int, _int, _int, _flt, _f32p]
@@ -86,6 +87,16 @@ def kv_store_f16(kc, vc, k, v, n_kv, d, n_ctx, pos_base, batch):
     k, v = _c(k, np.float32), _c(v, np.float32)
     assert kc.dtype == np.uint16 and kc.flags.c_contiguous and kc.size == n_kv * n_ctx * d
     lib().orc_kv_store_f16(_p(kc, _u16p), _p(vc, _u16p), _p(k, _f32p), _p(v, _f32p), n_kv, d, n_ctx, pos_base, batch)
+
+
+def rope_batch(x, head_dim, n_rot, theta, n_past, heads, freq_factors=None, neox=True):
+    """x: fp32 [rows][head_dim] (row = token * heads + head); returns the rotated copy."""
+    x = np.array(x, dtype=np.float32, order="C", copy=True)
+    rows = x.size // head_dim
+    ff = None if freq_factors is None else _c(freq_factors, np.float32)
+    lib().orc_rope_batch(_p(x, _f32p), rows, head_dim, n_rot, np.float32(theta), n_past, heads,
+                         None if ff is None else _p(ff, _f32p), 1 if neox else 0)
+    return x
 
 
 def kv_shift_u16(kc, vc, n_layer, n_kv, d, n_ctx, n_keep, shift):

@@ -3,7 +3,8 @@
 //
 // Boundary: the reference's llm::cuda::flash_attention and flash_attention_decode_ind
 // (reference: src/kernels.h:77-81, launchers at src/kernels.cu:1944-2000) and its KV-cache
-// mutators kv_store_batch / kv_store_ind / kv_shift (src/kernels.h:66-73, src/kernels.cu:2079-2093).
+// mutators kv_store_batch / kv_store_ind / kv_shift (src/kernels.h:66-73, src/kernels.cu:2079-2093) and the
+// rotary embedding rope_{neox,normal}_{batch,ind} (src/kernels.h:55-62, src/kernels.cu:2059-2075).
 #include "fa_common.hpp"
 
 #include <stdio.h>
@@ -205,6 +206,26 @@ int orin_fa_kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head
     if (n_keep < 0 || shift < 0 || (long long)n_keep + shift > n_ctx) return ORIN_FA_E_INVALID;
     if (shift == 0) return ORIN_FA_OK;
     return hip_code(kv_shift_launch(kc, vc, n_layer, n_kv, head_dim, n_ctx, n_keep, shift, g_state.stream));
+}
+
+int orin_fa_rope_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                       const float* freq_factors, int neox) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!x) return ORIN_FA_E_INVALID;
+    if (rows < 0 || head_dim <= 0 || heads <= 0 || n_past < 0 || rows % heads != 0) return ORIN_FA_E_INVALID;
+    if (n_rot < 0 || n_rot > head_dim || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    if (rows == 0 || n_rot == 0) return ORIN_FA_OK;
+    return hip_code(rope_launch(x, rows, head_dim, n_rot, theta, n_past, heads, nullptr, freq_factors, neox != 0, g_state.stream));
+}
+
+int orin_fa_rope_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos,
+                     const float* freq_factors, int neox) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!x || !d_pos) return ORIN_FA_E_INVALID;
+    if (rows < 0 || head_dim <= 0) return ORIN_FA_E_INVALID;
+    if (n_rot < 0 || n_rot > head_dim || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    if (rows == 0 || n_rot == 0) return ORIN_FA_OK;
+    return hip_code(rope_launch(x, rows, head_dim, n_rot, theta, 0, rows, d_pos, freq_factors, neox != 0, g_state.stream));
 }
 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {

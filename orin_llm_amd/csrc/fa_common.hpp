@@ -61,6 +61,10 @@ hipError_t kv_store_launch(uint16_t* kc, uint16_t* vc, const float* k, const flo
 hipError_t kv_shift_launch(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep,
                            int shift, hipStream_t stream);
 
+// Rotary embedding (rope.hip).  d_pos not null selects the single-token form.
+hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                       const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream);
+
 template <int N>
 struct IntC {
     static constexpr int value = N;

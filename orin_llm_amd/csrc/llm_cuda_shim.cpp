@@ -1,5 +1,5 @@
 // llm::cuda::* entry points with the reference's signatures (reference:
-// src/kernels.h:8-10,66-73,77-81; definitions src/kernels.cu:1728-1737,1974-2000,2079-2093),
+// src/kernels.h:8-10,55-62,66-73,77-81; definitions src/kernels.cu:1728-1737,1974-2000,2059-2093),
 // forwarding to the C ABI.  Plain C++: no HIP headers, no device code.
 #include "../../include/orin_llm_amd/kernels.h"
 
@@ -33,6 +33,26 @@ int init() {
 
 void set_stream(void* stream) { orin_fa_set_stream(stream); }
 #endif
+
+void rope_neox_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors) {
+    const int rc = orin_fa_rope_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors, 1);
+    if (rc != ORIN_FA_OK) die("rope_neox_batch", rc);
+}
+
+void rope_normal_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors) {
+    const int rc = orin_fa_rope_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors, 0);
+    if (rc != ORIN_FA_OK) die("rope_normal_batch", rc);
+}
+
+void rope_neox_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos, const float* freq_factors) {
+    const int rc = orin_fa_rope_ind(x, rows, head_dim, n_rot, theta, d_pos, freq_factors, 1);
+    if (rc != ORIN_FA_OK) die("rope_neox_ind", rc);
+}
+
+void rope_normal_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos, const float* freq_factors) {
+    const int rc = orin_fa_rope_ind(x, rows, head_dim, n_rot, theta, d_pos, freq_factors, 0);
+    if (rc != ORIN_FA_OK) die("rope_normal_ind", rc);
+}
 
 void kv_store_batch(uint16_t* kc, uint16_t* vc, const float* k, const float* v,
                     int heads, int head_dim, int n_ctx, int pos_base, int batch) {

@@ -1,0 +1,101 @@
+// Rotary position embedding for gfx950 (MI355X), in place on fp32 rows [rows][head_dim].
+//
+// Replaces the reference's rope_neox_k / rope_normal_k and their four wrappers (reference:
+// src/kernels.cu:1619-1657, 2059-2075; CPU statement src/model_cpu.cpp:179-203; call sites
+// src/model_gpu.cu:277-279, 379-381).  Pair i of a row is rotated by the angle pos * freq_i,
+// freq_i = theta^(-2i/n_rot) (divided by freq_factors[i] when given); "neox" pairs element i
+// with i + n_rot/2, "normal" pairs 2i with 2i + 1; elements at or past n_rot are left alone.
+// pos = n_past + row / heads (batch form) or *d_pos (single-token form, read on the device).
+//
+// Every head of a token shares the token's angles, so one thread owns (token, pair, group of up
+// to 8 heads): the block's first threads compute the frequency of each pair once into LDS, each
+// thread forms its angle and one sine/cosine, then rotates its heads with all loads issued
+// before the first store -- where the reference spends a power, a sine and a cosine per element
+// pair of every head.
+// Arithmetic follows the CPU statement operation by operation in fp32 (no contraction of
+// the rotation into fused multiply-adds); the frequency is the double-precision power rounded
+// to fp32, which is what a correctly rounded powf returns, because at position 32768 one ulp
+// of the frequency already moves the angle by 2e-3 rad.  Sine and cosine are the accurate
+// library versions (full range reduction), not the fast hardware approximations the reference's
+// GPU path uses.
+#include "fa_common.hpp"
+
+namespace orin_fa {
+namespace {
+
+constexpr int kHeadsPerThread = 8;
+
+template <bool NEOX, bool IND>
+__global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int heads, int head_dim, int n_rot,
+                                                   float theta, int n_past, const int* d_pos,
+                                                   const float* freq_factors) {
+#pragma clang fp contract(off)
+    __shared__ float sh_freq[128];
+    const int half = n_rot / 2;
+    const int n_hgroups = (heads + kHeadsPerThread - 1) / kHeadsPerThread;
+    // pair index fastest, then head group, then token; a block covers whole runs of pairs when
+    // half divides 256, otherwise every thread computes its own frequency
+    const bool shared_freq = half <= 128 && (256 % half) == 0;
+    if (shared_freq && (int)threadIdx.x < half) {
+        const int i = threadIdx.x;
+        const float expo = -2.0f * (float)i / (float)n_rot;
+        float f = (float)pow((double)theta, (double)expo);
+        if (freq_factors) f /= freq_factors[i];
+        sh_freq[i] = f;
+    }
+    if (shared_freq) __syncthreads();
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (long long)tokens * n_hgroups * half) return;
+    const int i = (int)(t % half);
+    const long long th = t / half;
+    const int hgroup = (int)(th % n_hgroups), token = (int)(th / n_hgroups);
+    float freq;
+    if (shared_freq) {
+        freq = sh_freq[i];
+    } else {
+        const float expo = -2.0f * (float)i / (float)n_rot;
+        freq = (float)pow((double)theta, (double)expo);
+        if (freq_factors) freq /= freq_factors[i];
+    }
+    const int pos = IND ? *d_pos : n_past + token;
+    const float ang = (float)pos * freq;
+    const float c = cosf(ang), s = sinf(ang);
+    const int h0 = hgroup * kHeadsPerThread;
+    float* row = x + ((size_t)token * heads + h0) * head_dim;
+    const int i0 = NEOX ? i : 2 * i, i1 = NEOX ? i + half : 2 * i + 1;
+    float x0[kHeadsPerThread], x1[kHeadsPerThread];
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread; ++u)
+        if (h0 + u < heads) {
+            x0[u] = row[(size_t)u * head_dim + i0];
+            x1[u] = row[(size_t)u * head_dim + i1];
+        }
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread; ++u)
+        if (h0 + u < heads) {
+            row[(size_t)u * head_dim + i0] = x0[u] * c - x1[u] * s;
+            row[(size_t)u * head_dim + i1] = x0[u] * s + x1[u] * c;
+        }
+}
+
+} // namespace
+
+hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
+                       const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream) {
+    // batch form: rows = tokens * heads; single-token form: every row belongs to the one token
+    const int tokens = d_pos ? 1 : rows / heads;
+    const int heads_per_token = d_pos ? rows : heads;
+    const int n_hgroups = (heads_per_token + kHeadsPerThread - 1) / kHeadsPerThread;
+    const long long threads = (long long)tokens * n_hgroups * (n_rot / 2);
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (grid == 0) return hipSuccess;
+#define ORIN_ROPE_LAUNCH(NEOX, IND) \
+    hipLaunchKernelGGL((rope_kernel<NEOX, IND>), dim3(grid), dim3(256), 0, stream, x, tokens, heads_per_token, \
+                       head_dim, n_rot, theta, n_past, d_pos, freq_factors)
+    if (neox) { if (d_pos) ORIN_ROPE_LAUNCH(true, true); else ORIN_ROPE_LAUNCH(true, false); }
+    else      { if (d_pos) ORIN_ROPE_LAUNCH(false, true); else ORIN_ROPE_LAUNCH(false, false); }
+#undef ORIN_ROPE_LAUNCH
+    return hipGetLastError();
+}
+
+} // namespace orin_fa

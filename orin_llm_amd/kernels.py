@@ -43,6 +43,10 @@ def lib():
         L.orin_fa_prefill.restype = _int
         L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_rope_batch.argtypes = [_vp, _int, _int, _int, _flt, _int, _int, _vp, _int]
+        L.orin_fa_rope_batch.restype = _int
+        L.orin_fa_rope_ind.argtypes = [_vp, _int, _int, _int, _flt, _vp, _vp, _int]
+        L.orin_fa_rope_ind.restype = _int
         L.orin_fa_kv_store_batch.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int]
         L.orin_fa_kv_store_batch.restype = _int
         L.orin_fa_kv_store_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _vp]
@@ -108,6 +112,30 @@ def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_
                                   _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def rope_neox_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors=None):
+    rc = lib().orin_fa_rope_batch(_ptr(x), rows, head_dim, n_rot, theta, n_past, heads, _ptr(freq_factors), 1)
+    if rc != 0:
+        raise OrinFaError("rope_neox_batch", rc)
+
+
+def rope_normal_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors=None):
+    rc = lib().orin_fa_rope_batch(_ptr(x), rows, head_dim, n_rot, theta, n_past, heads, _ptr(freq_factors), 0)
+    if rc != 0:
+        raise OrinFaError("rope_normal_batch", rc)
+
+
+def rope_neox_ind(x, rows, head_dim, n_rot, theta, d_pos, freq_factors=None):
+    rc = lib().orin_fa_rope_ind(_ptr(x), rows, head_dim, n_rot, theta, _ptr(d_pos), _ptr(freq_factors), 1)
+    if rc != 0:
+        raise OrinFaError("rope_neox_ind", rc)
+
+
+def rope_normal_ind(x, rows, head_dim, n_rot, theta, d_pos, freq_factors=None):
+    rc = lib().orin_fa_rope_ind(_ptr(x), rows, head_dim, n_rot, theta, _ptr(d_pos), _ptr(freq_factors), 0)
+    if rc != 0:
+        raise OrinFaError("rope_normal_ind", rc)
 
 
 def kv_store_batch(kc, vc, k, v, heads, head_dim, n_ctx, pos_base, batch):

@@ -34,7 +34,7 @@ def test_header_declares_the_expected_entry_points():
     assert _declared_c_functions() == sorted([
         "orin_fa_init", "orin_fa_set_stream", "orin_fa_workspace_bytes", "orin_fa_set_workspace",
         "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_ind_timed", "orin_fa_decode_splits",
-        "orin_fa_kv_store_batch", "orin_fa_kv_store_ind", "orin_fa_kv_shift", "orin_fa_cu_count",
+        "orin_fa_kv_store_batch", "orin_fa_kv_store_ind", "orin_fa_kv_shift", "orin_fa_rope_batch", "orin_fa_rope_ind", "orin_fa_cu_count",
         "orin_fa_error_string"])
 
 
@@ -76,6 +76,10 @@ def test_shim_symbols_have_the_reference_manglings():
     expected = [
         "_ZN3llm4cuda15flash_attentionEPKfPKtS4_Pfiiiiiif",
         "_ZN3llm4cuda26flash_attention_decode_indEPKfPKtS4_PfiiiiPKif",
+        "_ZN3llm4cuda15rope_neox_batchEPfiiifiiPKf",
+        "_ZN3llm4cuda17rope_normal_batchEPfiiifiiPKf",
+        "_ZN3llm4cuda13rope_neox_indEPfiiifPKiPKf",
+        "_ZN3llm4cuda15rope_normal_indEPfiiifPKiPKf",
         "_ZN3llm4cuda14kv_store_batchEPtS1_PKfS3_iiiii",
         "_ZN3llm4cuda12kv_store_indEPtS1_PKfS3_iiiPKi",
         "_ZN3llm4cuda8kv_shiftEPtS1_iiiiii",
@@ -95,5 +99,6 @@ def _decl(text, name):
 @pytest.mark.skipif(not os.path.exists(REF_HDR), reason="reference tree not present on this machine")
 def test_shim_header_matches_reference_declarations():
     ref, ours = open(REF_HDR).read(), open(SHIM_HDR).read()
-    for name in ("flash_attention", "flash_attention_decode_ind", "kv_store_batch", "kv_store_ind", "kv_shift"):
+    for name in ("flash_attention", "flash_attention_decode_ind", "kv_store_batch", "kv_store_ind", "kv_shift",
+                 "rope_neox_batch", "rope_normal_batch", "rope_neox_ind", "rope_normal_ind"):
         assert _decl(ours, name) == _decl(ref, name)
