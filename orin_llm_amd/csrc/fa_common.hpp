@@ -42,6 +42,8 @@ struct FaArgs {
     int r;             // query heads per KV head
     int n_hgroups;     // head groups per KV head
     int n_ttiles;      // prefill: token tiles
+    int tq;            // prefill: tokens per token tile
+    int heads_per_group; // prefill: query heads per head group
     int n_splits;      // decode: KV splits
     float c;           // |scale| * log2(e), clamped away from zero
     float qsign;       // sign of scale, folded into Q

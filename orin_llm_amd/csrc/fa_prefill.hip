@@ -3,25 +3,27 @@
 // Replaces the reference's flash_attention_prefill_mma_k and its launcher (reference:
 // src/kernels.cu:1347-1568, 1944-1981).
 //
-// A workgroup is 4 wave64s that own one KV head, a block of NQB*16 query columns (TQ tokens x
+// A workgroup is 4 wave64s that own one KV head, a block of NCB*32 query columns (tq tokens x
 // the heads of the group) and the 32-row KV tiles those columns can see; wave w takes tiles
 // w, w+4, ... and keeps its own online-softmax state, so the main loop has no workgroup
-// barrier.  S^T = K Q^T and O^T = V^T P run on v_mfma_f32_16x16x32_f16: the accumulator layout
-// of the first product (lane = query column, 4 KV rows per lane-group) is the B-operand layout
-// of the second once the 32 KV rows of a tile are numbered (lane-group, sub-tile, row), so P
-// needs no shuffle and every per-column quantity is a per-lane scalar.
+// barrier.  S^T = K Q^T and O^T = V^T P run on v_mfma_f32_32x32x16_f16 (a single wave reaches
+// 94 % of the matrix pipe's rate with this shape against 75 % with 16x16x32, and each
+// instruction leaves three times the room for vector work beside it).  The accumulator layout
+// of the first product -- lane = query column, lane-half h holds KV rows 8q + 4h + 0..3 -- is
+// the B-operand layout of the second once the 16 KV rows of a k-step are numbered
+// (lane-half, register), so P needs no shuffle and every per-column quantity is a per-lane scalar.
 //
 // The three stages of a tile
-//     A: S = K Q^T (MFMA)      B: P = 2^(S*c + b) (VALU)      C: O += V^T P, l += 1^T P (MFMA)
+//     A: S = K Q^T (MFMA)      B: P = 2^(S*c + b) (VALU)      C: O += V^T P (MFMA)
 // run skewed -- iteration t issues A(t+1), B(t) and C(t-1), which are independent of one
 // another -- in one hand-ordered instruction stream, so the matrix pipe works while the vector
 // pipe exponentiates.  What keeps the vector share small:
 //   * B is one fused multiply-add (scale*log2(e) and the column's offset b = shift - reference
 //     maximum; Q itself stays unscaled, so fp16-representable inputs enter the products exactly),
-//     one v_exp_f32 per score and one v_cvt_pk_f16_f32 per pair.
-//   * Row sums are one more matrix instruction per query block (a ones operand times P).
+//     one v_exp_f32 per score, and per pair of scores one v_cvt_pk_f16_f32, one v_max3_f32 and one
+//     v_dot2_f32_f16 against packed ones (the row sum of the rounded weights, in fp32).
 //   * The reference maximum is lazy: exponentials are computed optimistically while the largest
-//     exponent of the tile is tracked; only if it exceeds the fp16-safe bound (on a handful of
+//     weight of the tile is tracked; only if it exceeds the fp16-safe bound (on a handful of
 //     early tiles) does a slow path move the reference, redo the tile's P and rescale O and l.
 // K and V tiles are copied global->LDS by the load unit itself (no staging registers, two
 // buffers each per wave, tile base in the scalar offset so the copies need no vector
@@ -38,10 +40,13 @@
 namespace orin_fa {
 namespace {
 
-template <int D, int NQB>
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <int D, int NCB>
 struct PGeom {
-    static constexpr int kSteps = D / 32;
-    static constexpr int kDBlk = D / 16;
+    static constexpr int kSteps = D / 16;             // k-steps of A over head_dim
+    static constexpr int kDBlk = D / 32;              // 32-wide output blocks over head_dim
+    static constexpr int kCols = NCB * 32;            // query columns per workgroup
     static constexpr int kRowB = D * 2;               // bytes per K/V row in LDS (no padding; chunks are XOR-swizzled)
     static constexpr int kChunks = D / 8;             // 16-byte chunks per row
     static constexpr int kTileB = kTile * kRowB;      // one K or V tile
@@ -50,21 +55,20 @@ struct PGeom {
     static constexpr int kKOff = 0;                   // wave slice: K buffers 0/1, then V buffers 0/1
     static constexpr int kVOff = 2 * kTileB;
     static constexpr int kOStride = D + 4;
-    static constexpr int kMergeB = NQB * 16 * kOStride * 4;
-    static constexpr int kScratchOff = 4 * kTileB;    // 1 KB per wave: 16 bytes per lane for accumulator round trips
-    static constexpr int kWaveB = (4 * kTileB + 1024 > kMergeB) ? 4 * kTileB + 1024 : kMergeB;
+    static constexpr int kMergeB = kCols * kOStride * 4;
+    static constexpr int kWaveB = (4 * kTileB > kMergeB) ? 4 * kTileB : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
-    static constexpr int kQOff = kMlOff + kPrefillWaves * NQB * 16 * 2 * 4; // the query block as fp16, [column][head_dim]
-    static constexpr int kQStride = D * 2 + 16;       // (padded: 16 columns read 16 bytes each without bank conflicts)
-    static constexpr int kLdsB = kQOff + NQB * 16 * kQStride;
+    static constexpr int kQOff = kMlOff + kPrefillWaves * kCols * 2 * 4; // the query block as fp16, [column][head_dim]
+    static constexpr int kQStride = D * 2 + 16;       // (padded against bank conflicts of the operand reads)
+    static constexpr int kLdsB = kQOff + kCols * kQStride;
 };
 
 // ---------------------------------------------------------------------------------------------
 // Instructions with the register file of each operand spelled out.  The kernel keeps its score
 // accumulators in ordinary vector registers (the exponentials read them with no copy) and its
-// output accumulators and the query operands in the accumulation-register file, and it fixes the issue order of matrix
-// and vector work by hand -- neither of which the builtin forms allow.  The price: the compiler
-// knows nothing about the hazards of these blocks.
+// output accumulators and the query operands in the accumulation-register file, and it fixes the
+// issue order of matrix and vector work by hand -- neither of which the builtin forms allow.
+// The price: the compiler knows nothing about the hazards of these blocks.
 //   (1) Result latency: a non-matrix instruction reads a matrix result only a pipeline stage
 //       (at least two later matrix instructions) after it was issued, or behind settle().
 //   (2) A matrix instruction must not read an operand in the two cycles after a vector
@@ -73,50 +77,41 @@ struct PGeom {
 //       (prologue, drain); the main loop uses the bare forms, where every operand was written
 //       a long way back (LDS reads, the previous iteration's conversions, loop invariants).
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void mfma_v_n(f4& acc, h8 a_op, h8 b_acc) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
+__device__ __forceinline__ void mfma_s_n(f16v& acc, h8 a_op, h8 b_acc) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
 }
-__device__ __forceinline__ void mfma_v_zero_n(f4& acc, h8 a_op, h8 b_acc) { // acc = A B
+__device__ __forceinline__ void mfma_s_zero_n(f16v& acc, h8 a_op, h8 b_acc) { // acc = A B
     // early clobber: the destination must not share registers with an operand that dies here
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
 }
-__device__ __forceinline__ void mfma_a_n(f4& acc, h8 a_op, h8 b_op) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
+__device__ __forceinline__ void mfma_o_n(f16v& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
 }
-__device__ __forceinline__ void mfma_a_zero_n(f4& acc, h8 a_op, h8 b_op) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&a"(acc) : "v"(a_op), "v"(b_op));
+__device__ __forceinline__ void mfma_o_zero_n(f16v& acc, h8 a_op, h8 b_op) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&a"(acc) : "v"(a_op), "v"(b_op));
 }
-__device__ __forceinline__ void mfma_v(f4& acc, h8 a_op, h8 b_acc) {
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
+__device__ __forceinline__ void mfma_s(f16v& acc, h8 a_op, h8 b_acc) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_op), "a"(b_acc));
 }
-__device__ __forceinline__ void mfma_v_zero(f4& acc, h8 a_op, h8 b_acc) { // acc = A B
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
+__device__ __forceinline__ void mfma_s_zero(f16v& acc, h8 a_op, h8 b_acc) { // acc = A B
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a_op), "a"(b_acc));
 }
-__device__ __forceinline__ void mfma_a(f4& acc, h8 a_op, h8 b_op) {
-    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
+__device__ __forceinline__ void mfma_o(f16v& acc, h8 a_op, h8 b_op) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a_op), "v"(b_op));
 }
-// Lets the matrix pipe drain (32 wait states, more than any 16x16x32 result needs) and stops the
+// Lets the matrix pipe drain (48 wait states, more than any 32x32x16 result needs) and stops the
 // compiler from moving anything across.
 __device__ __forceinline__ void settle() {
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 }
-// 16 bytes between LDS and the accumulation-register file, without a detour through vector
-// registers.  The output accumulators are only ever touched by these and by the matrix
-// instructions, which keeps them in that file for the whole kernel.
-__device__ __forceinline__ void lds_store_acc(unsigned lds_addr, const f4& acc) {
-    asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(lds_addr), "a"(acc) : "memory");
-}
-template <int OFF>
-__device__ __forceinline__ void lds_store_acc_nowait(unsigned lds_addr, const f4& acc) { // caller waits
-    asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(lds_addr), "a"(acc), "n"(OFF) : "memory");
-}
-// (The accumulator is declared read-write although its old value is dead: a tied operand keeps it in
-// the same registers, where a fresh definition on a rarely taken path costs a copy of the whole set.)
-__device__ __forceinline__ void lds_load_acc(f4& acc, unsigned lds_addr) {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "+a"(acc) : "v"(lds_addr) : "memory");
-}
+// Empty blocks that tie a 16-register value to a register file at a point of the program: the
+// compiler can neither move its reads of the value above the block nor hand out the registers
+// before it (keep_v).
+__device__ __forceinline__ void pin_v(f16v& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin_a(f16v& x) { asm volatile("" : "+a"(x)); }
+__device__ __forceinline__ void keep_v(const f16v& x) { asm volatile("" : : "v"(x)); }
 // The vector side of the main loop, as volatile blocks so that it stays where it is written,
 // interleaved with the matrix instructions.
 __device__ __forceinline__ void v_fma(float& r, float x, float y, float z) { asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z)); }
@@ -126,6 +121,10 @@ __device__ __forceinline__ void v_cvt_pk(unsigned& r, float lo, float hi) { // t
 }
 __device__ __forceinline__ void v_max2(float& r, float x, float y) { asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y)); }
 __device__ __forceinline__ void v_max3_acc(float& r, float x, float y) { asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(r) : "v"(x), "v"(y)); }
+// acc += p.lo * q.lo + p.hi * q.hi (packed fp16 factors, fp32 sum)
+__device__ __forceinline__ void v_dot2_acc(float& acc, unsigned p, unsigned q) {
+    asm volatile("v_dot2_f32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(p), "v"(q));
+}
 
 // maxima without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
 // for results that feed a lane-swap instruction, which must not read a register in the cycle
@@ -140,11 +139,14 @@ __device__ __forceinline__ float max2(float x, float y) {
     asm("v_max_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(x), "v"(y));
     return r;
 }
-__device__ __forceinline__ float xor_max_fast(float v) { // all-reduce over lanes l, l^16, l^32, l^48; inputs never NaN
-    u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    float r = max2(__uint_as_float(s.x), __uint_as_float(s.y));
-    s = __builtin_amdgcn_permlane16_swap(__float_as_uint(r), __float_as_uint(r), false, false);
+// The two lanes that hold a column's rows are l and l ^ 32: maximum / sum over the pair.
+__device__ __forceinline__ float pair_max(float v) {
+    const u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return max2(__uint_as_float(s.x), __uint_as_float(s.y));
+}
+__device__ __forceinline__ float pair_sum(float v) {
+    const u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(s.x) + __uint_as_float(s.y);
 }
 
 // Buffer descriptor words for the global->LDS copies below: base address, stride 0, byte
@@ -184,39 +186,71 @@ __device__ __forceinline__ void reg_load16(u32x4& dst, i32x4 desc, int off, int 
 }
 
 // One such copy, for the main loop, which deals them out between the matrix instructions so
-// that the vector-memory issue queue never backs up.
+// that the vector-memory issue queue never backs up.  The LDS base is whatever set_lds_base()
+// put into M0 last: nothing else in the loop touches that register (the compiler has no reason
+// to -- it generates no LDS-directed loads, relative moves or lane reads of its own there).
+__device__ __forceinline__ void set_lds_base(unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0" : : "s"(lds_base) : "memory", "m0");
+}
 template <int IMM>
-__device__ __forceinline__ void lds_copy_1k(i32x4 desc, unsigned lds_base, int off, int soff) {
-    asm volatile(
-        "s_mov_b32 m0, %0\n\t"
-        "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
-        :
-        : "s"(lds_base), "v"(off), "s"(desc), "s"(soff), "n"(IMM)
-        : "memory", "m0");
+__device__ __forceinline__ void lds_copy_1k(i32x4 desc, int off, int soff) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds" : : "v"(off), "s"(desc), "s"(soff), "n"(IMM) : "memory", "m0");
 }
 
-template <int D, int NQB, int TQ>
+// The vector instructions of stage B for one 32x32 score block (16 scores per lane), in issue
+// order.  Pair p = scores (2p, 2p+1).  Kinds: 0 multiply-add (the exponent), 1 exponential,
+// 2 conversion of a pair to packed fp16, 3 row-sum update from a packed pair.  The four kinds run
+// as a software pipeline one pair apart, so no instruction reads a result younger than three
+// instructions.
+struct ItemTable {
+    int kind[48];
+    int arg[48];
+};
+constexpr ItemTable make_items() {
+    ItemTable t{};
+    int n = 0;
+    for (int p = 0; p < 11; ++p) {
+        if (p < 8) {
+            t.kind[n] = 0; t.arg[n++] = 2 * p;
+            t.kind[n] = 0; t.arg[n++] = 2 * p + 1;
+        }
+        if (p >= 1 && p <= 8) {
+            t.kind[n] = 1; t.arg[n++] = 2 * p - 2;
+            t.kind[n] = 1; t.arg[n++] = 2 * p - 1;
+        }
+        if (p >= 2 && p <= 9) {
+            t.kind[n] = 2; t.arg[n++] = p - 2;
+        }
+        if (p >= 3) {
+            t.kind[n] = 3; t.arg[n++] = p - 3;
+        }
+    }
+    return t;
+}
+constexpr ItemTable kItemsOfBlock = make_items();
+constexpr int kItemsPerBlock = 48;
+
+template <int D, int NCB>
 __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const FaArgs a) {
-    using G = PGeom<D, NQB>;
+    using G = PGeom<D, NCB>;
     constexpr int kWaves = kPrefillWaves;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     FA_STAMP(0);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: tile indices live in scalar registers
-    const int col = lane & 15;
-    const int grp = lane >> 4;
+    const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
+    const int hh = lane >> 5;  // lane-half: 8-wide k slice of an operand, rows 8q + 4*hh + 0..3 of an accumulator
 
     int id = blockIdx.x;
     const int kvh = id % a.n_kv;
     id /= a.n_kv;
     const int hg = id % a.n_hgroups;
     id /= a.n_hgroups;
-    const int n_past = a.n_past, batch = a.batch;
-    const int t0 = (a.n_ttiles - 1 - id) * TQ; // longest rows first
-    constexpr int kHeadsPerGroup = NQB * 16 / TQ;
-    const int head_lo = hg * kHeadsPerGroup;
-    const int tok_hi = (t0 + TQ < batch) ? t0 + TQ : batch;
+    const int n_past = a.n_past, batch = a.batch, tq = a.tq;
+    const int t0 = (a.n_ttiles - 1 - id) * tq; // longest rows first
+    const int head_lo = hg * a.heads_per_group;
+    const int tok_hi = (t0 + tq < batch) ? t0 + tq : batch;
     const int kv_end = n_past + tok_hi;   // the workgroup's columns see rows [0, kv_end) at most
     const int full_end = n_past + t0 + 1; // rows below this are visible to every column
     const int n_tiles = (kv_end + kTile - 1) / kTile;
@@ -224,6 +258,12 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // end map to negative tiles, whose copies fetch nothing.
     const int n_mine = n_tiles > wave ? (n_tiles - 1 - wave) / kWaves + 1 : 0;
     auto tile_of = [&](int j) { return wave + kWaves * (n_mine - 1 - j); };
+    // column c of the block -> (token, head of the group); columns past the group's heads are padding
+    auto col_valid = [&](int c, int& tok, int& hl) {
+        tok = t0 + c % tq;
+        hl = head_lo + c / tq;
+        return c / tq < a.heads_per_group && hl < a.r && tok < batch;
+    };
 
     unsigned char* const ws = smem + wave * G::kWaveB; // this wave's LDS slice
     const unsigned ws_addr = __builtin_amdgcn_readfirstlane(
@@ -244,19 +284,23 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         }
     }
     constexpr int kOdd = (G::kRowsPerCopy == 4) ? 1 : 0;
-    // K operand read: lane (col, grp) takes row t*16 + col, logical chunk kk*4 + grp.  The
-    // pointers carry every per-lane term; buffer parity and sub-tile are immediate offsets.
+    // K operand read: lane (c32, hh) takes row c32, logical chunk ks*2 + hh.  The pointers carry
+    // every per-lane term; the buffer parity is an immediate offset.
     const unsigned char* kp[G::kSteps];
 #pragma unroll
-    for (int kk = 0; kk < G::kSteps; ++kk) kp[kk] = ws + G::kKOff + col * G::kRowB + (((kk * 4 + grp) ^ (col & 7)) * 16);
-    // V transposing read: lane (col, grp) addresses row grp*4 + col/4 (+16 for the second half),
-    // 8-byte column db*4 + col%4.
+    for (int ks = 0; ks < G::kSteps; ++ks) kp[ks] = ws + G::kKOff + c32 * G::kRowB + (((ks * 2 + hh) ^ (c32 & 7)) * 16);
+    // V transposing read, per 16-lane group (lane i of the group): addresses row R + i/4, 8-byte
+    // column (d0/4 + i%4) and receives rows R..R+3 at head_dim index d0 + i, where d0 = db*32 +
+    // 16 * (lane/16 % 2) and R = 16*kh + 4*hh (+8 for the second half of the operand): the
+    // operand's k index (hh, j) is KV row 16*kh + 8*(j/4) + 4*hh + j%4, the row that score
+    // register 8*kh + j of lane-half hh belongs to.
     const unsigned char* vp[G::kDBlk];
     {
-        const int r0 = grp * 4 + (col >> 2), sw = r0 & 7;
+        const int i16 = lane & 15, g2 = (lane >> 4) & 1;
+        const int r0 = 4 * hh + (i16 >> 2), sw = r0 & 7;
 #pragma unroll
         for (int db = 0; db < G::kDBlk; ++db)
-            vp[db] = ws + G::kVOff + r0 * G::kRowB + (((db * 2 + ((col & 3) >> 1)) ^ sw) * 16) + (col & 1) * 8;
+            vp[db] = ws + G::kVOff + r0 * G::kRowB + (((db * 4 + g2 * 2 + ((i16 & 3) >> 1)) ^ sw) * 16) + (i16 & 1) * 8;
     }
 
     // Prologue copies: the whole offset is in the (range-checked) vector operand, so rows at or
@@ -268,38 +312,26 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     };
     // Main-loop copies: every tile they name is either wholly inside the visible range, and its
     // base travels as the scalar offset, or below zero, and then the descriptor is emptied.
-    auto copy_fast = [&](const i32x4& desc, unsigned lds_dst, int tile) {
-        const bool live = tile >= 0;
-        const i32x4 d = i32x4{desc[0], desc[1], live ? desc[2] : 0, desc[3]};
-        const int soff = live ? tile * G::kTileB : 0;
-        lds_copy_4k(d, lds_dst, g_off[0], g_off[kOdd], soff);
-        if (G::kCopies > 4) lds_copy_4k(d, lds_dst + 4096, g_off[0], g_off[kOdd], soff + 4096);
-    };
-    // Copy number i (of kCopies) of a main-loop tile; desc and soff as prepared by live_desc / tile_soff.
     auto live_desc = [&](const i32x4& desc, int tile) { return i32x4{desc[0], desc[1], tile >= 0 ? desc[2] : 0, desc[3]}; };
     auto tile_soff = [&](int tile) { return tile >= 0 ? tile * G::kTileB : 0; };
-    auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) {
+    auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
-        lds_copy_1k<sub * 1024>(d, lds_dst + half * 4096, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
+        if constexpr (sub == 0) set_lds_base(lds_dst + half * 4096);
+        lds_copy_1k<sub * 1024>(d, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
     };
     auto k_buf = [&](int par) { return ws_addr + G::kKOff + par * G::kTileB; };
     auto v_buf = [&](int par) { return ws_addr + G::kVOff + par * G::kTileB; };
 
     // ---- state ----
-    h8 q[NQB][G::kSteps]; // B operands of A: the query columns, fp16
-    float nb[NQB];        // each column's exponent offset: shift - reference maximum * c (log2 units)
-    f4 o[NQB][G::kDBlk];  // O^T accumulators (accumulation registers)
-    f4 lacc[NQB];         // row sums: every element of a lane's four holds the column's sum
-    f4 s[2][2][NQB];      // scores: [parity][sub-tile][query block]
-    u32x4 pw[2][NQB];     // P as packed fp16: [parity][query block]
-    h8 ones;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
-    asm volatile("" : "+v"(ones)); // stays in registers; never rematerialised in front of a matrix instruction
-
-    const unsigned scratch_addr = ws_addr + G::kScratchOff + lane * 16;
-    float* const scratch = reinterpret_cast<float*>(ws + G::kScratchOff) + lane * 4;
+    h8 q[NCB][G::kSteps];   // B operands of A: the query columns, fp16
+    float nb[NCB];          // each column's exponent offset: shift - reference maximum * c (log2 units)
+    float lsum[NCB];        // this lane's share (16 of a tile's 32 rows) of the column's row sum
+    f16v o[NCB][G::kDBlk];  // O^T accumulators (accumulation registers)
+    f16v s[2][NCB];         // scores: [parity][column block]
+    u32x4 pw[2][NCB][2];    // P as packed fp16: [parity][column block][k-step of C]
+    unsigned ones_pk = 0x3c003c00u;
+    asm volatile("" : "+v"(ones_pk)); // stays in a register; never rematerialised between the hand-placed instructions
 
     // ---- prologue loads, most urgent first: the query block, then the first K tile; the rest of
     // the first two tiles follows once the queries are on their way into LDS.  All of them are
@@ -308,8 +340,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // The query block is loaded once per workgroup: wave w takes a quarter of the columns with
     // coalesced 16-byte loads (a column is D/4 lanes wide), converts to fp16 and leaves it in LDS;
     // after the barrier every wave picks up its B operands from there. ----
-    constexpr int kColsPerLoad = 256 / D;              // columns one load instruction covers
-    constexpr int kQLoads = NQB * 4 / kColsPerLoad;    // load instructions per wave
+    constexpr int kColsPerLoad = 256 / D;                 // columns one load instruction covers
+    constexpr int kQLoads = G::kCols / 4 / kColsPerLoad;  // load instructions per wave
     u32x4 qraw[kQLoads];
     float qmul[kQLoads];
     int qcol[kQLoads];
@@ -317,10 +349,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         const i32x4 qdesc = make_desc(a.q, (unsigned)batch * a.n_head * D * 4);
         static_for<0, kQLoads>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const int c = wave * (NQB * 4) + j * kColsPerLoad + lane / (D / 4);
-            const int tok = t0 + c % TQ;
-            const int hl = head_lo + c / TQ;
-            const bool valid = (hl < a.r) && (tok < batch);
+            const int c = wave * (G::kCols / 4) + j * kColsPerLoad + lane / (D / 4);
+            int tok, hl;
+            const bool valid = col_valid(c, tok, hl);
             qcol[j] = c;
             qmul[j] = valid ? a.qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
             const int q_off = valid ? ((tok * a.n_head + kvh * a.r + hl) * D + (lane % (D / 4)) * 4) * 4 : 0;
@@ -329,18 +360,19 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     }
     if (n_mine > 0) copy_checked(kdesc, k_buf(0), tile_of(0));
     FA_STAMP(9);
-    // O = 0, l = 0: a matrix instruction with a zero addend writes the accumulation registers
-    // without touching memory.
+    // O = 0: a matrix instruction with a zero addend writes the accumulation registers without
+    // touching memory.
     {
         h8 zero;
 #pragma unroll
         for (int e = 0; e < 8; ++e) zero[e] = (_Float16)0.0f;
         asm volatile("" : "+v"(zero));
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
+        for (int cb = 0; cb < NCB; ++cb) {
+            lsum[cb] = 0.0f;
+            nb[cb] = 0.0f;
 #pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db) mfma_a_zero_n(o[qb][db], zero, zero);
-            mfma_a_zero_n(lacc[qb], zero, zero);
+            for (int db = 0; db < G::kDBlk; ++db) mfma_o_zero_n(o[cb][db], zero, zero);
         }
     }
     if (n_mine > 0) {
@@ -365,19 +397,17 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     if (n_mine > 0) {
         copy_checked(vdesc, v_buf(0), tile_of(0));
         copy_checked(kdesc, k_buf(1), tile_of(1));
-        copy_checked(vdesc, v_buf(1), tile_of(1));
     }
-    int limit[NQB];
+    int limit[NCB];
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-        const int c = qb * 16 + col;
-        const int tok = t0 + c % TQ;
-        const int hl = head_lo + c / TQ;
-        limit[qb] = (hl < a.r) && (tok < batch) ? n_past + tok + 1 : 0x7fffffff;
+    for (int cb = 0; cb < NCB; ++cb) {
+        const int c = cb * 32 + c32;
+        int tok, hl;
+        limit[cb] = col_valid(c, tok, hl) ? n_past + tok + 1 : 0x7fffffff;
 #pragma unroll
-        for (int kk = 0; kk < G::kSteps; ++kk) {
-            const h8 hv = *reinterpret_cast<const h8*>(smem + G::kQOff + c * G::kQStride + (kk * 32 + grp * 8) * 2);
-            asm volatile("" : "=a"(q[qb][kk]) : "0"(hv)); // parked in the accumulation-register file for good
+        for (int ks = 0; ks < G::kSteps; ++ks) {
+            const h8 hv = *reinterpret_cast<const h8*>(smem + G::kQOff + c * G::kQStride + (ks * 16 + hh * 8) * 2);
+            asm volatile("" : "=a"(q[cb][ks]) : "0"(hv)); // parked in the accumulation-register file for good
         }
     }
     FA_STAMP(1);
@@ -396,252 +426,256 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         // Prologue form of A: S[spar] = K[kpar] Q^T with a zero addend, operands read up front.
         auto stage_a0 = [&](auto kpar, auto spar) {
             constexpr int KP = decltype(kpar)::value, SP = decltype(spar)::value;
-            h8 ka[G::kSteps][2];
+            h8 ka[G::kSteps];
 #pragma unroll
-            for (int kk = 0; kk < G::kSteps; ++kk)
+            for (int ks = 0; ks < G::kSteps; ++ks) ka[ks] = *reinterpret_cast<const h8*>(kp[ks] + KP * G::kTileB);
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    ka[kk][t] = *reinterpret_cast<const h8*>(kp[kk] + KP * G::kTileB + t * 16 * G::kRowB);
+            for (int ks = 0; ks < G::kSteps; ++ks)
 #pragma unroll
-            for (int kk = 0; kk < G::kSteps; ++kk)
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int qb = 0; qb < NQB; ++qb) {
-                        if (kk == 0) mfma_v_zero_n(s[SP][t][qb], ka[kk][t], q[qb][kk]);
-                        else mfma_v_n(s[SP][t][qb], ka[kk][t], q[qb][kk]);
-                        // With few query blocks the next k-step of the same accumulator is only a
-                        // couple of instructions away; give the result time to leave the pipe.
-                        if (2 * NQB < 8) asm volatile("s_nop 15");
-                    }
+                for (int cb = 0; cb < NCB; ++cb) {
+                    if (ks == 0) mfma_s_zero_n(s[SP][cb], ka[ks], q[cb][ks]);
+                    else mfma_s_n(s[SP][cb], ka[ks], q[cb][ks]);
+                }
         };
-        // Copy issue order: K0 V0 K1 V1 | K2 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
-        // (within a step, K goes out over the first tickets and V over the last)
+        // Copy issue order: K0 V0 K1 | K2 V1 (step 0) | K3 V2 (step 1) | K4 V3 (step 2) | ...
+        // (within a step, K goes out over the first half of the tickets and V over the second)
         // ---- step 0: the diagonal tile, the only one that can need the causal mask ----
-        wait_copies(IntC<3 * kC>{});        // K0 landed (V0 K1 V1 may be in flight)
+        wait_copies(IntC<2 * kC>{});        // K0 landed (V0 K1 may be in flight)
         stage_a0(IntC<0>{}, IntC<0>{});     // S(0)
         __builtin_amdgcn_s_waitcnt(0xC07F); // its LDS reads have returned: K buffer 0 is free
-        copy_fast(kdesc, k_buf(0), tile_of(2));
-        if (R > 0) {
-            wait_copies(IntC<2 * kC>{});    // K1 landed (V1 K2 may be in flight)
-            stage_a0(IntC<1>{}, IntC<1>{}); // S(1)
+        {
+            const i32x4 kd = live_desc(kdesc, tile_of(2));
+            const int ksoff = tile_soff(tile_of(2));
+            static_for<0, kC>([&](auto ic) { copy_one(ic, kd, k_buf(0), ksoff); });
+            copy_checked(vdesc, v_buf(1), tile_of(1));
         }
+        wait_copies(IntC<2 * kC>{});        // K1 and V0 landed (K2 V1 may be in flight)
+        if (R > 0) stage_a0(IntC<1>{}, IntC<1>{}); // S(1)
         settle();
         FA_STAMP(2);
         // Reference maximum of each column: over its visible scores of tile 0 and, when there is
         // one, tile 1 (every row of which is visible to every column).  A column with no visible
         // row in this wave keeps weight zero whatever the reference.
         {
-            const int row0 = tile_of(0) * kTile + grp * 4;
+            const int row0 = tile_of(0) * kTile + 4 * hh;
             const bool masked = tile_of(0) * kTile + kTile > full_end;
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) {
-                float v[8];
+            for (int cb = 0; cb < NCB; ++cb) {
+                pin_v(s[0][cb]); // (the reads below stay behind the settled pipe)
+                if (R > 0) pin_v(s[1][cb]);
+                float v[16];
+                float mx = -INFINITY;
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        v[t * 4 + i] = s[0][t][qb][i];
-                        if (masked && row0 + t * 16 + i >= limit[qb]) v[t * 4 + i] = -INFINITY;
-                    }
-                float mx = max3(v[0], v[1], v[2]);
-                mx = max3(mx, v[3], v[4]);
-                mx = max3(mx, v[5], v[6]);
-                mx = max2(mx, v[7]);
-                if (R > 0) {
-                    mx = max3(mx, s[1][0][qb][0], s[1][0][qb][1]);
-                    mx = max3(mx, s[1][0][qb][2], s[1][0][qb][3]);
-                    mx = max3(mx, s[1][1][qb][0], s[1][1][qb][1]);
-                    mx = max3(mx, s[1][1][qb][2], s[1][1][qb][3]);
-                    mx = max2(mx, mx);
+                for (int r = 0; r < 16; ++r) {
+                    v[r] = s[0][cb][r];
+                    if (masked && row0 + 8 * (r / 4) + (r % 4) >= limit[cb]) v[r] = -INFINITY;
+                    mx = fmaxf(mx, v[r]);
                 }
-                mx = xor_max_fast(mx);
-                nb[qb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
-                h8 ph;
+                if (R > 0) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) ph[e] = (_Float16)fast_exp2(__builtin_fmaf(v[e], a.c, nb[qb]));
-                pw[0][qb] = __builtin_bit_cast(u32x4, ph);
+                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][cb][r]);
+                }
+                mx = pair_max(mx);
+                nb[cb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
+                float sum = 0.0f;
+#pragma unroll
+                for (int kh = 0; kh < 2; ++kh) {
+                    h8 ph;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        ph[j] = (_Float16)fast_exp2(__builtin_fmaf(v[kh * 8 + j], a.c, nb[cb]));
+                        sum += (float)ph[j];
+                    }
+                    pw[0][cb][kh] = __builtin_bit_cast(u32x4, ph);
+                }
+                lsum[cb] = sum;
             }
         }
         settle(); // (the vector writes of P are well clear of the next matrix instruction)
         FA_STAMP(3);
 
         // ---- steps t >= 1: A(t+1), B(t) and C(t-1) in one instruction stream.  The matrix
-        // instructions are cut into groups of NQB that share an LDS operand (A: one (k-step,
-        // sub-tile) of K; C: one 16-wide block of V^T; last, the row sums), ordered A0 C0 A1 C1
-        // ... L; the 24 vector instructions per query block of B are dealt out evenly between
-        // them.  Operands are read from LDS kAhead groups ahead of their use.
-        // `newer` = copies issued after K(t+1) and before the wait: none at t == 1 (step 0 issued
-        // K(2) last), V(t) afterwards. ----
-        static_assert(2 * G::kSteps == G::kDBlk, "A and C groups alternate one to one");
-        constexpr int kGroups = 2 * G::kSteps + G::kDBlk; // groups with an LDS operand
-        constexpr int kTickets = (kGroups + 1) * NQB;     // matrix instructions per step
-        constexpr int kItems = 24 * NQB;                  // vector instructions of B per step
-        constexpr int kAhead = 3;
-        constexpr float kBound = kLazy + kPShift;         // largest exponent P may be built from
-        constexpr float kBoundP = 32768.0f;               // = 2^kBound
-        // (The last step has no tile t+1: its A stage multiplies whatever the K buffer holds and
-        // nobody reads the result -- cheaper than a second copy of the loop body without it.)
+        // instructions are cut into groups of NCB that share an LDS operand -- C: one 32-wide block
+        // of V^T for one half of the tile's rows, A: one k-step of K -- with all of C first: the V
+        // buffer C reads is then free for the copy of V(t+1) from the middle of the step, and
+        // both copies (K(t+2) over the first half, V(t+1) over the second) have more than a step
+        // to land, so neither wait in the step ever stalls.  The 48 vector instructions per
+        // column block of B are dealt out evenly between the matrix instructions.  Operands are
+        // read from LDS kAhead groups ahead of their use, across the end of the step too: the
+        // first groups' operands arrive in `carry`, read during the previous step. ----
+        constexpr int kCG = 2 * G::kDBlk;             // groups of C
+        constexpr int kGroups = kCG + G::kSteps;      // groups of matrix instructions per step
+        constexpr int kTickets = kGroups * NCB;       // matrix instructions per step
+        constexpr int kHalf = kCG * NCB;              // tickets of C
+        constexpr int kItems = kItemsPerBlock * NCB;  // vector instructions of B per step
+        constexpr int kAhead = NCB == 2 ? 3 : 4;
+        static_assert(kAhead <= kCG && kAhead <= G::kSteps, "the reads carried over a step boundary are reads of V");
+        static_assert(kHalf == kC * NCB && kTickets - kHalf == kC * NCB, "one copy every NCB tickets");
+        constexpr float kBound = 15.0f;               // a column whose largest exponent is above this is moved
         float c = a.c;
         asm volatile("" : "+v"(c)); // a vector register for the whole loop, not a move per step
-        auto body = [&](auto tpar, auto newer, int t) {
+        h8 carry[kAhead];
+        // The V operand of C group g (block g % kDBlk of head_dim, half g / kDBlk of the tile's rows).
+        auto read_v = [&](auto gc, int par_off) {
+            constexpr int g = decltype(gc)::value;
+            constexpr int db = g % G::kDBlk, kh = g / G::kDBlk;
+            const h4 v0 = lds_read_tr(vp[db] + par_off + kh * 16 * G::kRowB);
+            const h4 v1 = lds_read_tr(vp[db] + par_off + (kh * 16 + 8) * G::kRowB);
+            return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        static_for<0, kAhead>([&](auto gc) { carry[decltype(gc)::value] = read_v(gc, 0); }); // for step 1: V(0)
+        // (The last step has no tile t+1: its A stage multiplies whatever the K buffer holds and
+        // nobody reads the result -- cheaper than a second copy of the loop body without it.)
+        auto body = [&](auto tpar, int t) {
             constexpr int TP = decltype(tpar)::value; // t & 1
-            // (Every LDS read of the previous step has been consumed by a matrix instruction that
-            // was issued before this point, so the K buffer A(t) read is free.)
-            // K(t+2) goes to the buffer A(t) read; its copies are dealt out over the first tickets.
-            // (Issued after this step's wait, they are not among the `newer` copies any more.)
+            // K(t+2) goes to the buffer A(t) read, V(t+1) to the buffer C(t-1) reads in the first half of this step.
             const i32x4 kd = live_desc(kdesc, tile_of(t + 2));
             const int ksoff = tile_soff(tile_of(t + 2));
             const i32x4 vd = live_desc(vdesc, tile_of(t + 1));
             const int vsoff = tile_soff(tile_of(t + 1));
-            wait_copies(newer);                          // K(t+1) landed; V(t-1) is older
             h8 gop[kGroups];
-            auto issue_read = [&](auto gc) {
-                constexpr int g = decltype(gc)::value;
+            static_for<0, kAhead>([&](auto gc) { gop[decltype(gc)::value] = carry[decltype(gc)::value]; });
+            // Issue order of the copies is ... K(t+1) V(t) | K(t+2) V(t+1): a wait that leaves the
+            // copies issued since outstanding guarantees the older tile.  T = the ticket about to issue.
+            auto issue_read = [&](auto gc, auto tc) {
+                constexpr int g = decltype(gc)::value, T = decltype(tc)::value;
+                constexpr int k_issued = T / NCB < kC ? T / NCB : kC;
+                constexpr int v_issued = T < kHalf ? 0 : ((T - kHalf) / NCB < kC ? (T - kHalf) / NCB : kC);
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (g % 2 == 0) {
-                    constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
-                    gop[g] = *reinterpret_cast<const h8*>(kp[kk] + (TP ^ 1) * G::kTileB + tt * 16 * G::kRowB);
-                } else {
-                    constexpr int db = g / 2;
-                    const h4 v0 = lds_read_tr(vp[db] + (TP ^ 1) * G::kTileB);
-                    const h4 v1 = lds_read_tr(vp[db] + (TP ^ 1) * G::kTileB + 16 * G::kRowB);
-                    gop[g] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
+                if constexpr (g == kCG) wait_copies(IntC<kC + k_issued>{});           // K(t+1) landed
+                if constexpr (g == kGroups) wait_copies(IntC<k_issued + v_issued>{}); // V(t) landed
+                if constexpr (g < kCG) gop[g] = read_v(gc, (TP ^ 1) * G::kTileB);
+                else if constexpr (g < kGroups) gop[g] = *reinterpret_cast<const h8*>(kp[g - kCG] + (TP ^ 1) * G::kTileB);
+                else carry[g - kGroups] = read_v(IntC<g - kGroups>{}, TP * G::kTileB);     // for C(t) of the next step
                 __builtin_amdgcn_sched_barrier(0);
             };
-            float pe[NQB][8];
-            float amax;
-            // Vector instruction j of B(t).  Per query block and pair of scores: two multiply-adds
-            // (the exponents), two exponentials, the running maximum of the weights, the conversion;
-            // no instruction reads the result of the one right before it.
+            float pe[NCB][16];
+            float l_before[NCB]; // the row sums without this tile, for the slow path
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) l_before[cb] = lsum[cb];
+            // Vector instruction j of B(t) (see ItemTable).
             auto item = [&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                constexpr int qb = j / 24, r = j % 24;
-                // 0 multiply-add, 1 maximum, 2 exponential, 3 conversion
-                constexpr int kind[24] = {0, 0, 2, 2, 0, 0, 1, 2, 2, 3, 0, 0, 1, 2, 2, 3, 0, 0, 1, 2, 2, 3, 1, 3};
-                constexpr int arg[24] = {0, 1, 0, 1, 2, 3, 0, 2, 3, 0, 4, 5, 1, 4, 5, 1, 6, 7, 2, 6, 7, 2, 3, 3};
-                constexpr int x = arg[r];
-                if constexpr (kind[r] == 0) {
-                    v_fma(pe[qb][x], s[TP][x / 4][qb][x % 4], c, nb[qb]);
-                } else if constexpr (kind[r] == 2) {
-                    v_exp2(pe[qb][x]);
-                } else if constexpr (kind[r] == 3) {
+                constexpr int cb = j / kItemsPerBlock, r = j % kItemsPerBlock;
+                constexpr int kind = kItemsOfBlock.kind[r], x = kItemsOfBlock.arg[r];
+                if constexpr (kind == 0) {
+                    v_fma(pe[cb][x], s[TP][cb][x], c, nb[cb]);
+                } else if constexpr (kind == 1) {
+                    v_exp2(pe[cb][x]);
+                } else if constexpr (kind == 2) {
                     unsigned packed;
-                    v_cvt_pk(packed, pe[qb][2 * x], pe[qb][2 * x + 1]);
-                    pw[TP][qb][x] = packed;
+                    v_cvt_pk(packed, pe[cb][2 * x], pe[cb][2 * x + 1]);
+                    pw[TP][cb][x / 4][x % 4] = packed;
                 } else {
-                    if constexpr (j == 6) v_max2(amax, pe[qb][2 * x], pe[qb][2 * x + 1]);
-                    else v_max3_acc(amax, pe[qb][2 * x], pe[qb][2 * x + 1]);
+                    v_dot2_acc(lsum[cb], pw[TP][cb][x / 4][x % 4], ones_pk);
                 }
             };
-            static_for<0, kAhead>(issue_read);
             static_for<0, kTickets>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                constexpr int g = i / NQB, m = i % NQB;
-                if constexpr (m == 0 && g + kAhead < kGroups) issue_read(IntC<g + kAhead>{});
-                if constexpr (g == kGroups) {
-                    mfma_a(lacc[m], ones, __builtin_bit_cast(h8, pw[TP ^ 1][m]));
-                } else if constexpr (g % 2 == 0) {
-                    constexpr int kk = (g / 2) / 2, tt = (g / 2) % 2;
-                    if constexpr (kk == 0) mfma_v_zero(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
-                    else mfma_v(s[TP ^ 1][tt][m], gop[g], q[m][kk]);
+                constexpr int g = i / NCB, m = i % NCB;
+                if constexpr (m == 0) issue_read(IntC<g + kAhead>{}, ic);
+                if constexpr (g < kCG) {
+                    constexpr int db = g % G::kDBlk, kh = g / G::kDBlk;
+                    mfma_o(o[m][db], gop[g], __builtin_bit_cast(h8, pw[TP ^ 1][m][kh]));
                 } else {
-                    mfma_a(o[m][g / 2], gop[g], __builtin_bit_cast(h8, pw[TP ^ 1][m]));
+                    constexpr int ks = g - kCG;
+                    if constexpr (ks == 0) mfma_s_zero(s[TP ^ 1][m], gop[g], q[m][ks]);
+                    else mfma_s(s[TP ^ 1][m], gop[g], q[m][ks]);
                 }
                 static_for<(i * kItems) / kTickets, ((i + 1) * kItems) / kTickets>(item);
-                if constexpr (i % 2 == 1 && i / 2 < kC) copy_one(IntC<i / 2>{}, kd, k_buf(TP), ksoff);
-                // V(t+1) goes to the buffer C(t-1) reads: its copies wait for the last of those reads
-                // to be consumed, which the row-sum group (no LDS operand) marks.
-                if constexpr (g == kGroups) {
-                    constexpr int per = (kC + NQB - 1) / NQB;
-                    static_for<m * per, (m + 1) * per < kC ? (m + 1) * per : kC>([&](auto cc) { copy_one(cc, vd, v_buf(TP ^ 1), vsoff); });
+                if constexpr (m == NCB - 1) {
+                    if constexpr (i < kHalf) copy_one(IntC<i / NCB>{}, kd, k_buf(TP), ksoff);
+                    else copy_one(IntC<(i - kHalf) / NCB>{}, vd, v_buf(TP ^ 1), vsoff);
                 }
             });
             // S(t+1) is alive to the end of the step even when nobody reads it (last step): its
             // registers must not be handed out while the matrix instructions that write them are in flight.
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) {
-                asm volatile("" : : "v"(s[TP ^ 1][0][qb]));
-                asm volatile("" : : "v"(s[TP ^ 1][1][qb]));
-            }
-            // ---- slow path: some exponent of this tile is above the bound.  Move the reference of
-            // the columns concerned to their new maximum, redo P(t) and rescale O and l -- one
-            // accumulator at a time through a 16-byte-per-lane LDS scratch, so that they never
-            // become operands of a vector instruction. ----
-            if (__builtin_amdgcn_ballot_w64(amax > kBoundP) != 0) {
+            for (int cb = 0; cb < NCB; ++cb) keep_v(s[TP ^ 1][cb]);
+            // ---- slow path: a weight of this tile overflowed fp16 (the row sum, which adds up the
+            // rounded weights, is then infinite).  Move the reference of the columns concerned to
+            // their new maximum, redo P(t) and rescale O and l. ----
+            bool over = false;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) over |= !(lsum[cb] < 3.0e38f);
+            if (__builtin_amdgcn_ballot_w64(over) != 0) {
                 settle(); // C(t-1) has left the matrix pipe
-                float alpha[NQB];
 #pragma unroll
-                for (int qb = 0; qb < NQB; ++qb) {
-                    float mx = max3(s[TP][0][qb][0], s[TP][0][qb][1], s[TP][0][qb][2]);
-                    mx = max3(mx, s[TP][0][qb][3], s[TP][1][qb][0]);
-                    mx = max3(mx, s[TP][1][qb][1], s[TP][1][qb][2]);
-                    mx = xor_max_fast(max2(mx, s[TP][1][qb][3]));
-                    const float top = __builtin_fmaf(mx, c, nb[qb]); // the column's largest exponent
+                for (int cb = 0; cb < NCB; ++cb) {
+                    float mx = s[TP][cb][0];
+#pragma unroll
+                    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[TP][cb][r]);
+                    mx = pair_max(mx);
+                    const float top = __builtin_fmaf(mx, c, nb[cb]); // the column's largest exponent
                     const float delta = top > kBound ? top - kPShift : 0.0f;
-                    alpha[qb] = fast_exp2(-delta);
-                    nb[qb] -= delta;
-                    h8 ph;
+                    const float alpha = fast_exp2(-delta);
+                    nb[cb] -= delta;
+                    // l: this tile's share was added under the old offset and may have overflowed:
+                    // start again from the sum before this step
+                    float new_sum = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) ph[e] = (_Float16)fast_exp2(__builtin_fmaf(s[TP][e / 4][qb][e % 4], c, nb[qb]));
-                    pw[TP][qb] = __builtin_bit_cast(u32x4, ph);
+                    for (int kh = 0; kh < 2; ++kh) {
+                        h8 ph;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            ph[j] = (_Float16)fast_exp2(__builtin_fmaf(s[TP][cb][kh * 8 + j], c, nb[cb]));
+                            new_sum += (float)ph[j];
+                        }
+                        pw[TP][cb][kh] = __builtin_bit_cast(u32x4, ph);
+                    }
+                    lsum[cb] = l_before[cb] * alpha + new_sum;
+#pragma unroll
+                    for (int db = 0; db < G::kDBlk; ++db) {
+                        pin_a(o[cb][db]); // the reads below stay behind the settled pipe
+                        o[cb][db] *= alpha;
+                        pin_a(o[cb][db]);
+                    }
                 }
-                auto scale_acc = [&](f4& acc, float al) {
-                    lds_store_acc(scratch_addr, acc);
-                    f4 x = *reinterpret_cast<f4*>(scratch);
-                    x *= al;
-                    *reinterpret_cast<f4*>(scratch) = x;
-                    lds_load_acc(acc, scratch_addr);
-                };
-                static_for<0, NQB>([&](auto qbc) {
-                    constexpr int qb = decltype(qbc)::value;
-                    static_for<0, G::kDBlk>([&](auto dbc) { scale_acc(o[qb][decltype(dbc)::value], alpha[qb]); });
-                    scale_acc(lacc[qb], alpha[qb]);
-                });
                 settle();
             }
         };
-        if (R >= 1) body(IntC<1>{}, IntC<0>{}, 1);
+        if (R >= 1) body(IntC<1>{}, 1);
         int t = 2;
         for (; t + 1 <= R; t += 2) {
-            body(IntC<0>{}, IntC<kC>{}, t);
-            body(IntC<1>{}, IntC<kC>{}, t + 1);
+            body(IntC<0>{}, t);
+            body(IntC<1>{}, t + 1);
         }
-        if (t == R) body(IntC<0>{}, IntC<kC>{}, t);
+        if (t == R) body(IntC<0>{}, t);
         FA_STAMP(4);
         // ---- drain: C(R) ----
         wait_copies(IntC<0>{});
         settle(); // P(R) was converted just above
-        {   // O += V(R)^T P(R), l += 1^T P(R); both live in the buffers of parity R & 1
+        {   // O += V(R)^T P(R); both live in the buffers of parity R & 1
             const bool odd = (R & 1) != 0;
             const int v_par = odd ? G::kTileB : 0;
-            h8 va[G::kDBlk], pl[NQB];
+            h8 va[2 * G::kDBlk], pl[NCB][2];
             if (odd) {
 #pragma unroll
-                for (int qb = 0; qb < NQB; ++qb) pw[0][qb] = pw[1][qb];
+                for (int cb = 0; cb < NCB; ++cb) {
+                    pw[0][cb][0] = pw[1][cb][0];
+                    pw[0][cb][1] = pw[1][cb][1];
+                }
             }
 #pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db) {
-                const h4 v0 = lds_read_tr(vp[db] + v_par);
-                const h4 v1 = lds_read_tr(vp[db] + v_par + 16 * G::kRowB);
-                va[db] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+            for (int j = 0; j < 2 * G::kDBlk; ++j) {
+                const int db = j % G::kDBlk, kh = j / G::kDBlk;
+                const h4 v0 = lds_read_tr(vp[db] + v_par + kh * 16 * G::kRowB);
+                const h4 v1 = lds_read_tr(vp[db] + v_par + (kh * 16 + 8) * G::kRowB);
+                va[j] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
             }
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) pl[qb] = __builtin_bit_cast(h8, pw[0][qb]);
+            for (int cb = 0; cb < NCB; ++cb) {
+                pl[cb][0] = __builtin_bit_cast(h8, pw[0][cb][0]);
+                pl[cb][1] = __builtin_bit_cast(h8, pw[0][cb][1]);
+            }
 #pragma unroll
-            for (int db = 0; db < G::kDBlk; ++db)
+            for (int j = 0; j < 2 * G::kDBlk; ++j)
 #pragma unroll
-                for (int qb = 0; qb < NQB; ++qb) mfma_a_n(o[qb][db], va[db], pl[qb]);
-#pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) mfma_a_n(lacc[qb], ones, pl[qb]);
+                for (int cb = 0; cb < NCB; ++cb) mfma_o_n(o[cb][j % G::kDBlk], va[j], pl[cb][j / G::kDBlk]);
         }
         __builtin_amdgcn_s_waitcnt(0xC07F); // every read of the tile buffers has returned: the merge reuses them
-    } else {
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) nb[qb] = 0.0f;
     }
-    settle(); // O and l are out of the matrix pipe
+    settle(); // O is out of the matrix pipe
     wave_lds_sync();
     FA_STAMP(5);
 
@@ -650,22 +684,25 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // a wave that saw no visible row of a column has l = 0 and is given m = -inf (weight 0).
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-        asm volatile("" : "+a"(lacc[qb])); // pins the read below behind the settled pipe
-        const float l_tot = lacc[qb][0];
-        if (grp == 0) {
-            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 0] = l_tot > 0.0f ? -nb[qb] : -INFINITY;
-            ml[(wave * NQB * 16 + qb * 16 + col) * 2 + 1] = l_tot;
+    for (int cb = 0; cb < NCB; ++cb) {
+        const float l_tot = pair_sum(lsum[cb]);
+        if (hh == 0) {
+            ml[(wave * G::kCols + cb * 32 + c32) * 2 + 0] = l_tot > 0.0f ? -nb[cb] : -INFINITY;
+            ml[(wave * G::kCols + cb * 32 + c32) * 2 + 1] = l_tot;
         }
     }
-    const unsigned obuf_addr = ws_addr + (col * G::kOStride + grp * 4) * 4;
-    static_for<0, NQB>([&](auto qbc) {
-        static_for<0, G::kDBlk>([&](auto dbc) {
-            constexpr int qb = decltype(qbc)::value, db = decltype(dbc)::value;
-            lds_store_acc_nowait<(qb * 16 * G::kOStride + db * 16) * 4>(obuf_addr, o[qb][db]);
-        });
-    });
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // O^T -> [column][head_dim] fp32: accumulator registers 4q..4q+3 of lane (c32, hh) are
+    // head_dim indices db*32 + 8q + 4*hh + 0..3 of column cb*32 + c32.
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int db = 0; db < G::kDBlk; ++db) {
+            pin_a(o[cb][db]); // (read behind the settled pipe)
+            float* const dst = reinterpret_cast<float*>(ws) + (cb * 32 + c32) * G::kOStride + db * 32 + 4 * hh;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd)
+                *reinterpret_cast<f4*>(dst + 8 * qd) = f4{o[cb][db][4 * qd], o[cb][db][4 * qd + 1], o[cb][db][4 * qd + 2], o[cb][db][4 * qd + 3]};
+        }
     FA_STAMP(6);
     __syncthreads();
     FA_STAMP(7);
@@ -673,22 +710,20 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // Four threads per column: the weights are computed once, then each thread merges and stores
     // a quarter of the column's head_dim in 16-byte pieces (the four pieces of a step are one
     // contiguous 64 bytes of the output row).
-    constexpr int kCols = NQB * 16;
-    const int c = threadIdx.x >> 2, part = threadIdx.x & 3;
-    const int tok = t0 + c % TQ;
-    const int hl = head_lo + c / TQ;
-    if (c < kCols && hl < a.r && tok < batch) {
+    const int cm = threadIdx.x >> 2, part = threadIdx.x & 3;
+    int tok, hl;
+    if (cm < G::kCols && col_valid(cm, tok, hl)) {
         float wgt[kWaves];
         float m_all = -INFINITY, l_all = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            wgt[w] = ml[(w * kCols + c) * 2 + 0];
+            wgt[w] = ml[(w * G::kCols + cm) * 2 + 0];
             m_all = fmaxf(m_all, wgt[w]);
         }
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
             wgt[w] = fast_exp2(wgt[w] - m_all); // the wave that holds the column's diagonal has a finite m
-            l_all += ml[(w * kCols + c) * 2 + 1] * wgt[w];
+            l_all += ml[(w * G::kCols + cm) * 2 + 1] * wgt[w];
         }
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
         float* const dst = a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D;
@@ -698,68 +733,46 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             f4 acc = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int w = 0; w < kWaves; ++w)
-                acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4) * wgt[w];
+                acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + d4) * 4) * wgt[w];
             *reinterpret_cast<f4*>(dst + d4) = acc * inv;
         }
     }
     FA_STAMP(8);
 }
 
-template <int D, int NQB, int TQ>
+template <int D, int NCB>
 hipError_t launch_kernel(const FaArgs& a, int grid, hipStream_t stream) {
-    constexpr int lds = PGeom<D, NQB>::kLdsB;
-    hipLaunchKernelGGL((fa_prefill_kernel<D, NQB, TQ>), dim3(grid), dim3(kPrefillWaves * 64), lds, stream, a);
+    constexpr int lds = PGeom<D, NCB>::kLdsB;
+    hipLaunchKernelGGL((fa_prefill_kernel<D, NCB>), dim3(grid), dim3(kPrefillWaves * 64), lds, stream, a);
     return hipGetLastError();
 }
 
-template <int D, int NQB, int TQ>
+template <int D, int NCB>
 hipError_t allow_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_prefill_kernel<D, NQB, TQ>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, PGeom<D, NQB>::kLdsB);
-}
-
-template <int D>
-hipError_t allow_lds_all() {
-    hipError_t e;
-    if ((e = allow_lds<D, 1, 16>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 2, 16>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 16>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 4, 16>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 3, 8>()) != hipSuccess) return e;
-    if ((e = allow_lds<D, 2, 4>()) != hipSuccess) return e;
-    return allow_lds<D, 4, 8>();
+    void (*const kernel)(const FaArgs) = fa_prefill_kernel<D, NCB>;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               PGeom<D, NCB>::kLdsB);
 }
 
 template <int D>
 hipError_t launch(FaArgs a, int cu_count, hipStream_t stream) {
-    // Column packing per GQA ratio: (16-column blocks, tokens per workgroup).
-    // r <= 4: 16 tokens x r heads; r in 5..8: 8 tokens x up to 8 heads; larger ratios
-    // are cut into groups of 8 heads that each re-read the KV head.
+    // Column packing: a workgroup's columns are (heads of the group) x (tq tokens), 64 of them
+    // (two 32-column blocks) or 32.  GQA ratios up to 8 are one group; larger ratios are cut
+    // into groups of 8 heads that each re-read the KV head.
     const int r = a.r;
-    int nqb, tq;
-    if (r <= 4) { nqb = r; tq = 16; }
-    else if (r <= 6) { nqb = 3; tq = 8; }
-    else { nqb = 4; tq = 8; }
+    a.heads_per_group = r < 8 ? r : 8;
+    a.n_hgroups = (r + a.heads_per_group - 1) / a.heads_per_group;
+    int ncb = 2;
+    a.tq = 64 / a.heads_per_group;
     // A workgroup occupies a whole CU and the kernel lasts as long as its longest workgroup, so
-    // a grid that leaves half the CUs idle is better cut finer: 4 tokens x up to 8 heads, which
-    // halves the columns (and the time) per workgroup for r = 5..8.
-    if (r > 4 && 2 * a.n_kv * ((r + nqb * 16 / tq - 1) / (nqb * 16 / tq)) * ((a.batch + tq - 1) / tq) <= cu_count) {
-        nqb = 2;
-        tq = 4;
+    // a grid that would leave half the CUs idle is cut finer: 32 columns per workgroup.
+    if (2 * a.n_kv * a.n_hgroups * ((a.batch + a.tq - 1) / a.tq) <= cu_count) {
+        ncb = 1;
+        a.tq = 32 / a.heads_per_group;
     }
-    const int heads_per_group = nqb * 16 / tq;
-    a.n_hgroups = (r + heads_per_group - 1) / heads_per_group;
-    a.n_ttiles = (a.batch + tq - 1) / tq;
+    a.n_ttiles = (a.batch + a.tq - 1) / a.tq;
     const int grid = a.n_kv * a.n_hgroups * a.n_ttiles;
-    switch (nqb * 100 + tq) {
-        case 204: return launch_kernel<D, 2, 4>(a, grid, stream);
-        case 116: return launch_kernel<D, 1, 16>(a, grid, stream);
-        case 216: return launch_kernel<D, 2, 16>(a, grid, stream);
-        case 316: return launch_kernel<D, 3, 16>(a, grid, stream);
-        case 416: return launch_kernel<D, 4, 16>(a, grid, stream);
-        case 308: return launch_kernel<D, 3, 8>(a, grid, stream);
-        default:  return launch_kernel<D, 4, 8>(a, grid, stream);
-    }
+    return ncb == 2 ? launch_kernel<D, 2>(a, grid, stream) : launch_kernel<D, 1>(a, grid, stream);
 }
 
 } // namespace
@@ -770,8 +783,11 @@ hipError_t prefill_launch(const FaArgs& a, int head_dim, int cu_count, hipStream
 
 // The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at init.
 hipError_t prefill_allow_lds() {
-    hipError_t e = allow_lds_all<128>();
-    return e != hipSuccess ? e : allow_lds_all<64>();
+    hipError_t e;
+    if ((e = allow_lds<128, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds<128, 2>()) != hipSuccess) return e;
+    if ((e = allow_lds<64, 1>()) != hipSuccess) return e;
+    return allow_lds<64, 2>();
 }
 
 } // namespace orin_fa
