@@ -43,6 +43,7 @@ struct FaArgs {
     int n_hgroups;     // head groups per KV head
     int n_ttiles;      // prefill: token tiles
     int tq;            // prefill: tokens per token tile
+    int tq_magic;      // prefill: 65536 / tq + 1 (division of a column index by tq as multiply and shift)
     int heads_per_group; // prefill: query heads per head group
     int n_splits;      // decode: KV splits
     float c;           // |scale| * log2(e), clamped away from zero

@@ -242,13 +242,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
     const int hh = lane >> 5;  // lane-half: 8-wide k slice of an operand, rows 8q + 4*hh + 0..3 of an accumulator
 
-    int id = blockIdx.x;
-    const int kvh = id % a.n_kv;
-    id /= a.n_kv;
-    const int hg = id % a.n_hgroups;
-    id /= a.n_hgroups;
+    const int kvh = blockIdx.x, hg = blockIdx.y; // (the KV head varies fastest in dispatch order)
     const int n_past = a.n_past, batch = a.batch, tq = a.tq;
-    const int t0 = (a.n_ttiles - 1 - id) * tq; // longest rows first
+    const int t0 = (a.n_ttiles - 1 - (int)blockIdx.z) * tq; // longest rows first
     const int head_lo = hg * a.heads_per_group;
     const int tok_hi = (t0 + tq < batch) ? t0 + tq : batch;
     const int kv_end = n_past + tok_hi;   // the workgroup's columns see rows [0, kv_end) at most
@@ -260,9 +256,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     auto tile_of = [&](int j) { return wave + kWaves * (n_mine - 1 - j); };
     // column c of the block -> (token, head of the group); columns past the group's heads are padding
     auto col_valid = [&](int c, int& tok, int& hl) {
-        tok = t0 + c % tq;
-        hl = head_lo + c / tq;
-        return c / tq < a.heads_per_group && hl < a.r && tok < batch;
+        const int hq = (c * a.tq_magic) >> 16; // = c / tq for the c < 64 that occur (tq_magic = 65536 / tq + 1)
+        tok = t0 + c - hq * tq;
+        hl = head_lo + hq;
+        return hq < a.heads_per_group && hl < a.r && tok < batch;
     };
 
     unsigned char* const ws = smem + wave * G::kWaveB; // this wave's LDS slice
@@ -311,9 +308,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         if (G::kCopies > 4) lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[kOdd], 0);
     };
     // Main-loop copies: every tile they name is either wholly inside the visible range, and its
-    // base travels as the scalar offset, or below zero, and then the descriptor is emptied.
-    auto live_desc = [&](const i32x4& desc, int tile) { return i32x4{desc[0], desc[1], tile >= 0 ? desc[2] : 0, desc[3]}; };
-    auto tile_soff = [&](int tile) { return tile >= 0 ? tile * G::kTileB : 0; };
+    // base travels as the scalar offset, or below zero (steps past the wave's last tile), and then
+    // tile 0 is copied instead, into a buffer nobody reads any more.
+    auto tile_soff = [&](int tile) { return (tile > 0 ? tile : 0) * G::kTileB; };
     auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
@@ -444,9 +441,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         stage_a0(IntC<0>{}, IntC<0>{});     // S(0)
         __builtin_amdgcn_s_waitcnt(0xC07F); // its LDS reads have returned: K buffer 0 is free
         {
-            const i32x4 kd = live_desc(kdesc, tile_of(2));
             const int ksoff = tile_soff(tile_of(2));
-            static_for<0, kC>([&](auto ic) { copy_one(ic, kd, k_buf(0), ksoff); });
+            static_for<0, kC>([&](auto ic) { copy_one(ic, kdesc, k_buf(0), ksoff); });
             copy_checked(vdesc, v_buf(1), tile_of(1));
         }
         wait_copies(IntC<2 * kC>{});        // K1 and V0 landed (K2 V1 may be in flight)
@@ -508,8 +504,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         constexpr int kTickets = kGroups * NCB;       // matrix instructions per step
         constexpr int kHalf = kCG * NCB;              // tickets of C
         constexpr int kItems = kItemsPerBlock * NCB;  // vector instructions of B per step
-        constexpr int kAhead = NCB == 2 ? 3 : 4;
+        constexpr int kSkip = NCB == 1 ? 1 : 0;       // tickets without vector work at the start of a step: S(t) of
+                                                      // column block 0 is two matrix instructions old when it is read
+        constexpr int kAhead = 4;
         static_assert(kAhead <= kCG && kAhead <= G::kSteps, "the reads carried over a step boundary are reads of V");
+        static_assert(kAhead % 2 == 0 && kCG % 2 == 0 && kGroups % 2 == 0, "operands are read in pairs of groups");
         static_assert(kHalf == kC * NCB && kTickets - kHalf == kC * NCB, "one copy every NCB tickets");
         constexpr float kBound = 15.0f;               // a column whose largest exponent is above this is moved
         float c = a.c;
@@ -523,30 +522,35 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             const h4 v1 = lds_read_tr(vp[db] + par_off + (kh * 16 + 8) * G::kRowB);
             return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
         };
-        static_for<0, kAhead>([&](auto gc) { carry[decltype(gc)::value] = read_v(gc, 0); }); // for step 1: V(0)
+        static_for<0, kAhead>([&](auto gc) { carry[kAhead - 1 - decltype(gc)::value] = read_v(IntC<kAhead - 1 - decltype(gc)::value>{}, 0); }); // for step 1: V(0)
         // (The last step has no tile t+1: its A stage multiplies whatever the K buffer holds and
         // nobody reads the result -- cheaper than a second copy of the loop body without it.)
         auto body = [&](auto tpar, int t) {
             constexpr int TP = decltype(tpar)::value; // t & 1
             // K(t+2) goes to the buffer A(t) read, V(t+1) to the buffer C(t-1) reads in the first half of this step.
-            const i32x4 kd = live_desc(kdesc, tile_of(t + 2));
             const int ksoff = tile_soff(tile_of(t + 2));
-            const i32x4 vd = live_desc(vdesc, tile_of(t + 1));
             const int vsoff = tile_soff(tile_of(t + 1));
             h8 gop[kGroups];
             static_for<0, kAhead>([&](auto gc) { gop[decltype(gc)::value] = carry[decltype(gc)::value]; });
             // Issue order of the copies is ... K(t+1) V(t) | K(t+2) V(t+1): a wait that leaves the
             // copies issued since outstanding guarantees the older tile.  T = the ticket about to issue.
-            auto issue_read = [&](auto gc, auto tc) {
+            // Reads are issued for two groups at a time, the later group first: LDS returns data
+            // in order, so the wait for the earlier group's operand covers the later group's too.
+            auto read_group = [&](auto gc) {
+                constexpr int g = decltype(gc)::value;
+                if constexpr (g < kCG) gop[g] = read_v(gc, (TP ^ 1) * G::kTileB);
+                else if constexpr (g < kGroups) gop[g] = *reinterpret_cast<const h8*>(kp[g - kCG] + (TP ^ 1) * G::kTileB);
+                else carry[g - kGroups] = read_v(IntC<g - kGroups>{}, TP * G::kTileB);     // for C(t) of the next step
+            };
+            auto issue_reads = [&](auto gc, auto tc) { // groups g + 1 and g
                 constexpr int g = decltype(gc)::value, T = decltype(tc)::value;
                 constexpr int k_issued = T / NCB < kC ? T / NCB : kC;
                 constexpr int v_issued = T < kHalf ? 0 : ((T - kHalf) / NCB < kC ? (T - kHalf) / NCB : kC);
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (g == kCG) wait_copies(IntC<kC + k_issued>{});           // K(t+1) landed
                 if constexpr (g == kGroups) wait_copies(IntC<k_issued + v_issued>{}); // V(t) landed
-                if constexpr (g < kCG) gop[g] = read_v(gc, (TP ^ 1) * G::kTileB);
-                else if constexpr (g < kGroups) gop[g] = *reinterpret_cast<const h8*>(kp[g - kCG] + (TP ^ 1) * G::kTileB);
-                else carry[g - kGroups] = read_v(IntC<g - kGroups>{}, TP * G::kTileB);     // for C(t) of the next step
+                read_group(IntC<g + 1>{});
+                read_group(gc);
                 __builtin_amdgcn_sched_barrier(0);
             };
             float pe[NCB][16];
@@ -559,21 +563,22 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 constexpr int cb = j / kItemsPerBlock, r = j % kItemsPerBlock;
                 constexpr int kind = kItemsOfBlock.kind[r], x = kItemsOfBlock.arg[r];
                 if constexpr (kind == 0) {
-                    v_fma(pe[cb][x], s[TP][cb][x], c, nb[cb]);
+                    pe[cb][x] = __builtin_fmaf(s[TP][cb][x], c, nb[cb]);
                 } else if constexpr (kind == 1) {
-                    v_exp2(pe[cb][x]);
+                    pe[cb][x] = __builtin_amdgcn_exp2f(pe[cb][x]);
                 } else if constexpr (kind == 2) {
-                    unsigned packed;
-                    v_cvt_pk(packed, pe[cb][2 * x], pe[cb][2 * x + 1]);
-                    pw[TP][cb][x / 4][x % 4] = packed;
+                    typedef float f2 __attribute__((ext_vector_type(2)));
+                    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                    const h2 hp = __builtin_convertvector(f2{pe[cb][2 * x], pe[cb][2 * x + 1]}, h2); // round to nearest even
+                    pw[TP][cb][x / 4][x % 4] = __builtin_bit_cast(unsigned, hp);
                 } else {
-                    v_dot2_acc(lsum[cb], pw[TP][cb][x / 4][x % 4], ones_pk);
+                    v_dot2_acc(lsum[cb], pw[TP][cb][x / 4][x % 4], ones_pk); // (as a builtin next to the builtin conversion, the compiler drops three of every four pairs)
                 }
             };
             static_for<0, kTickets>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
                 constexpr int g = i / NCB, m = i % NCB;
-                if constexpr (m == 0) issue_read(IntC<g + kAhead>{}, ic);
+                if constexpr (m == 0 && g % 2 == 0) issue_reads(IntC<g + kAhead>{}, ic);
                 if constexpr (g < kCG) {
                     constexpr int db = g % G::kDBlk, kh = g / G::kDBlk;
                     mfma_o(o[m][db], gop[g], __builtin_bit_cast(h8, pw[TP ^ 1][m][kh]));
@@ -582,10 +587,15 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                     if constexpr (ks == 0) mfma_s_zero(s[TP ^ 1][m], gop[g], q[m][ks]);
                     else mfma_s(s[TP ^ 1][m], gop[g], q[m][ks]);
                 }
-                static_for<(i * kItems) / kTickets, ((i + 1) * kItems) / kTickets>(item);
+                // (the compiler orders the vector instructions within a ticket, not across tickets:
+                // the scores they read were written two or more matrix instructions earlier)
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (i >= kSkip)
+                    static_for<((i - kSkip) * kItems) / (kTickets - kSkip), ((i + 1 - kSkip) * kItems) / (kTickets - kSkip)>(item);
+                __builtin_amdgcn_sched_barrier(0);
                 if constexpr (m == NCB - 1) {
-                    if constexpr (i < kHalf) copy_one(IntC<i / NCB>{}, kd, k_buf(TP), ksoff);
-                    else copy_one(IntC<(i - kHalf) / NCB>{}, vd, v_buf(TP ^ 1), vsoff);
+                    if constexpr (i < kHalf) copy_one(IntC<i / NCB>{}, kdesc, k_buf(TP), ksoff);
+                    else copy_one(IntC<(i - kHalf) / NCB>{}, vdesc, v_buf(TP ^ 1), vsoff);
                 }
             });
             // S(t+1) is alive to the end of the step even when nobody reads it (last step): its
@@ -598,7 +608,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             bool over = false;
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) over |= !(lsum[cb] < 3.0e38f);
-            if (__builtin_amdgcn_ballot_w64(over) != 0) {
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
                 settle(); // C(t-1) has left the matrix pipe
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
@@ -741,9 +751,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
 }
 
 template <int D, int NCB>
-hipError_t launch_kernel(const FaArgs& a, int grid, hipStream_t stream) {
+hipError_t launch_kernel(const FaArgs& a, dim3 grid, hipStream_t stream) {
     constexpr int lds = PGeom<D, NCB>::kLdsB;
-    hipLaunchKernelGGL((fa_prefill_kernel<D, NCB>), dim3(grid), dim3(kPrefillWaves * 64), lds, stream, a);
+    hipLaunchKernelGGL((fa_prefill_kernel<D, NCB>), grid, dim3(kPrefillWaves * 64), lds, stream, a);
     return hipGetLastError();
 }
 
@@ -771,7 +781,9 @@ hipError_t launch(FaArgs a, int cu_count, hipStream_t stream) {
         a.tq = 32 / a.heads_per_group;
     }
     a.n_ttiles = (a.batch + a.tq - 1) / a.tq;
-    const int grid = a.n_kv * a.n_hgroups * a.n_ttiles;
+    a.tq_magic = 65536 / a.tq + 1;
+    if (a.n_hgroups > 65535 || a.n_ttiles > 65535) return hipErrorInvalidValue;
+    const dim3 grid(a.n_kv, a.n_hgroups, a.n_ttiles);
     return ncb == 2 ? launch_kernel<D, 2>(a, grid, stream) : launch_kernel<D, 1>(a, grid, stream);
 }
 
