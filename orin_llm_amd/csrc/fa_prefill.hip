@@ -121,11 +121,6 @@ __device__ __forceinline__ void v_cvt_pk(unsigned& r, float lo, float hi) { // t
 }
 __device__ __forceinline__ void v_max2(float& r, float x, float y) { asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y)); }
 __device__ __forceinline__ void v_max3_acc(float& r, float x, float y) { asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(r) : "v"(x), "v"(y)); }
-// acc += p.lo * q.lo + p.hi * q.hi (packed fp16 factors, fp32 sum)
-__device__ __forceinline__ void v_dot2_acc(float& acc, unsigned p, unsigned q) {
-    asm volatile("v_dot2_f32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(p), "v"(q));
-}
-
 // maxima without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
 // for results that feed a lane-swap instruction, which must not read a register in the cycle
 // after a vector instruction wrote it (the compiler cannot see that this block is one)
@@ -153,7 +148,9 @@ __device__ __forceinline__ float pair_sum(float v) {
 // count, raw 32-bit format.  Vector offsets at or past the byte count are not fetched.
 __device__ __forceinline__ i32x4 make_desc(const void* base, unsigned bytes) {
     const unsigned long long b = reinterpret_cast<unsigned long long>(base);
-    return i32x4{(int)(unsigned)b, (int)((unsigned)(b >> 32) & 0xffffu), (int)bytes, 0x00020000};
+    // (uniform by construction; saying so keeps the words in scalar registers, where the copies need them)
+    return i32x4{__builtin_amdgcn_readfirstlane((int)(unsigned)b), __builtin_amdgcn_readfirstlane((int)((unsigned)(b >> 32) & 0xffffu)),
+                 __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
 }
 
 // Four 1 KB global->LDS copies (buffer_load ... lds): lane l of copy i fetches 16 bytes at
@@ -199,7 +196,7 @@ __device__ __forceinline__ void lds_copy_1k(i32x4 desc, int off, int soff) {
 
 // The vector instructions of stage B for one 32x32 score block (16 scores per lane), in issue
 // order.  Pair p = scores (2p, 2p+1).  Kinds: 0 multiply-add (the exponent), 1 exponential,
-// 2 conversion of a pair to packed fp16, 3 row-sum update from a packed pair.  The four kinds run
+// 2 conversion of a pair to packed fp16, 3 row-sum and running-maximum update from a pair.  The four kinds run
 // as a software pipeline one pair apart, so no instruction reads a result younger than three
 // instructions.
 struct ItemTable {
@@ -242,9 +239,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
     const int hh = lane >> 5;  // lane-half: 8-wide k slice of an operand, rows 8q + 4*hh + 0..3 of an accumulator
 
-    const int kvh = blockIdx.x, hg = blockIdx.y; // (the KV head varies fastest in dispatch order)
+    const int kvh = __builtin_amdgcn_readfirstlane(blockIdx.x), hg = __builtin_amdgcn_readfirstlane(blockIdx.y); // (the KV head varies fastest in dispatch order)
     const int n_past = a.n_past, batch = a.batch, tq = a.tq;
-    const int t0 = (a.n_ttiles - 1 - (int)blockIdx.z) * tq; // longest rows first
+    const int t0 = (a.n_ttiles - 1 - __builtin_amdgcn_readfirstlane(blockIdx.z)) * tq; // longest rows first
     const int head_lo = hg * a.heads_per_group;
     const int tok_hi = (t0 + tq < batch) ? t0 + tq : batch;
     const int kv_end = n_past + tok_hi;   // the workgroup's columns see rows [0, kv_end) at most
@@ -310,7 +307,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // Main-loop copies: every tile they name is either wholly inside the visible range, and its
     // base travels as the scalar offset, or below zero (steps past the wave's last tile), and then
     // tile 0 is copied instead, into a buffer nobody reads any more.
-    auto tile_soff = [&](int tile) { return (tile > 0 ? tile : 0) * G::kTileB; };
+    auto tile_soff = [&](int tile) { return __builtin_amdgcn_readfirstlane((tile > 0 ? tile : 0) * G::kTileB); };
     auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
@@ -323,12 +320,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // ---- state ----
     h8 q[NCB][G::kSteps];   // B operands of A: the query columns, fp16
     float nb[NCB];          // each column's exponent offset: shift - reference maximum * c (log2 units)
-    float lsum[NCB];        // this lane's share (16 of a tile's 32 rows) of the column's row sum
+    float lsum[NCB][2];     // this lane's share (16 of a tile's 32 rows) of the column's row sum, as two partial sums
     f16v o[NCB][G::kDBlk];  // O^T accumulators (accumulation registers)
     f16v s[2][NCB];         // scores: [parity][column block]
     u32x4 pw[2][NCB][2];    // P as packed fp16: [parity][column block][k-step of C]
-    unsigned ones_pk = 0x3c003c00u;
-    asm volatile("" : "+v"(ones_pk)); // stays in a register; never rematerialised between the hand-placed instructions
 
     // ---- prologue loads, most urgent first: the query block, then the first K tile; the rest of
     // the first two tiles follows once the queries are on their way into LDS.  All of them are
@@ -366,7 +361,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         asm volatile("" : "+v"(zero));
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            lsum[cb] = 0.0f;
+            lsum[cb][0] = lsum[cb][1] = 0.0f;
             nb[cb] = 0.0f;
 #pragma unroll
             for (int db = 0; db < G::kDBlk; ++db) mfma_o_zero_n(o[cb][db], zero, zero);
@@ -484,7 +479,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                     }
                     pw[0][cb][kh] = __builtin_bit_cast(u32x4, ph);
                 }
-                lsum[cb] = sum;
+                lsum[cb][0] = sum;
+                lsum[cb][1] = 0.0f;
             }
         }
         settle(); // (the vector writes of P are well clear of the next matrix instruction)
@@ -510,7 +506,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         static_assert(kAhead <= kCG && kAhead <= G::kSteps, "the reads carried over a step boundary are reads of V");
         static_assert(kAhead % 2 == 0 && kCG % 2 == 0 && kGroups % 2 == 0, "operands are read in pairs of groups");
         static_assert(kHalf == kC * NCB && kTickets - kHalf == kC * NCB, "one copy every NCB tickets");
-        constexpr float kBound = 15.0f;               // a column whose largest exponent is above this is moved
+        constexpr float kBound = 15.0f;               // a column whose largest exponent is above this is moved ...
+        constexpr float kBoundP = 60000.0f;           // ... once some weight of the tile exceeds this (fp16 ends at 65504)
         float c = a.c;
         asm volatile("" : "+v"(c)); // a vector register for the whole loop, not a move per step
         h8 carry[kAhead];
@@ -554,9 +551,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 __builtin_amdgcn_sched_barrier(0);
             };
             float pe[NCB][16];
+            float amax = 0.0f;   // the largest weight of this tile
             float l_before[NCB]; // the row sums without this tile, for the slow path
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) l_before[cb] = lsum[cb];
+            for (int cb = 0; cb < NCB; ++cb) l_before[cb] = lsum[cb][0] + lsum[cb][1];
             // Vector instruction j of B(t) (see ItemTable).
             auto item = [&](auto jc) {
                 constexpr int j = decltype(jc)::value;
@@ -572,7 +570,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                     const h2 hp = __builtin_convertvector(f2{pe[cb][2 * x], pe[cb][2 * x + 1]}, h2); // round to nearest even
                     pw[TP][cb][x / 4][x % 4] = __builtin_bit_cast(unsigned, hp);
                 } else {
-                    v_dot2_acc(lsum[cb], pw[TP][cb][x / 4][x % 4], ones_pk); // (as a builtin next to the builtin conversion, the compiler drops three of every four pairs)
+                    // (plain adds: v_dot2_f32_f16 on the rounded pair would be one instruction
+                    // instead of two, but it stalls behind the matrix instructions in flight)
+                    lsum[cb][0] += pe[cb][2 * x];
+                    lsum[cb][1] += pe[cb][2 * x + 1];
+                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, pe[cb][2 * x]), pe[cb][2 * x + 1]);
                 }
             };
             static_for<0, kTickets>([&](auto ic) {
@@ -598,17 +600,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                     else copy_one(IntC<(i - kHalf) / NCB>{}, vdesc, v_buf(TP ^ 1), vsoff);
                 }
             });
-            // S(t+1) is alive to the end of the step even when nobody reads it (last step): its
-            // registers must not be handed out while the matrix instructions that write them are in flight.
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) keep_v(s[TP ^ 1][cb]);
-            // ---- slow path: a weight of this tile overflowed fp16 (the row sum, which adds up the
-            // rounded weights, is then infinite).  Move the reference of the columns concerned to
-            // their new maximum, redo P(t) and rescale O and l. ----
-            bool over = false;
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) over |= !(lsum[cb] < 3.0e38f);
-            if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
+            // ---- slow path: a weight of this tile is at the edge of the fp16 range or beyond.  Move
+            // the reference of the columns concerned to their new maximum, redo P(t) and rescale
+            // O and l. ----
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(amax < kBoundP)) != 0, 0)) {
                 settle(); // C(t-1) has left the matrix pipe
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
@@ -633,7 +628,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                         }
                         pw[TP][cb][kh] = __builtin_bit_cast(u32x4, ph);
                     }
-                    lsum[cb] = l_before[cb] * alpha + new_sum;
+                    lsum[cb][0] = l_before[cb] * alpha + new_sum;
+                    lsum[cb][1] = 0.0f;
 #pragma unroll
                     for (int db = 0; db < G::kDBlk; ++db) {
                         pin_a(o[cb][db]); // the reads below stay behind the settled pipe
@@ -643,6 +639,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 }
                 settle();
             }
+            // S(t+1) is alive to the very end of the step even when nobody reads it (last step): its
+            // registers must not be handed out while the matrix instructions that write them are
+            // in flight (the compiler is free to sink the step's last vector instructions down to here).
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) keep_v(s[TP ^ 1][cb]);
         };
         if (R >= 1) body(IntC<1>{}, 1);
         int t = 2;
@@ -695,7 +696,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
-        const float l_tot = pair_sum(lsum[cb]);
+        const float l_tot = pair_sum(lsum[cb][0] + lsum[cb][1]);
         if (hh == 0) {
             ml[(wave * G::kCols + cb * 32 + c32) * 2 + 0] = l_tot > 0.0f ? -nb[cb] : -INFINITY;
             ml[(wave * G::kCols + cb * 32 + c32) * 2 + 1] = l_tot;
