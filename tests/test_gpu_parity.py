@@ -144,6 +144,38 @@ def test_prefill_chunk_edges(fa):
         check(got[rows[:, 0], rows[:, 1]], want, f"prefill edges ctx{n_ctx} P{n_past} B{batch}")
 
 
+@pytest.mark.parametrize("d,r", [(64, 1), (64, 4), (64, 7), (128, 1), (128, 2), (128, 3), (128, 5), (128, 8), (128, 12)])
+def test_prefill_wide_blocks(fa, d, r):
+    """Grids with more workgroups than half the CUs take the 64-column packing: every ratio's
+    column -> (token, head) map, padded columns and the second head group (r = 12)."""
+    G = 8
+    H = G * r
+    n_ctx = 1536
+    scale = 1.0 / np.sqrt(d)
+    n_past, batch = 200, 1100
+    q, kc, vc = make_case(500 + r + d, H, G, d, n_ctx, n_past + batch, batch, outliers=2, poison_tail=True)
+    toks = sorted({0, 1, 8, 9, 20, 21, 31, 32, 63, 64, 65, 500, batch - 2, batch - 1})
+    rows = np.array([(t, h) for t in toks for h in range(H)], np.int32)
+    want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, n_past, np.float32(scale))
+    got = gpu_prefill(fa, q, kc, vc, H, G, d, n_ctx, n_past, batch, scale)
+    check(got[rows[:, 0], rows[:, 1]], want, f"prefill wide d{d} r{r}")
+
+
+@pytest.mark.parametrize("scale", [1.0, 0.35, -0.0883883])
+@pytest.mark.parametrize("H,G,batch", [(4, 2, 96), (32, 8, 600)])
+def test_prefill_moving_reference(fa, scale, H, G, batch):
+    """Large and negative scales: the scores of early tiles exceed the reference taken from the
+    tiles next to the diagonal by far more than the fp16 range of the weights allows, so the
+    rescaling path runs on most tiles (both column packings)."""
+    d, n_ctx, n_past = 128, 1024, 300
+    q, kc, vc = make_case(77 + batch, H, G, d, n_ctx, n_past + batch, batch, outliers=4, poison_tail=True)
+    toks = sorted({0, 1, 31, 32, 33, batch // 2, batch - 1})
+    rows = np.array([(t, h) for t in toks for h in range(H)], np.int32)
+    want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, n_past, np.float32(scale))
+    got = gpu_prefill(fa, q, kc, vc, H, G, d, n_ctx, n_past, batch, scale)
+    check(got[rows[:, 0], rows[:, 1]], want, f"prefill scale {scale} H{H} B{batch}")
+
+
 # ---------------------------------------------------------------- invariants on the GPU path
 
 def test_prefill_row_equals_decode_and_chunk_split(fa):
