@@ -16,14 +16,17 @@
 // The three stages of a tile
 //     A: S = K Q^T (MFMA)      B: P = 2^(S*c + b) (VALU)      C: O += V^T P (MFMA)
 // run skewed -- iteration t issues A(t+1), B(t) and C(t-1), which are independent of one
-// another -- in one hand-ordered instruction stream, so the matrix pipe works while the vector
-// pipe exponentiates.  What keeps the vector share small:
+// another -- in one instruction stream whose matrix instructions, LDS reads and copies sit at
+// fixed places, with the vector work of B dealt out evenly between them, so the matrix pipe
+// works while the vector pipe exponentiates.  What keeps the vector share small:
 //   * B is one fused multiply-add (scale*log2(e) and the column's offset b = shift - reference
-//     maximum; Q itself stays unscaled, so fp16-representable inputs enter the products exactly),
-//     one v_exp_f32 per score, and per pair of scores one v_cvt_pk_f16_f32, one v_max3_f32 and one
-//     v_dot2_f32_f16 against packed ones (the row sum of the rounded weights, in fp32).
+//     maximum; Q itself stays unscaled, so fp16-representable inputs enter the products exactly)
+//     and one v_exp_f32 per score, and per pair of scores one v_cvt_pk_f16_f32, two adds (the
+//     row sum, in fp32) and one v_max3_f32.  (v_dot2_f32_f16 against packed ones would sum a
+//     pair in one instruction, but it waits for the matrix instructions in flight: measured,
+//     16 of them per step cost more than everything else in B together.)
 //   * The reference maximum is lazy: exponentials are computed optimistically while the largest
-//     weight of the tile is tracked; only if it exceeds the fp16-safe bound (on a handful of
+//     weight of the tile is tracked; only if it nears the end of the fp16 range (on a handful of
 //     early tiles) does a slow path move the reference, redo the tile's P and rescale O and l.
 // K and V tiles are copied global->LDS by the load unit itself (no staging registers, two
 // buffers each per wave, tile base in the scalar offset so the copies need no vector
@@ -112,23 +115,9 @@ __device__ __forceinline__ void settle() {
 __device__ __forceinline__ void pin_v(f16v& x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void pin_a(f16v& x) { asm volatile("" : "+a"(x)); }
 __device__ __forceinline__ void keep_v(const f16v& x) { asm volatile("" : : "v"(x)); }
-// The vector side of the main loop, as volatile blocks so that it stays where it is written,
-// interleaved with the matrix instructions.
-__device__ __forceinline__ void v_fma(float& r, float x, float y, float z) { asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z)); }
-__device__ __forceinline__ void v_exp2(float& r) { asm volatile("v_exp_f32 %0, %0" : "+v"(r)); }
-__device__ __forceinline__ void v_cvt_pk(unsigned& r, float lo, float hi) { // two fp32 -> packed fp16, round to nearest even
-    asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
-}
-__device__ __forceinline__ void v_max2(float& r, float x, float y) { asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y)); }
-__device__ __forceinline__ void v_max3_acc(float& r, float x, float y) { asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(r) : "v"(x), "v"(y)); }
-// maxima without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
+// A maximum without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
 // for results that feed a lane-swap instruction, which must not read a register in the cycle
-// after a vector instruction wrote it (the compiler cannot see that this block is one)
-__device__ __forceinline__ float max3(float x, float y, float z) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
-    return r;
-}
+// after a vector instruction wrote it (the compiler cannot see that this block is one).
 __device__ __forceinline__ float max2(float x, float y) {
     float r;
     asm("v_max_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(x), "v"(y));
