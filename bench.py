@@ -41,6 +41,7 @@ SHAPES = {
 WORKLOADS = {
     # name: (shape, kind, n_ctx, list of (P, B) for prefill | L for decode)
     "qwen1.5b-prefill512": ("qwen1.5b", "prefill", 4096, [(0, 512), (3584, 512)]),
+    "qwen1.5b-prefill512-d3584": ("qwen1.5b", "prefill", 4096, [(3584, 512)]),  # the default workload's second chunk alone
     "llama8b-prefill512-d4096": ("llama8b", "prefill", 8192, [(4096, 512)]),
     "llama8b-prefill512-d0": ("llama8b", "prefill", 8192, [(0, 512)]),
     "llama8b-prefill512-d7680": ("llama8b", "prefill", 8192, [(7680, 512)]),
@@ -63,7 +64,11 @@ WORKLOADS = {
 # WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy.  These are
 # recorded measurements (a counter pass cannot run inside the timed benchmark); None where not taken.
 TRAFFIC = {
-    "llama8b-prefill512-d4096": 27.60e6 + 8.39e6,
+    # (2 KV heads over 8 XCDs: each of the 4 L2s that serve a head fetches that head's K and V itself,
+    # 4 x 4.19 MB, mostly from the Infinity Cache; Q 3.15 MB in, 3.15 MB out)
+    "qwen1.5b-prefill512": 20.12e6 + 3.15e6,
+    "qwen1.5b-prefill512-d3584": 20.12e6 + 3.15e6,
+    "llama8b-prefill512-d4096": 27.53e6 + 8.39e6,
     "qwen1.5b-decode-32k": 33.68e6 + 0.80e6 + 0.97e6 + 0.006e6,
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
