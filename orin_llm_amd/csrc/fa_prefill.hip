@@ -643,7 +643,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         if (t == R) body(IntC<0>{}, t);
         FA_STAMP(4);
         // ---- drain: C(R) ----
-        wait_copies(IntC<0>{});
+        // V(R) has landed once the two tiles of copies issued after it are all that is outstanding
+        // (those, for steps past the last, land in buffers nobody reads; their latency hides
+        // behind the matrix instructions below).
+        wait_copies(IntC<2 * kC>{});
         settle(); // P(R) was converted just above
         {   // O += V(R)^T P(R); both live in the buffers of parity R & 1
             const bool odd = (R & 1) != 0;
@@ -673,7 +676,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) mfma_o_n(o[cb][j % G::kDBlk], va[j], pl[cb][j / G::kDBlk]);
         }
-        __builtin_amdgcn_s_waitcnt(0xC07F); // every read of the tile buffers has returned: the merge reuses them
+        __builtin_amdgcn_s_waitcnt(0x0070); // every read of the tile buffers has returned and every copy into them has landed: the merge reuses them
     }
     settle(); // O is out of the matrix pipe
     wave_lds_sync();
