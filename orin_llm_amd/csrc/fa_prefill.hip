@@ -115,18 +115,10 @@ __device__ __forceinline__ void settle() {
 __device__ __forceinline__ void pin_v(f16v& x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void pin_a(f16v& x) { asm volatile("" : "+a"(x)); }
 __device__ __forceinline__ void keep_v(const f16v& x) { asm volatile("" : : "v"(x)); }
-// A maximum without the NaN-quieting moves the library fmaxf carries; the trailing wait state is
-// for results that feed a lane-swap instruction, which must not read a register in the cycle
-// after a vector instruction wrote it (the compiler cannot see that this block is one).
-__device__ __forceinline__ float max2(float x, float y) {
-    float r;
-    asm("v_max_f32 %0, %1, %2\n\ts_nop 1" : "=v"(r) : "v"(x), "v"(y));
-    return r;
-}
 // The two lanes that hold a column's rows are l and l ^ 32: maximum / sum over the pair.
 __device__ __forceinline__ float pair_max(float v) {
     const u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return max2(__uint_as_float(s.x), __uint_as_float(s.y));
+    return fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
 }
 __device__ __forceinline__ float pair_sum(float v) {
     const u32x2 s = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -716,28 +708,52 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const int cm = threadIdx.x >> 2, part = threadIdx.x & 3;
     int tok, hl;
     if (cm < G::kCols && col_valid(cm, tok, hl)) {
+        // every LDS read first (the partial outputs in two halves of 16 reads), so that their
+        // latencies overlap instead of adding up
+        float mw[kWaves], lw[kWaves];
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            mw[w] = ml[(w * G::kCols + cm) * 2 + 0];
+            lw[w] = ml[(w * G::kCols + cm) * 2 + 1];
+        }
+        constexpr int kHalfJ = D / 32;
+        f4 x[kHalfJ][kWaves];
+        auto load_half = [&](int j0) {
+#pragma unroll
+            for (int j = 0; j < kHalfJ; ++j)
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w)
+                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((j0 + j) * 4 + part) * 4) * 4);
+        };
+        load_half(0);
+        __builtin_amdgcn_sched_barrier(0);
         float wgt[kWaves];
         float m_all = -INFINITY, l_all = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            wgt[w] = ml[(w * G::kCols + cm) * 2 + 0];
-            m_all = fmaxf(m_all, wgt[w]);
-        }
+        for (int w = 0; w < kWaves; ++w) m_all = fmaxf(m_all, mw[w]);
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            wgt[w] = fast_exp2(wgt[w] - m_all); // the wave that holds the column's diagonal has a finite m
-            l_all += ml[(w * G::kCols + cm) * 2 + 1] * wgt[w];
+            wgt[w] = fast_exp2(mw[w] - m_all); // the wave that holds the column's diagonal has a finite m
+            l_all += lw[w] * wgt[w];
         }
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) wgt[w] *= inv;
         float* const dst = a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D;
 #pragma unroll
-        for (int j = 0; j < D / 16; ++j) {
-            const int d4 = (j * 4 + part) * 4;
-            f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+        for (int h = 0; h < 2; ++h) {
+            f4 acc[kHalfJ];
 #pragma unroll
-            for (int w = 0; w < kWaves; ++w)
-                acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + d4) * 4) * wgt[w];
-            *reinterpret_cast<f4*>(dst + d4) = acc * inv;
+            for (int j = 0; j < kHalfJ; ++j) {
+                acc[j] = x[j][0] * wgt[0];
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w) acc[j] += x[j][w] * wgt[w];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (h == 0) load_half(kHalfJ);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < kHalfJ; ++j) *reinterpret_cast<f4*>(dst + ((h * kHalfJ + j) * 4 + part) * 4) = acc[j];
         }
     }
     FA_STAMP(8);
