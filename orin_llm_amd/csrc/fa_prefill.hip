@@ -377,11 +377,14 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         const int c = cb * 32 + c32;
         int tok, hl;
         limit[cb] = col_valid(c, tok, hl) ? n_past + tok + 1 : 0x7fffffff;
+        h8 hv[G::kSteps]; // (all reads of a block first: a read per parking block would wait out its latency alone)
 #pragma unroll
-        for (int ks = 0; ks < G::kSteps; ++ks) {
-            const h8 hv = *reinterpret_cast<const h8*>(smem + G::kQOff + c * G::kQStride + (ks * 16 + hh * 8) * 2);
-            asm volatile("" : "=a"(q[cb][ks]) : "0"(hv)); // parked in the accumulation-register file for good
-        }
+        for (int ks = 0; ks < G::kSteps; ++ks)
+            hv[ks] = *reinterpret_cast<const h8*>(smem + G::kQOff + c * G::kQStride + (ks * 16 + hh * 8) * 2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ++ks)
+            asm volatile("" : "=a"(q[cb][ks]) : "0"(hv[ks])); // parked in the accumulation-register file for good
     }
     FA_STAMP(1);
 
