@@ -21,13 +21,14 @@
 // works while the vector pipe exponentiates.  What keeps the vector share small:
 //   * B is one fused multiply-add (scale*log2(e) and the column's offset b = shift - reference
 //     maximum; Q itself stays unscaled, so fp16-representable inputs enter the products exactly)
-//     and one v_exp_f32 per score, and per pair of scores one v_cvt_pk_f16_f32, two adds (the
-//     row sum, in fp32) and one v_max3_f32.  (v_dot2_f32_f16 against packed ones would sum a
-//     pair in one instruction, but it waits for the matrix instructions in flight: measured,
-//     16 of them per step cost more than everything else in B together.)
-//   * The reference maximum is lazy: exponentials are computed optimistically while the largest
-//     weight of the tile is tracked; only if it nears the end of the fp16 range (on a handful of
-//     early tiles) does a slow path move the reference, redo the tile's P and rescale O and l.
+//     and one v_exp_f32 per score, and per pair of scores one v_cvt_pk_f16_f32 and one packed
+//     fp16 add (the tile's share of the row sum: eight terms per half, added to the fp32 sum at
+//     the end of the step).  (v_dot2_f32_f16 against packed ones would add a pair to an fp32 sum
+//     directly, but it waits for the matrix instructions in flight: measured, 16 of them per
+//     step cost more than everything else in B together.)
+//   * The reference maximum is lazy: exponentials are computed optimistically; only if a tile's
+//     fp16 partial sums show a weight above 2^12 (on a handful of early tiles; the reference sits
+//     at 2^7) does a slow path move the reference, redo the tile's P and rescale O and l.
 // K and V tiles are copied global->LDS by the load unit itself (no staging registers, two
 // buffers each per wave, tile base in the scalar offset so the copies need no vector
 // arithmetic) in an XOR-swizzled layout that both the 1 KB copy bursts and the operand reads
@@ -490,8 +491,9 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         static_assert(kAhead <= kCG && kAhead <= G::kSteps, "the reads carried over a step boundary are reads of V");
         static_assert(kAhead % 2 == 0 && kCG % 2 == 0 && kGroups % 2 == 0, "operands are read in pairs of groups");
         static_assert(kHalf == kC * NCB && kTickets - kHalf == kC * NCB, "one copy every NCB tickets");
-        constexpr float kBound = 15.0f;               // a column whose largest exponent is above this is moved ...
-        constexpr float kBoundP = 60000.0f;           // ... once some weight of the tile exceeds this (fp16 ends at 65504)
+        constexpr float kBound = 12.0f;               // a column whose largest exponent is above this is moved ...
+        constexpr float kBoundP = 32768.0f;           // ... once a half-sum (eight weights) of the tile reaches this: then some
+                                                      // weight is above 2^12; below, no half-sum can leave the fp16 range
         float c = a.c;
         asm volatile("" : "+v"(c)); // a vector register for the whole loop, not a move per step
         h8 carry[kAhead];
@@ -535,7 +537,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 __builtin_amdgcn_sched_barrier(0);
             };
             float pe[NCB][16];
-            float amax = 0.0f;   // the largest weight of this tile
+            typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+            h2v hp[NCB][8];      // the pairs of weights, as converted
+            h2v hsum[NCB];       // this tile's share of the row sums, two fp16 partial sums per column block
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) hsum[cb] = h2v{(_Float16)0.0f, (_Float16)0.0f};
             float l_before[NCB]; // the row sums without this tile, for the slow path
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) l_before[cb] = lsum[cb][0] + lsum[cb][1];
@@ -551,14 +557,17 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 } else if constexpr (kind == 2) {
                     typedef float f2 __attribute__((ext_vector_type(2)));
                     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-                    const h2 hp = __builtin_convertvector(f2{pe[cb][2 * x], pe[cb][2 * x + 1]}, h2); // round to nearest even
-                    pw[TP][cb][x / 4][x % 4] = __builtin_bit_cast(unsigned, hp);
+                    hp[cb][x] = __builtin_convertvector(f2{pe[cb][2 * x], pe[cb][2 * x + 1]}, h2); // round to nearest even
+                    pw[TP][cb][x / 4][x % 4] = __builtin_bit_cast(unsigned, hp[cb][x]);
                 } else {
-                    // (plain adds: v_dot2_f32_f16 on the rounded pair would be one instruction
-                    // instead of two, but it stalls behind the matrix instructions in flight)
-                    lsum[cb][0] += pe[cb][2 * x];
-                    lsum[cb][1] += pe[cb][2 * x + 1];
-                    amax = __builtin_fmaxf(__builtin_fmaxf(amax, pe[cb][2 * x]), pe[cb][2 * x + 1]);
+                    // The tile's share of the row sum is added up in packed fp16, one instruction per
+                    // pair (eight terms per half; the rounding of these short sums averages out over
+                    // the tiles), and joins the fp32 sum at the end of the step.  (v_dot2_f32_f16
+                    // would add a pair to an fp32 sum directly, but it stalls behind the matrix
+                    // instructions in flight.)
+                    // (hp, not the element of pw it was stored to: read back through a bit cast, the
+                    // compiler takes element 0 of the vector for every pair)
+                    hsum[cb] += hp[cb][x];
                 }
             };
             static_for<0, kTickets>([&](auto ic) {
@@ -587,6 +596,14 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             // ---- slow path: a weight of this tile is at the edge of the fp16 range or beyond.  Move
             // the reference of the columns concerned to their new maximum, redo P(t) and rescale
             // O and l. ----
+            float amax = 0.0f;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const float lo = (float)hsum[cb][0], hi = (float)hsum[cb][1];
+                lsum[cb][0] += lo;
+                lsum[cb][1] += hi;
+                amax = __builtin_fmaxf(__builtin_fmaxf(amax, lo), hi);
+            }
             if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(amax < kBoundP)) != 0, 0)) {
                 settle(); // C(t-1) has left the matrix pipe
 #pragma unroll
