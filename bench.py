@@ -51,6 +51,9 @@ WORKLOADS = {
     "qwen1.5b-decode-32k": ("qwen1.5b", "decode", 32768, 32768),
     "llama8b-decode-8k": ("llama8b", "decode", 8192, 8192),
     "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
+    # the decode layer's call pair (store the token's K/V rows, then attend; reference src/model_gpu.cu:281-282)
+    # through the entry point that does both in the attention launches; the two calls are timed beside it
+    "qwen1.5b-decode-store-32k": ("qwen1.5b", "decode_store", 32768, 32768),
     # the two mutators of the cache (byte movers; value = bytes read + written per second)
     "llama8b-kv-store-512": ("llama8b", "kv_store", 8192, (4096, 512)),
     "qwen1.5b-kv-shift-32k": ("qwen1.5b", "kv_shift", 32768, (4, 16382)),
@@ -72,7 +75,7 @@ TRAFFIC = {
     "qwen1.5b-decode-32k": 33.68e6 + 0.80e6 + 0.97e6 + 0.006e6,
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
-ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k",
+ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k", "qwen1.5b-decode-store-32k",
         "llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
 
 
@@ -251,9 +254,22 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
             stack.append((q[0].contiguous(), k, v, torch.empty((H, d), dtype=torch.float32, device="cuda")))
         stacks.append(stack)
     dpos = torch.tensor([L - 1], dtype=torch.int32, device="cuda")
+    store = WORKLOADS[name][1] == "decode_store"
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    k_new = torch.randn((G, d), generator=gen, device="cuda", dtype=torch.float32)
+    v_new = torch.randn((G, d), generator=gen, device="cuda", dtype=torch.float32)
 
     def one_stack(si):
         for q, k, v, out in stacks[si]:
+            if store:
+                kernels.flash_attention_decode_store_ind(q, k_new, v_new, k, v, out, H, G, d, n_ctx, dpos, scale)
+            else:
+                kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
+
+    def one_stack_two_calls(si):
+        for q, k, v, out in stacks[si]:
+            kernels.kv_store_ind(k, v, k_new, v_new, G, d, n_ctx, dpos)
             kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
 
     # eager
@@ -293,6 +309,18 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     wall_graph = time.perf_counter() - t0
     dev_graph_ms = e0.elapsed_time(e1)
 
+    two_calls_us = None
+    if store:  # the same step as the reference makes it: two calls per layer
+        for i in range(warmup):
+            one_stack_two_calls(i % n_stacks)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(steps):
+            one_stack_two_calls(i % n_stacks)
+        e1.record()
+        torch.cuda.synchronize()
+        two_calls_us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+
     # Duration of each of the two kernels: events between them, recorded by the library on its stream.
     split_us, combine_us = [], []
     for si in range(n_stacks):
@@ -327,6 +355,10 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
         graph=dict(ms_per_step=wall_graph / steps * 1e3, device_ms_per_step=dev_graph_ms / steps),
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="all heads, layer 0, vs CPU oracle"),
     )
+    if store:
+        res["roofline"]["kernel"] = f"fa_decode_split_kernel<{d}, store> + fa_decode_combine_kernel<{d}> (one layer)"
+        res["roofline"]["launch_us_two_calls"] = two_calls_us
+        res["roofline"]["note"] += "; launch_us_two_calls: kv_store_ind + flash_attention_decode_ind per layer, eager, back to back"
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline_decode(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
                                                   v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, L, scale)
@@ -495,7 +527,7 @@ def run_copy(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "copy": run_copy, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "copy": run_copy, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 

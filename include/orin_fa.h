@@ -107,6 +107,17 @@ int orin_fa_kv_store_ind(uint16_t* kc, uint16_t* vc, const float* k, const float
  * move to [n_keep, n_ctx - shift) and the last `shift` rows are cleared, in place. */
 int orin_fa_kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep, int shift);
 
+/* orin_fa_kv_store_ind followed by orin_fa_decode_ind, in the launches of the latter alone.
+ * No counterpart in the reference, whose decode layer makes the two calls back to back
+ * (src/model_gpu.cu:281-282; kv_store_ind src/kernels.cu:2084-2088): k_new, v_new are the
+ * current token's rows, fp32 [n_kv][head_dim], 16-byte aligned.  The workgroup whose tile
+ * holds row *d_pos takes the row from them, rounded to fp16 exactly as the store rounds, and
+ * writes it to the cache; cache contents and output equal those of the two calls bit for bit
+ * (a position outside [0, n_ctx) stores nothing and attends as orin_fa_decode_ind does).
+ * Capture-safe like orin_fa_decode_ind. */
+int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
+                             float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
+
 /* Measurement aid with no counterpart in the reference: orin_fa_decode_ind with HIP events
  * recorded before, between and after its two kernels on the library's stream.  Synchronises
  * on the last event and returns the elapsed time of the split kernel and of the combine

@@ -130,12 +130,20 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 
 namespace {
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
-                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid);
+                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
+                const float* k_new, const float* v_new);
 }
 
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
-    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr);
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr);
+}
+
+int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
+                             float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
+    if (!k_new || !v_new) return ORIN_FA_E_INVALID;
+    if (((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15u) != 0) return ORIN_FA_E_INVALID;
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, k_new, v_new);
 }
 
 int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
@@ -147,7 +155,7 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
         if (!ev[i]) e = hipEventCreate(&ev[i]);
     if (e != hipSuccess) return hip_code(e);
     if ((e = hipEventRecord(ev[0], g_state.stream)) != hipSuccess) return hip_code(e);
-    const int rc = decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, ev[1]);
+    const int rc = decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, ev[1], nullptr, nullptr);
     if (rc != ORIN_FA_OK) return rc;
     if ((e = hipEventRecord(ev[2], g_state.stream)) != hipSuccess) return hip_code(e);
     if ((e = hipEventSynchronize(ev[2])) != hipSuccess) return hip_code(e);
@@ -161,12 +169,14 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
 
 namespace {
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
-                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid) {
+                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
+                const float* k_new, const float* v_new) {
     int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
     if (rc != ORIN_FA_OK) return rc;
     if (!d_pos) return ORIN_FA_E_INVALID;
     FaArgs a{};
     a.q = q; a.kc = kc; a.vc = vc; a.out = out; a.d_pos = d_pos;
+    a.k_new = k_new; a.v_new = v_new;
     a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.batch = 1;
     a.r = n_head / n_kv;
     a.n_hgroups = (a.r + 15) / 16;

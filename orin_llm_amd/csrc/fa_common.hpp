@@ -37,6 +37,8 @@ struct FaArgs {
     float* part_o;    // decode: [split][n_head][D]
     float* part_ml;   // decode: [split][n_head][2] = (reference maximum in log2 units, row sum)
     const int* d_pos; // decode only
+    const float* k_new; // decode with store: the current token's K and V rows, fp32 [n_kv][head_dim];
+    const float* v_new; // null for plain decode (the cache pointers are then never written through)
     int n_head, n_kv, n_ctx;
     int n_past, batch; // prefill only
     int r;             // query heads per KV head

@@ -47,7 +47,11 @@ struct DGeom {
     static constexpr int kLdsB = kMlOff + kDecodeWaves * 16 * 2 * 4;
 };
 
-template <int D>
+// STORE: the current token's K and V rows arrive as fp32 beside the cache (FaArgs::k_new, v_new).
+// The wave whose tile holds row *d_pos takes that row from them -- rounded to fp16 exactly as
+// the store kernel rounds -- instead of from the cache, and writes it to the cache on the way:
+// the store kernel's launch is saved and the result is the same bit for bit.
+template <int D, bool STORE>
 __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(const FaArgs a) {
     using G = DGeom<D>;
     constexpr int kWaves = kDecodeWaves;
@@ -90,10 +94,28 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     int tile = tile_first;
     fetch_k(tile); // in flight while the position and the query heads are loaded
     fetch_v(tile);
+    // The new row's pieces a lane would substitute do not depend on where the row falls: lane
+    // (col, grp) holds bytes (kk*4 + grp)*16 of a K row and piece lane % (D/8) of a V row.  They
+    // are requested now, by every lane, before the position is known.
+    u32x4 k_new16[G::kSteps], v_new16;
+    if constexpr (STORE) {
+        auto load8 = [&](const float* p) {
+            const float4 x0 = *reinterpret_cast<const float4*>(p);
+            const float4 x1 = *reinterpret_cast<const float4*>(p + 4);
+            h8 h;
+            h[0] = (_Float16)x0.x; h[1] = (_Float16)x0.y; h[2] = (_Float16)x0.z; h[3] = (_Float16)x0.w;
+            h[4] = (_Float16)x1.x; h[5] = (_Float16)x1.y; h[6] = (_Float16)x1.z; h[7] = (_Float16)x1.w;
+            return __builtin_bit_cast(u32x4, h);
+        };
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps; ++kk) k_new16[kk] = load8(a.k_new + (size_t)kvh * D + (kk * 4 + grp) * 8);
+        v_new16 = load8(a.v_new + (size_t)kvh * D + (lane % G::kChunksPerRow) * 8);
+    }
 
-    int p = *a.d_pos;
-    p = p < 0 ? 0 : p;
+    const int pos = *a.d_pos;
+    int p = pos < 0 ? 0 : pos;
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
+    const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
     if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
 
@@ -128,6 +150,26 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 
     for (; tile < n_tiles; tile += tile_step) {
         const bool more = tile + tile_step < n_tiles;
+        if constexpr (STORE) {
+            if (store && tile == pos / kTile) { // the tile of the new row (the last visible one)
+                const int row = pos % kTile;
+                const size_t row_off = ((size_t)kvh * a.n_ctx + pos) * D;
+                if (col == row % 16) {
+#pragma unroll
+                    for (int kk = 0; kk < G::kSteps; ++kk) {
+                        kreg[(row / 16) * G::kSteps + kk] = k_new16[kk];
+                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.kc) + row_off + (kk * 4 + grp) * 8) = k_new16[kk];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < G::kLoads; ++i) {
+                    if ((i * 64 + lane) / G::kChunksPerRow == row) {
+                        vreg[i] = v_new16;
+                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.vc) + row_off + (lane % G::kChunksPerRow) * 8) = v_new16;
+                    }
+                }
+            }
+        }
         // ---- S^T = K Q^T : rows = KV row (sub-tile t, row col), columns = query head ----
         f4 s[2], s2[2]; // the Q-lo product runs as its own accumulation chain
 #pragma unroll
@@ -343,7 +385,8 @@ template <int D>
 hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     const int grid = a.n_kv * a.n_hgroups * a.n_splits;
     constexpr int lds = DGeom<D>::kLdsB;
-    hipLaunchKernelGGL(fa_decode_split_kernel<D>, dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, true>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    else hipLaunchKernelGGL((fa_decode_split_kernel<D, false>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
@@ -359,12 +402,21 @@ hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream, hipE
 
 // The split kernel uses more than 64 KB of dynamic LDS; the opt-in is set once at init so
 // that no launch path touches function attributes (decode runs under stream capture).
+namespace {
+template <int D, bool STORE>
+hipError_t allow_lds() {
+    void (*const kernel)(const FaArgs) = fa_decode_split_kernel<D, STORE>;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               DGeom<D>::kLdsB);
+}
+} // namespace
+
 hipError_t decode_allow_lds() {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_decode_split_kernel<128>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, DGeom<128>::kLdsB);
-    if (e != hipSuccess) return e;
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(fa_decode_split_kernel<64>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, DGeom<64>::kLdsB);
+    hipError_t e;
+    if ((e = allow_lds<128, false>()) != hipSuccess) return e;
+    if ((e = allow_lds<128, true>()) != hipSuccess) return e;
+    if ((e = allow_lds<64, false>()) != hipSuccess) return e;
+    return allow_lds<64, true>();
 }
 
 } // namespace orin_fa

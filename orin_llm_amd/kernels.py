@@ -43,6 +43,8 @@ def lib():
         L.orin_fa_prefill.restype = _int
         L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_decode_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
+        L.orin_fa_decode_store_ind.restype = _int
         L.orin_fa_rope_batch.argtypes = [_vp, _int, _int, _int, _flt, _int, _int, _vp, _int]
         L.orin_fa_rope_batch.restype = _int
         L.orin_fa_rope_ind.argtypes = [_vp, _int, _int, _int, _flt, _vp, _vp, _int]
@@ -112,6 +114,15 @@ def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_
                                   _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def flash_attention_decode_store_ind(q, k_new, v_new, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):
+    """kv_store_ind(kc, vc, k_new, v_new, n_kv, ...) followed by flash_attention_decode_ind(...), in the
+    launches of the latter alone (no counterpart in the reference; the results are identical)."""
+    rc = lib().orin_fa_decode_store_ind(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(kc), _ptr(vc), _ptr(out),
+                                        n_head, n_kv, head_dim, n_ctx, _ptr(d_pos), scale)
+    if rc != 0:
+        raise OrinFaError("flash_attention_decode_store_ind", rc)
 
 
 def rope_neox_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors=None):

@@ -171,6 +171,49 @@ def test_store_then_attend_equals_attending_a_prebuilt_cache(fa):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,n_ctx", [(12, 2, 128, 4096), (28, 4, 128, 32768), (8, 8, 64, 600), (40, 2, 128, 1024)])
+def test_decode_store_equals_store_then_decode(fa, H, G, d, n_ctx):
+    """The fused entry point against the two calls it stands for (reference call site:
+    src/model_gpu.cu:281-282): same cache bytes and same output, bit for bit, at positions on
+    both sides of tile and split edges, at the last row of the cache, out of range, and replayed
+    from a graph with the position changed on the device."""
+    import torch
+    scale = float(1.0 / np.sqrt(d))
+    rng = np.random.default_rng(H + n_ctx)
+    base_k = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    base_v = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    q = torch.from_numpy(rng.standard_normal((H, d)).astype(np.float32)).cuda()
+    k_new = torch.zeros((G, d), device="cuda")
+    v_new = torch.zeros((G, d), device="cuda")
+    dpos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ka, va = torch.from_numpy(base_k).cuda(), torch.from_numpy(base_v).cuda()   # two calls
+    kb, vb = ka.clone(), va.clone()                                             # fused
+    out_a = torch.empty((H, d), device="cuda")
+    out_b = torch.empty((H, d), device="cuda")
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            fa.set_stream(torch.cuda.current_stream().cuda_stream)
+            fa.flash_attention_decode_store_ind(q, k_new, v_new, kb, vb, out_b, H, G, d, n_ctx, dpos, scale)
+    finally:
+        fa.set_stream(torch.cuda.current_stream().cuda_stream)
+    positions = [0, 1, 30, 31, 32, 33, 255, 256, 257, n_ctx // 2 - 1, n_ctx // 2, n_ctx - 2, n_ctx - 1, n_ctx, -1]
+    for i, pos in enumerate(positions):
+        k_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        v_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        dpos.fill_(pos)
+        fa.kv_store_ind(ka, va, k_new, v_new, G, d, n_ctx, dpos)
+        fa.flash_attention_decode_ind(q, ka, va, out_a, H, G, d, n_ctx, dpos, scale)
+        if i % 2 == 0:
+            g.replay()
+        else:
+            fa.flash_attention_decode_store_ind(q, k_new, v_new, kb, vb, out_b, H, G, d, n_ctx, dpos, scale)
+        torch.cuda.synchronize()
+        assert torch.equal(ka, kb) and torch.equal(va, vb), pos
+        assert torch.equal(out_a.view(torch.int32), out_b.view(torch.int32)), pos
+
+
+@pytest.mark.gpu
 def test_kv_mutators_reject_bad_arguments(fa):
     import torch
     from orin_llm_amd.kernels import OrinFaError
