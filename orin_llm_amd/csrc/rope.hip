@@ -9,9 +9,9 @@
 //
 // Every head of a token shares the token's angles, so one thread owns (token, pair, group of up
 // to 8 heads): the block's first threads compute the frequency of each pair once into LDS, each
-// thread forms its angle and one sine/cosine, then rotates its heads with all loads issued
-// before the first store -- where the reference spends a power, a sine and a cosine per element
-// pair of every head.
+// thread forms its angle and one sine/cosine, then rotates its heads; all loads are issued
+// before any of that arithmetic -- where the reference spends a power, a sine and a cosine per
+// element pair of every head.
 // Arithmetic follows the CPU statement operation by operation in fp32 (no contraction of
 // the rotation into fused multiply-adds); the frequency is the double-precision power rounded
 // to fp32, which is what a correctly rounded powf returns, because at position 32768 one ulp
@@ -36,19 +36,33 @@ __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int hea
     // pair index fastest, then head group, then token; a block covers whole runs of pairs when
     // half divides 256, otherwise every thread computes its own frequency
     const bool shared_freq = half <= 128 && (256 % half) == 0;
-    if (shared_freq && (int)threadIdx.x < half) {
-        const int i = threadIdx.x;
-        const float expo = -2.0f * (float)i / (float)n_rot;
-        float f = (float)pow((double)theta, (double)expo);
-        if (freq_factors) f /= freq_factors[i];
-        sh_freq[i] = f;
-    }
-    if (shared_freq) __syncthreads();
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
-    if (t >= (long long)tokens * n_hgroups * half) return;
+    const bool active = t < (long long)tokens * n_hgroups * half;
     const int i = (int)(t % half);
     const long long th = t / half;
     const int hgroup = (int)(th % n_hgroups), token = (int)(th / n_hgroups);
+    const int h0 = hgroup * kHeadsPerThread;
+    float* row = x + ((size_t)token * heads + h0) * head_dim;
+    const int i0 = NEOX ? i : 2 * i, i1 = NEOX ? i + half : 2 * i + 1;
+    // The loads go out first: nothing they need depends on the angle, and the power, sine and
+    // cosine below then run while the rows are on their way.
+    float x0[kHeadsPerThread], x1[kHeadsPerThread];
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread; ++u)
+        if (active && h0 + u < heads) {
+            x0[u] = row[(size_t)u * head_dim + i0];
+            x1[u] = row[(size_t)u * head_dim + i1];
+        }
+    const int pos = IND ? *d_pos : n_past + token;
+    if (shared_freq && (int)threadIdx.x < half) {
+        const int fi = threadIdx.x;
+        const float expo = -2.0f * (float)fi / (float)n_rot;
+        float f = (float)pow((double)theta, (double)expo);
+        if (freq_factors) f /= freq_factors[fi];
+        sh_freq[fi] = f;
+    }
+    if (shared_freq) __syncthreads();
+    if (!active) return;
     float freq;
     if (shared_freq) {
         freq = sh_freq[i];
@@ -57,19 +71,8 @@ __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int hea
         freq = (float)pow((double)theta, (double)expo);
         if (freq_factors) freq /= freq_factors[i];
     }
-    const int pos = IND ? *d_pos : n_past + token;
     const float ang = (float)pos * freq;
     const float c = cosf(ang), s = sinf(ang);
-    const int h0 = hgroup * kHeadsPerThread;
-    float* row = x + ((size_t)token * heads + h0) * head_dim;
-    const int i0 = NEOX ? i : 2 * i, i1 = NEOX ? i + half : 2 * i + 1;
-    float x0[kHeadsPerThread], x1[kHeadsPerThread];
-#pragma unroll
-    for (int u = 0; u < kHeadsPerThread; ++u)
-        if (h0 + u < heads) {
-            x0[u] = row[(size_t)u * head_dim + i0];
-            x1[u] = row[(size_t)u * head_dim + i1];
-        }
 #pragma unroll
     for (int u = 0; u < kHeadsPerThread; ++u)
         if (h0 + u < heads) {
