@@ -440,30 +440,31 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
                 pin_v(s[0][cb]); // (the reads below stay behind the settled pipe)
                 if (R > 0) pin_v(s[1][cb]);
                 float v[16];
-                float mx = -INFINITY;
+                float mxp[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}; // four chains instead of one long one
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     v[r] = s[0][cb][r];
                     if (masked && row0 + 8 * (r / 4) + (r % 4) >= limit[cb]) v[r] = -INFINITY;
-                    mx = fmaxf(mx, v[r]);
+                    mxp[r % 4] = fmaxf(mxp[r % 4], v[r]);
                 }
                 if (R > 0) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[1][cb][r]);
+                    for (int r = 0; r < 16; ++r) mxp[r % 4] = fmaxf(mxp[r % 4], s[1][cb][r]);
                 }
-                mx = pair_max(mx);
+                const float mx = pair_max(fmaxf(fmaxf(mxp[0], mxp[1]), fmaxf(mxp[2], mxp[3])));
                 nb[cb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
-                float sum = 0.0f;
+                float sump[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int kh = 0; kh < 2; ++kh) {
                     h8 ph;
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         ph[j] = (_Float16)fast_exp2(__builtin_fmaf(v[kh * 8 + j], a.c, nb[cb]));
-                        sum += (float)ph[j];
+                        sump[j % 4] += (float)ph[j];
                     }
                     pw[0][cb][kh] = __builtin_bit_cast(u32x4, ph);
                 }
+                const float sum = (sump[0] + sump[1]) + (sump[2] + sump[3]);
                 lsum[cb][0] = sum;
                 lsum[cb][1] = 0.0f;
             }
