@@ -8,7 +8,8 @@ stack of synthetic inputs already resident in HBM (independent seeds and buffers
 
   qwen1.5b-prefill512   (default; BASELINE configs[1]) 28 layers x two 512-token causal chunks,
                         at cache depth 0 and 3584, 12 Q heads / 2 KV heads, d=128, K with 4
-                        outlier channels x8.  value = causal-exact TFLOP/s.
+                        outlier channels x8.  value = causal-exact TFLOP/s (step launched eagerly and as
+                        one HIP graph; the faster counts, both are reported).
   llama8b-prefill512-d4096, qwen7b-prefill512-d32256, qwen1.5b-decode-32k, llama8b-decode-8k,
   qwen7b-decode-32k     the other BASELINE shapes; the north-star cases are also run after the
                         default workload and reported under "also".
@@ -189,7 +190,26 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
     for i in range(steps):
         one_step(evs[i])
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall_eager = time.perf_counter() - t0
+
+    # The same step captured once as a HIP graph and replayed (the operator is capture-safe: no
+    # allocation, no synchronisation); the host may launch it either way, the faster one counts.
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            one_step()
+    finally:
+        kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+    for _ in range(warmup):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        g.replay()
+    torch.cuda.synchronize()
+    wall_graph = time.perf_counter() - t0
+    wall = min(wall_eager, wall_graph)
 
     # Per-launch duration of the dominant kernel: one event pair around every single launch of
     # one pass over the stack (the events sit on the stream the kernels are launched on).
@@ -225,6 +245,7 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
                       note="launch_us: median of event pairs around single launches; "
                            "launch_us_back_to_back: stack average including launch gaps"),
         per_chunk=per_chunk,
+        eager=dict(ms_per_step=wall_eager / steps * 1e3), graph=dict(ms_per_step=wall_graph / steps * 1e3),
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="sampled, layer 0, vs CPU oracle"),
     )
     if with_cpu:
