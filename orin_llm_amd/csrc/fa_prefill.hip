@@ -71,7 +71,7 @@ struct PGeom {
 // Instructions with the register file of each operand spelled out.  The kernel keeps its score
 // accumulators in ordinary vector registers (the exponentials read them with no copy) and its
 // output accumulators and the query operands in the accumulation-register file, and it fixes the
-// issue order of matrix and vector work by hand -- neither of which the builtin forms allow.
+// place of every matrix instruction in the stream by hand -- neither of which the builtin forms allow.
 // The price: the compiler knows nothing about the hazards of these blocks.
 //   (1) Result latency: a non-matrix instruction reads a matrix result only a pipeline stage
 //       (at least two later matrix instructions) after it was issued, or behind settle().
@@ -178,9 +178,9 @@ __device__ __forceinline__ void lds_copy_1k(i32x4 desc, int off, int soff) {
 
 // The vector instructions of stage B for one 32x32 score block (16 scores per lane), in issue
 // order.  Pair p = scores (2p, 2p+1).  Kinds: 0 multiply-add (the exponent), 1 exponential,
-// 2 conversion of a pair to packed fp16, 3 row-sum and running-maximum update from a pair.  The four kinds run
-// as a software pipeline one pair apart, so no instruction reads a result younger than three
-// instructions.
+// 2 conversion of a pair to packed fp16, 3 addition of the converted pair to the tile's packed
+// partial row sums.  The four kinds run as a software pipeline one pair apart, so that nothing
+// waits for the result of the instruction right before it.
 struct ItemTable {
     int kind[48];
     int arg[48];
