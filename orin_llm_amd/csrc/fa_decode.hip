@@ -91,8 +91,20 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 #pragma unroll
         for (int i = 0; i < G::kLoads; ++i) vreg[i] = buf_load16<true>(vrs, soff + (i * 64 + lane) * 16);
     };
+    // ---- query heads: requested before the first tile, so that they arrive before it (a wave's
+    // loads complete in order) and the score product can start while V is still on its way ----
+    const int hl = hg * 16 + col;
+    const bool valid = hl < a.r;
+    const float* qp = a.q + (size_t)(valid ? kvh * a.r + hl : 0) * D;
+    const float qmul = valid ? a.qsign : 0.0f;
+    float4 qx[2 * G::kSteps];
+#pragma unroll
+    for (int kk = 0; kk < G::kSteps; ++kk) {
+        qx[2 * kk] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
+        qx[2 * kk + 1] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+    }
     int tile = tile_first;
-    fetch_k(tile); // in flight while the position and the query heads are loaded
+    fetch_k(tile); // in flight while the position is loaded
     fetch_v(tile);
     // The new row's pieces a lane would substitute do not depend on where the row falls: lane
     // (col, grp) holds bytes (kk*4 + grp)*16 of a K row and piece lane % (D/8) of a V row.  They
@@ -121,15 +133,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 
     FA_STAMP(1);
     // ---- query heads -> B operands, fp16 hi + lo ----
-    const int hl = hg * 16 + col;
-    const bool valid = hl < a.r;
-    const float* qp = a.q + (size_t)(valid ? kvh * a.r + hl : 0) * D;
-    const float qmul = valid ? a.qsign : 0.0f;
     h8 qhi[G::kSteps], qlo[G::kSteps];
 #pragma unroll
     for (int kk = 0; kk < G::kSteps; ++kk) {
-        const float4 x0 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
-        const float4 x1 = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+        const float4 x0 = qx[2 * kk], x1 = qx[2 * kk + 1];
         const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
