@@ -55,6 +55,7 @@ WORKLOADS = {
     # the decode layer's call pair (store the token's K/V rows, then attend; reference src/model_gpu.cu:281-282)
     # through the entry point that does both in the attention launches; the two calls are timed beside it
     "qwen1.5b-decode-store-32k": ("qwen1.5b", "decode_store", 32768, 32768),
+    "qwen1.5b-decode-rope-store-32k": ("qwen1.5b", "decode_rope_store", 32768, 32768),
     # the two mutators of the cache (byte movers; value = bytes read + written per second)
     "llama8b-kv-store-512": ("llama8b", "kv_store", 8192, (4096, 512)),
     "qwen1.5b-kv-shift-32k": ("qwen1.5b", "kv_shift", 32768, (4, 16382)),
@@ -77,6 +78,7 @@ TRAFFIC = {
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
 ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k", "qwen1.5b-decode-store-32k",
+        "qwen1.5b-decode-rope-store-32k",
         "llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
 
 
@@ -275,23 +277,40 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
             stack.append((q[0].contiguous(), k, v, torch.empty((H, d), dtype=torch.float32, device="cuda")))
         stacks.append(stack)
     dpos = torch.tensor([L - 1], dtype=torch.int32, device="cuda")
-    store = WORKLOADS[name][1] == "decode_store"
+    rope = WORKLOADS[name][1] == "decode_rope_store"
+    store = rope or WORKLOADS[name][1] == "decode_store"
+    theta = 1.0e6  # Qwen2.5's rope base; "neox" pairing over the whole head
     gen = torch.Generator(device="cuda")
     gen.manual_seed(99)
     k_new = torch.randn((G, d), generator=gen, device="cuda", dtype=torch.float32)
     v_new = torch.randn((G, d), generator=gen, device="cuda", dtype=torch.float32)
 
+    angles = torch.zeros((d // 2, 2), device="cuda")
+
     def one_stack(si):
+        if rope:  # the token's angles once, then every layer
+            kernels.rope_angles_ind(angles, d, theta, dpos)
         for q, k, v, out in stacks[si]:
-            if store:
+            if rope:
+                kernels.flash_attention_decode_rope_store_ind(q, k_new, v_new, k, v, out, H, G, d, n_ctx, dpos, scale,
+                                                              d, theta, None, True, angles)
+            elif store:
                 kernels.flash_attention_decode_store_ind(q, k_new, v_new, k, v, out, H, G, d, n_ctx, dpos, scale)
             else:
                 kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
 
+    q_sep, k_sep = stacks[0][0][0].clone(), k_new.clone()  # rotated in place over and over by the separate calls
+
     def one_stack_two_calls(si):
         for q, k, v, out in stacks[si]:
-            kernels.kv_store_ind(k, v, k_new, v_new, G, d, n_ctx, dpos)
-            kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
+            if rope:
+                kernels.rope_neox_ind(q_sep, H, d, d, theta, dpos)
+                kernels.rope_neox_ind(k_sep, G, d, d, theta, dpos)
+                kernels.kv_store_ind(k, v, k_sep, v_new, G, d, n_ctx, dpos)
+                kernels.flash_attention_decode_ind(q_sep, k, v, out, H, G, d, n_ctx, dpos, scale)
+            else:
+                kernels.kv_store_ind(k, v, k_new, v_new, G, d, n_ctx, dpos)
+                kernels.flash_attention_decode_ind(q, k, v, out, H, G, d, n_ctx, dpos, scale)
 
     # eager
     for i in range(warmup):
@@ -330,8 +349,8 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     wall_graph = time.perf_counter() - t0
     dev_graph_ms = e0.elapsed_time(e1)
 
-    two_calls_us = None
-    if store:  # the same step as the reference makes it: two calls per layer
+    two_calls_us = two_calls_graph_us = None
+    if store:  # the same step as the reference makes it: two (with the rotary embedding four) calls per layer
         for i in range(warmup):
             one_stack_two_calls(i % n_stacks)
         torch.cuda.synchronize()
@@ -341,6 +360,26 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
         e1.record()
         torch.cuda.synchronize()
         two_calls_us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+        sep_graphs = []
+        for si in range(n_stacks):
+            g = torch.cuda.CUDAGraph()
+            try:
+                with torch.cuda.graph(g):
+                    kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+                    one_stack_two_calls(si)
+            finally:
+                kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            sep_graphs.append(g)
+        for i in range(warmup):
+            sep_graphs[i % n_stacks].replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(steps):
+            sep_graphs[i % n_stacks].replay()
+        e1.record()
+        torch.cuda.synchronize()
+        two_calls_graph_us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+        del sep_graphs
 
     # Duration of each of the two kernels: events between them, recorded by the library on its stream.
     split_us, combine_us = [], []
@@ -351,7 +390,14 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
             combine_us.append(b)
     split_us, combine_us = float(np.median(split_us)), float(np.median(combine_us))
 
+    if store:  # the check below is of the entry point this workload names, not of the last writer of `out`
+        one_stack((steps - 1) % n_stacks)
+        torch.cuda.synchronize()
     q, k, v, out = stacks[(steps - 1) % n_stacks][0]
+    if rope:  # the oracle attends with the rotated query; the cache already holds the rotated row
+        q = q.clone()
+        kernels.rope_neox_ind(q, H, d, d, theta, dpos)
+        torch.cuda.synchronize()
     rows = np.array([(0, h) for h in range(H)], np.int32)
     want = ref.flash_attention_rows(q.cpu().numpy()[None], k.view(torch.uint16).cpu().numpy(),
                                     v.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, L - 1,
@@ -377,9 +423,15 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="all heads, layer 0, vs CPU oracle"),
     )
     if store:
-        res["roofline"]["kernel"] = f"fa_decode_split_kernel<{d}, store> + fa_decode_combine_kernel<{d}> (one layer)"
-        res["roofline"]["launch_us_two_calls"] = two_calls_us
-        res["roofline"]["note"] += "; launch_us_two_calls: kv_store_ind + flash_attention_decode_ind per layer, eager, back to back"
+        mode = "rotate + store" if rope else "store"
+        res["roofline"]["kernel"] = f"fa_decode_split_kernel<{d}, {mode}> + fa_decode_combine_kernel<{d}> (one layer)"
+        res["roofline"]["launch_us_eager"] = dev_eager_ms * 1e3 / (steps * layers)
+        res["roofline"]["launch_us_graph"] = dev_graph_ms * 1e3 / (steps * layers)
+        res["roofline"]["launch_us_separate_calls"] = two_calls_us
+        res["roofline"]["launch_us_separate_calls_graph"] = two_calls_graph_us
+        sep = ("rope_neox_ind on q, rope_neox_ind on the new K row, kv_store_ind, flash_attention_decode_ind" if rope
+               else "kv_store_ind + flash_attention_decode_ind")
+        res["roofline"]["note"] += f"; launch_us_separate_calls: {sep} per layer, back to back, eager and replayed from a graph"
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline_decode(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
                                                   v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, L, scale)
@@ -548,7 +600,7 @@ def run_copy(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "copy": run_copy, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 

@@ -118,6 +118,29 @@ int orin_fa_kv_shift(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head
 int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
                              float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
 
+/* The decode layer's four calls around the cache -- rope_*_ind on q, rope_*_ind on the new K row,
+ * kv_store_ind, flash_attention_decode_ind (reference: src/model_gpu.cu:277-282) -- in the
+ * launches of the last alone.  No counterpart in the reference.  q [n_head][head_dim] and k_new
+ * [n_kv][head_dim] arrive BEFORE the rotary embedding and are left as they are; every workgroup
+ * rotates what it needs with the arithmetic of orin_fa_rope_ind (n_rot, theta, freq_factors,
+ * neox as there), so the cache contents and the output equal those of the four calls bit for
+ * bit.  Supported: the "normal" pairing with any even n_rot <= head_dim, the "neox" pairing
+ * with n_rot = head_dim (or n_rot = 0: no rotation); anything else returns ORIN_FA_E_INVALID and
+ * the separate calls apply.  Capture-safe like orin_fa_decode_ind.
+ * angles: NULL, or the table orin_fa_rope_angles_ind wrote for the same n_rot, theta,
+ * freq_factors and *d_pos (theta and freq_factors are then not used): every layer of a decode
+ * step rotates by the same angles, and with the table no workgroup spends its first
+ * microsecond and a half on the powers, sines and cosines.  Same results bit for bit. */
+int orin_fa_decode_rope_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
+                                  float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
+                                  int n_rot, float theta, const float* freq_factors, int neox, const float* angles);
+
+/* (cos, sin) of the n_rot/2 rotary pairs at position *d_pos (read on the device), as
+ * orin_fa_rope_ind forms them, into angles [n_rot/2][2] (device, 8-byte aligned).  No
+ * counterpart in the reference, whose kernels recompute them per element pair
+ * (src/kernels.cu:1619-1657); for orin_fa_decode_rope_store_ind, once per token. */
+int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* freq_factors, const int* d_pos);
+
 /* Measurement aid with no counterpart in the reference: orin_fa_decode_ind with HIP events
  * recorded before, between and after its two kernels on the library's stream.  Synchronises
  * on the last event and returns the elapsed time of the split kernel and of the combine

@@ -129,9 +129,16 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 }
 
 namespace {
+struct RopeArgs {
+    int n_rot;
+    float theta;
+    const float* freq_factors;
+    int neox;
+    const float* angles;
+};
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
                 int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
-                const float* k_new, const float* v_new);
+                const float* k_new, const float* v_new, const RopeArgs* rope = nullptr);
 }
 
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
@@ -144,6 +151,27 @@ int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_
     if (!k_new || !v_new) return ORIN_FA_E_INVALID;
     if (((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15u) != 0) return ORIN_FA_E_INVALID;
     return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, k_new, v_new);
+}
+
+int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* freq_factors, const int* d_pos) {
+    if (!angles || !d_pos || n_rot <= 0 || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    if (reinterpret_cast<uintptr_t>(angles) & 7u) return ORIN_FA_E_INVALID;
+    return hip_code(rope_angles_launch(angles, n_rot, theta, d_pos, freq_factors, g_state.stream));
+}
+
+int orin_fa_decode_rope_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
+                                  float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
+                                  int n_rot, float theta, const float* freq_factors, int neox, const float* angles) {
+    if (!k_new || !v_new) return ORIN_FA_E_INVALID;
+    if (reinterpret_cast<uintptr_t>(angles) & 7u) return ORIN_FA_E_INVALID;
+    if (((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15u) != 0) return ORIN_FA_E_INVALID;
+    if (n_rot < 0 || n_rot > head_dim || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    // the pairs must lie inside one lane's share of a row: always so for the "normal" pairing, and for
+    // "neox" when the rotation spans the whole head
+    if (neox && n_rot != 0 && n_rot != head_dim) return ORIN_FA_E_INVALID;
+    const RopeArgs rope{n_rot, theta, freq_factors, neox != 0, angles};
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, k_new, v_new,
+                       n_rot > 0 ? &rope : nullptr);
 }
 
 int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
@@ -170,13 +198,17 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
 namespace {
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
                 int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
-                const float* k_new, const float* v_new) {
+                const float* k_new, const float* v_new, const RopeArgs* rope) {
     int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
     if (rc != ORIN_FA_OK) return rc;
     if (!d_pos) return ORIN_FA_E_INVALID;
     FaArgs a{};
     a.q = q; a.kc = kc; a.vc = vc; a.out = out; a.d_pos = d_pos;
     a.k_new = k_new; a.v_new = v_new;
+    if (rope) {
+        a.n_rot = rope->n_rot; a.theta = rope->theta; a.freq_factors = rope->freq_factors; a.neox = rope->neox;
+        a.rope_angles = rope->angles;
+    }
     a.n_head = n_head; a.n_kv = n_kv; a.n_ctx = n_ctx; a.batch = 1;
     a.r = n_head / n_kv;
     a.n_hgroups = (a.r + 15) / 16;

@@ -39,6 +39,10 @@ struct FaArgs {
     const int* d_pos; // decode only
     const float* k_new; // decode with store: the current token's K and V rows, fp32 [n_kv][head_dim];
     const float* v_new; // null for plain decode (the cache pointers are then never written through)
+    const float* freq_factors; // decode with rotary embedding of q and k_new (n_rot > 0), as rope_launch takes them
+    const float* rope_angles;  // optional: (cos, sin) of every pair at this token's position, [n_rot/2][2], from rope_angles_launch
+    int n_rot, neox;
+    float theta;
     int n_head, n_kv, n_ctx;
     int n_past, batch; // prefill only
     int r;             // query heads per KV head
@@ -69,6 +73,8 @@ hipError_t kv_shift_launch(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, in
 // Rotary embedding (rope.hip).  d_pos not null selects the single-token form.
 hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
                        const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream);
+hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
+                              hipStream_t stream);
 
 template <int N>
 struct IntC {
@@ -130,6 +136,30 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The rotary embedding's arithmetic, in one place for the kernels that apply it (rope.hip and the
+// decode kernel that rotates its own q and k).  It follows the CPU statement (reference:
+// src/model_cpu.cpp:179-203) operation by operation in fp32, without contraction into fused
+// multiply-adds; the frequency is the double-precision power rounded to fp32, which is what a
+// correctly rounded powf returns (at position 32768 one ulp of the frequency moves the angle by
+// 2e-3 rad).
+__device__ __forceinline__ float rope_freq_base(int i, int n_rot, float theta) {
+#pragma clang fp contract(off)
+    const float expo = -2.0f * (float)i / (float)n_rot;
+    return (float)pow((double)theta, (double)expo);
+}
+__device__ __forceinline__ float rope_freq(int i, int n_rot, float theta, const float* freq_factors) {
+    float f = rope_freq_base(i, n_rot, theta);
+    if (freq_factors) f /= freq_factors[i];
+    return f;
+}
+__device__ __forceinline__ void rope_rotate(float& x0, float& x1, float c, float s) {
+#pragma clang fp contract(off)
+    const float r0 = x0 * c - x1 * s;
+    const float r1 = x0 * s + x1 * c;
+    x0 = r0;
+    x1 = r1;
 }
 
 } // namespace orin_fa

@@ -47,11 +47,19 @@ struct DGeom {
     static constexpr int kLdsB = kMlOff + kDecodeWaves * 16 * 2 * 4;
 };
 
-// STORE: the current token's K and V rows arrive as fp32 beside the cache (FaArgs::k_new, v_new).
-// The wave whose tile holds row *d_pos takes that row from them -- rounded to fp16 exactly as
-// the store kernel rounds -- instead of from the cache, and writes it to the cache on the way:
+// MODE 1 (store): the current token's K and V rows arrive as fp32 beside the cache (FaArgs::k_new,
+// v_new).  The wave whose tile holds row *d_pos takes that row from them -- rounded to fp16 exactly
+// as the store kernel rounds -- instead of from the cache, and writes it to the cache on the way:
 // the store kernel's launch is saved and the result is the same bit for bit.
-template <int D, bool STORE>
+// MODE 2 (rotate + store): q and k_new arrive before the rotary embedding, and every workgroup
+// rotates them itself (the inputs stay as they are): the first n_rot/2 lanes of every wave put
+// the angles' cosines and sines (computed, or read from the caller's table) into the wave's own
+// LDS table while the first tile is on its way, and the pairs a lane rotates are ones it holds
+// anyway -- "normal" pairs are neighbours, and for "neox" with
+// n_rot = head_dim element e pairs with e + head_dim/2, the same lane's k-step two (one, at
+// head_dim 64) further on.  Same arithmetic as the rotary kernel, so again bit for bit what the
+// separate launches give, four launches in the place of seven.
+template <int D, int MODE>
 __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(const FaArgs a) {
     using G = DGeom<D>;
     constexpr int kWaves = kDecodeWaves;
@@ -93,6 +101,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     };
     // ---- query heads: requested before the first tile, so that they arrive before it (a wave's
     // loads complete in order) and the score product can start while V is still on its way ----
+    const int pos = *a.d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
     const int hl = hg * 16 + col;
     const bool valid = hl < a.r;
     const float* qp = a.q + (size_t)(valid ? kvh * a.r + hl : 0) * D;
@@ -103,41 +112,114 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         qx[2 * kk] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
         qx[2 * kk + 1] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
     }
+    constexpr bool STORE = MODE != 0, ROPE = MODE == 2;
+    // (rotate + store) lane i < n_rot/2 of every wave fetches what pair i's angle needs: its
+    // cosine and sine when the caller supplies them, else its frequency factor if there is one.
+    // Both loads are made by every lane, from an address that can be read either way (the query,
+    // when the array is absent): a load under a branch makes the compiler wait for every load
+    // issued so far where the branch ends.
+    float2 cs_given = float2{1.0f, 0.0f};
+    float ff_given = 1.0f;
+    if constexpr (ROPE) {
+        const int pi = min(lane, a.n_rot / 2 - 1);
+        const float* anp = a.rope_angles ? a.rope_angles + 2 * pi : a.q;
+        const float* ffp = a.freq_factors ? a.freq_factors + pi : a.q;
+        cs_given = *reinterpret_cast<const float2*>(anp);
+        ff_given = *ffp;
+    }
+    __builtin_amdgcn_sched_barrier(0); // the small loads first: they return first, and nothing that needs them waits for a tile
+
     int tile = tile_first;
     fetch_k(tile); // in flight while the position is loaded
     fetch_v(tile);
-    // The new row's pieces a lane would substitute do not depend on where the row falls: lane
-    // (col, grp) holds bytes (kk*4 + grp)*16 of a K row and piece lane % (D/8) of a V row.  They
-    // are requested now, by every lane, before the position is known.
-    u32x4 k_new16[G::kSteps], v_new16;
-    if constexpr (STORE) {
-        auto load8 = [&](const float* p) {
-            const float4 x0 = *reinterpret_cast<const float4*>(p);
-            const float4 x1 = *reinterpret_cast<const float4*>(p + 4);
-            h8 h;
-            h[0] = (_Float16)x0.x; h[1] = (_Float16)x0.y; h[2] = (_Float16)x0.z; h[3] = (_Float16)x0.w;
-            h[4] = (_Float16)x1.x; h[5] = (_Float16)x1.y; h[6] = (_Float16)x1.z; h[7] = (_Float16)x1.w;
-            return __builtin_bit_cast(u32x4, h);
-        };
-#pragma unroll
-        for (int kk = 0; kk < G::kSteps; ++kk) k_new16[kk] = load8(a.k_new + (size_t)kvh * D + (kk * 4 + grp) * 8);
-        v_new16 = load8(a.v_new + (size_t)kvh * D + (lane % G::kChunksPerRow) * 8);
-    }
+    // Every load above is used only behind the early return below, and left alone the compiler
+    // moves them all there: position, then query, then the query's conversion, and only then the
+    // first tile -- three memory latencies one after another.  A statement that may write memory
+    // keeps them on this side of the branch, where they overlap the load of the position.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
-    const int pos = *a.d_pos;
     int p = pos < 0 ? 0 : pos;
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
     const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
     if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
 
+    // The new row, requested by the one wave whose tiles include the row's (its last one, so the
+    // row has long arrived when it is wanted) in as few loads as will do.  K: elements 4*lane ..
+    // 4*lane+3 (the lanes hand each other the pieces they hold of a K row through LDS then); V:
+    // piece lane % (D/8), which is what the lane holds of a V row.  The other waves make the same
+    // loads from the query, which their cache holds: no branch, so no wait where one would end.
+    float4 k_raw = float4{0.f, 0.f, 0.f, 0.f}, v_raw[2] = {k_raw, k_raw};
+    if constexpr (STORE) {
+        const int pt = pos / kTile;
+        const bool owner = store && pt >= tile_first && (pt - tile_first) % tile_step == 0;
+        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : a.q) + (lane % (D / 4)) * 4;
+        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : a.q) + (lane % G::kChunksPerRow) * 8;
+        k_raw = *reinterpret_cast<const float4*>(kp4);
+        v_raw[0] = *reinterpret_cast<const float4*>(vp8);
+        v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
+    }
     FA_STAMP(1);
+    float qf[G::kSteps][8]; // this lane's 8 elements of every k-step: head_dim indices kk*32 + grp*8 + 0..7
+#pragma unroll
+    for (int kk = 0; kk < G::kSteps; ++kk) {
+        const float4 x0 = qx[2 * kk], x1 = qx[2 * kk + 1];
+        qf[kk][0] = x0.x; qf[kk][1] = x0.y; qf[kk][2] = x0.z; qf[kk][3] = x0.w;
+        qf[kk][4] = x1.x; qf[kk][5] = x1.y; qf[kk][6] = x1.z; qf[kk][7] = x1.w;
+    }
+    // (rotate + store) the rotation of this lane's 8 elements of every k-step, by the wave's table
+    __shared__ float sh_cs_all[ROPE ? kWaves : 1][D / 2][2];
+    __shared__ __attribute__((aligned(16))) float sh_krow_all[STORE ? kWaves : 1][D];
+    float (*const sh_cs)[2] = sh_cs_all[ROPE ? wave : 0];
+    // x0, x1: this lane's elements of k-steps kk and kk + kSteps/2 (head_dim indices kk*32 + grp*8 + e
+    // and the same + head_dim/2)
+    auto rotate2 = [&](float (&x0)[8], float (&x1)[8], int kk) {
+        if (a.neox) { // n_rot == D (checked by the host): element e pairs with e + D/2
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int i = kk * 32 + grp * 8 + e;
+                rope_rotate(x0[e], x1[e], sh_cs[i][0], sh_cs[i][1]);
+            }
+        } else {      // elements 2i and 2i + 1, below n_rot
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const int el0 = kk * 32 + grp * 8 + e, el1 = el0 + D / 2;
+                if (el0 < a.n_rot) rope_rotate(x0[e], x0[e + 1], sh_cs[el0 / 2][0], sh_cs[el0 / 2][1]);
+                if (el1 < a.n_rot) rope_rotate(x1[e], x1[e + 1], sh_cs[el1 / 2][0], sh_cs[el1 / 2][1]);
+            }
+        }
+    };
+    if constexpr (ROPE) {
+        // (cos, sin) of pair i at the raw position, as the rotary kernel forms them
+        // A table per wave (head_dim <= 128: a wave's 64 lanes cover the pairs), so that no wave
+        // waits here for the others: the waves of a workgroup get their loads out at very
+        // different times when the whole chip is requesting its first tiles.  Write and reads
+        // are the same wave's, and a wave's LDS operations complete in order.
+        static_assert(D / 2 <= 64, "one lane per pair");
+        const int half = a.n_rot / 2;
+        if (lane < half) {
+            if (!a.rope_angles) {
+                float freq = rope_freq_base(lane, a.n_rot, a.theta);
+                if (a.freq_factors) freq /= ff_given;
+                const float ang = (float)pos * freq;
+                cs_given.x = cosf(ang);
+                cs_given.y = sinf(ang);
+            }
+            sh_cs[lane][0] = cs_given.x;
+            sh_cs[lane][1] = cs_given.y;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps / 2; ++kk) rotate2(qf[kk], qf[kk + G::kSteps / 2], kk);
+    }
     // ---- query heads -> B operands, fp16 hi + lo ----
     h8 qhi[G::kSteps], qlo[G::kSteps];
 #pragma unroll
     for (int kk = 0; kk < G::kSteps; ++kk) {
-        const float4 x0 = qx[2 * kk], x1 = qx[2 * kk + 1];
-        const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        const float* x = qf[kk];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float xe = x[e] * qmul;
@@ -161,13 +243,56 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
             if (store && tile == pos / kTile) { // the tile of the new row (the last visible one)
                 const int row = pos % kTile;
                 const size_t row_off = ((size_t)kvh * a.n_ctx + pos) * D;
-                if (col == row % 16) {
+                // (Nothing below may be started ahead of this branch: the compiler would otherwise
+                // convert the new row before the loop, in every wave, and wait there for the row's
+                // loads -- the last ones issued, so for the whole first tile.)
+                auto here = [](float x) { // a copy the compiler cannot make anywhere else
+                    float y;
+                    asm volatile("v_mov_b32 %0, %1" : "=v"(y) : "v"(x));
+                    return y;
+                };
+                const float4 k_own = float4{here(k_raw.x), here(k_raw.y), here(k_raw.z), here(k_raw.w)};
+                const float4 v_own[2] = {float4{here(v_raw[0].x), here(v_raw[0].y), here(v_raw[0].z), here(v_raw[0].w)},
+                                         float4{here(v_raw[1].x), here(v_raw[1].y), here(v_raw[1].z), here(v_raw[1].w)}};
+                auto put_k = [&](int kk, u32x4 piece) { // into the operand registers and (one head group's wave) the cache
+                    if (col == row % 16) {
+                        kreg[(row / 16) * G::kSteps + kk] = piece;
+                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.kc) + row_off + (kk * 4 + grp) * 8) = piece;
+                    }
+                };
+                {
+                    // The new K row is rotated (rotate + store) and converted here, by the one wave
+                    // that needs it.  It has waited in four registers a lane; the lanes now hand
+                    // each other the pieces they hold of a K row through the wave's LDS row.
+                    float* const krow = sh_krow_all[wave];
+                    if (lane < D / 4) *reinterpret_cast<float4*>(krow + lane * 4) = k_own;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-                    for (int kk = 0; kk < G::kSteps; ++kk) {
-                        kreg[(row / 16) * G::kSteps + kk] = k_new16[kk];
-                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.kc) + row_off + (kk * 4 + grp) * 8) = k_new16[kk];
+                    for (int kk = 0; kk < G::kSteps / 2; ++kk) { // two k-steps at a time: the pair of a "neox" rotation
+                        float x[2][8];
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            const float* src = krow + (kk + u * (G::kSteps / 2)) * 32 + grp * 8;
+                            const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+                            x[u][0] = lo.x; x[u][1] = lo.y; x[u][2] = lo.z; x[u][3] = lo.w;
+                            x[u][4] = hi.x; x[u][5] = hi.y; x[u][6] = hi.z; x[u][7] = hi.w;
+                        }
+                        if constexpr (ROPE) rotate2(x[0], x[1], kk);
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            h8 h;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) h[e] = (_Float16)x[u][e];
+                            put_k(kk + u * (G::kSteps / 2), __builtin_bit_cast(u32x4, h));
+                        }
                     }
                 }
+                h8 vh;
+                vh[0] = (_Float16)v_own[0].x; vh[1] = (_Float16)v_own[0].y; vh[2] = (_Float16)v_own[0].z; vh[3] = (_Float16)v_own[0].w;
+                vh[4] = (_Float16)v_own[1].x; vh[5] = (_Float16)v_own[1].y; vh[6] = (_Float16)v_own[1].z; vh[7] = (_Float16)v_own[1].w;
+                const u32x4 v_new16 = __builtin_bit_cast(u32x4, vh);
 #pragma unroll
                 for (int i = 0; i < G::kLoads; ++i) {
                     if ((i * 64 + lane) / G::kChunksPerRow == row) {
@@ -392,8 +517,9 @@ template <int D>
 hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     const int grid = a.n_kv * a.n_hgroups * a.n_splits;
     constexpr int lds = DGeom<D>::kLdsB;
-    if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, true>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
-    else hipLaunchKernelGGL((fa_decode_split_kernel<D, false>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    if (a.k_new && a.n_rot > 0) hipLaunchKernelGGL((fa_decode_split_kernel<D, 2>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    else if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, 1>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    else hipLaunchKernelGGL((fa_decode_split_kernel<D, 0>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
@@ -410,9 +536,9 @@ hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream, hipE
 // The split kernel uses more than 64 KB of dynamic LDS; the opt-in is set once at init so
 // that no launch path touches function attributes (decode runs under stream capture).
 namespace {
-template <int D, bool STORE>
+template <int D, int MODE>
 hipError_t allow_lds() {
-    void (*const kernel)(const FaArgs) = fa_decode_split_kernel<D, STORE>;
+    void (*const kernel)(const FaArgs) = fa_decode_split_kernel<D, MODE>;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                DGeom<D>::kLdsB);
 }
@@ -420,10 +546,12 @@ hipError_t allow_lds() {
 
 hipError_t decode_allow_lds() {
     hipError_t e;
-    if ((e = allow_lds<128, false>()) != hipSuccess) return e;
-    if ((e = allow_lds<128, true>()) != hipSuccess) return e;
-    if ((e = allow_lds<64, false>()) != hipSuccess) return e;
-    return allow_lds<64, true>();
+    if ((e = allow_lds<128, 0>()) != hipSuccess) return e;
+    if ((e = allow_lds<128, 1>()) != hipSuccess) return e;
+    if ((e = allow_lds<128, 2>()) != hipSuccess) return e;
+    if ((e = allow_lds<64, 0>()) != hipSuccess) return e;
+    if ((e = allow_lds<64, 1>()) != hipSuccess) return e;
+    return allow_lds<64, 2>();
 }
 
 } // namespace orin_fa

@@ -12,12 +12,9 @@
 // thread forms its angle and one sine/cosine, then rotates its heads; all loads are issued
 // before any of that arithmetic -- where the reference spends a power, a sine and a cosine per
 // element pair of every head.
-// Arithmetic follows the CPU statement operation by operation in fp32 (no contraction of
-// the rotation into fused multiply-adds); the frequency is the double-precision power rounded
-// to fp32, which is what a correctly rounded powf returns, because at position 32768 one ulp
-// of the frequency already moves the angle by 2e-3 rad.  Sine and cosine are the accurate
-// library versions (full range reduction), not the fast hardware approximations the reference's
-// GPU path uses.
+// Arithmetic (rope_freq, rope_rotate in fa_common.hpp) follows the CPU statement operation by
+// operation in fp32.  Sine and cosine are the accurate library versions (full range
+// reduction), not the fast hardware approximations the reference's GPU path uses.
 #include "fa_common.hpp"
 
 namespace orin_fa {
@@ -55,11 +52,7 @@ __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int hea
         }
     const int pos = IND ? *d_pos : n_past + token;
     if (shared_freq && (int)threadIdx.x < half) {
-        const int fi = threadIdx.x;
-        const float expo = -2.0f * (float)fi / (float)n_rot;
-        float f = (float)pow((double)theta, (double)expo);
-        if (freq_factors) f /= freq_factors[fi];
-        sh_freq[fi] = f;
+        sh_freq[threadIdx.x] = rope_freq(threadIdx.x, n_rot, theta, freq_factors);
     }
     if (shared_freq) __syncthreads();
     if (!active) return;
@@ -67,21 +60,41 @@ __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int hea
     if (shared_freq) {
         freq = sh_freq[i];
     } else {
-        const float expo = -2.0f * (float)i / (float)n_rot;
-        freq = (float)pow((double)theta, (double)expo);
-        if (freq_factors) freq /= freq_factors[i];
+        freq = rope_freq(i, n_rot, theta, freq_factors);
     }
     const float ang = (float)pos * freq;
     const float c = cosf(ang), s = sinf(ang);
 #pragma unroll
     for (int u = 0; u < kHeadsPerThread; ++u)
         if (h0 + u < heads) {
-            row[(size_t)u * head_dim + i0] = x0[u] * c - x1[u] * s;
-            row[(size_t)u * head_dim + i1] = x0[u] * s + x1[u] * c;
+            rope_rotate(x0[u], x1[u], c, s);
+            row[(size_t)u * head_dim + i0] = x0[u];
+            row[(size_t)u * head_dim + i1] = x1[u];
         }
 }
 
+// (cos, sin) of every pair at the position *d_pos: what each thread of rope_kernel forms for
+// itself, written out once for callers that rotate several rows of one token (every layer of a
+// decode step rotates by the same angles).
+__global__ __launch_bounds__(64) void rope_angles_kernel(float* angles, int n_rot, float theta, const int* d_pos,
+                                                         const float* freq_factors) {
+#pragma clang fp contract(off)
+    const int i = blockIdx.x * 64 + threadIdx.x;
+    if (i >= n_rot / 2) return;
+    const float ang = (float)*d_pos * rope_freq(i, n_rot, theta, freq_factors);
+    angles[2 * i] = cosf(ang);
+    angles[2 * i + 1] = sinf(ang);
+}
+
 } // namespace
+
+hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
+                              hipStream_t stream) {
+    const unsigned grid = (unsigned)((n_rot / 2 + 63) / 64);
+    if (grid == 0) return hipSuccess;
+    hipLaunchKernelGGL(rope_angles_kernel, dim3(grid), dim3(64), 0, stream, angles, n_rot, theta, d_pos, freq_factors);
+    return hipGetLastError();
+}
 
 hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
                        const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream) {

@@ -45,6 +45,11 @@ def lib():
         L.orin_fa_decode_ind.restype = _int
         L.orin_fa_decode_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_store_ind.restype = _int
+        L.orin_fa_decode_rope_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
+                                                    _int, _flt, _vp, _int, _vp]
+        L.orin_fa_rope_angles_ind.argtypes = [_vp, _int, _flt, _vp, _vp]
+        L.orin_fa_rope_angles_ind.restype = _int
+        L.orin_fa_decode_rope_store_ind.restype = _int
         L.orin_fa_rope_batch.argtypes = [_vp, _int, _int, _int, _flt, _int, _int, _vp, _int]
         L.orin_fa_rope_batch.restype = _int
         L.orin_fa_rope_ind.argtypes = [_vp, _int, _int, _int, _flt, _vp, _vp, _int]
@@ -123,6 +128,25 @@ def flash_attention_decode_store_ind(q, k_new, v_new, kc, vc, out, n_head, n_kv,
                                         n_head, n_kv, head_dim, n_ctx, _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_store_ind", rc)
+
+
+def flash_attention_decode_rope_store_ind(q, k_new, v_new, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale,
+                                          n_rot, theta, freq_factors=None, neox=True, angles=None):
+    """rope_*_ind on q and on k_new, kv_store_ind and flash_attention_decode_ind in the launches of the last
+    (no counterpart in the reference; q and k_new are taken before the rotation and left as they are).
+    angles: optionally the table rope_angles_ind wrote for this token."""
+    rc = lib().orin_fa_decode_rope_store_ind(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(kc), _ptr(vc), _ptr(out),
+                                             n_head, n_kv, head_dim, n_ctx, _ptr(d_pos), scale,
+                                             n_rot, theta, _ptr(freq_factors), 1 if neox else 0, _ptr(angles))
+    if rc != 0:
+        raise OrinFaError("flash_attention_decode_rope_store_ind", rc)
+
+
+def rope_angles_ind(angles, n_rot, theta, d_pos, freq_factors=None):
+    """(cos, sin) of the n_rot/2 pairs at *d_pos into angles [n_rot/2][2] (no counterpart in the reference)."""
+    rc = lib().orin_fa_rope_angles_ind(_ptr(angles), n_rot, theta, _ptr(freq_factors), _ptr(d_pos))
+    if rc != 0:
+        raise OrinFaError("rope_angles_ind", rc)
 
 
 def rope_neox_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors=None):

@@ -214,6 +214,97 @@ def test_decode_store_equals_store_then_decode(fa, H, G, d, n_ctx):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,n_ctx,n_rot,neox,ff", [
+    (12, 2, 128, 4096, 128, True, False),     # Qwen2.5-1.5B
+    (28, 4, 128, 32768, 128, True, True),
+    (32, 8, 128, 2048, 128, False, True),     # Llama-3 ("normal" pairing, frequency factors)
+    (8, 8, 64, 600, 64, True, False),
+    (8, 8, 64, 600, 32, False, False),        # partial rotation
+    (40, 2, 128, 1024, 96, False, True),
+    (12, 2, 128, 512, 0, True, False),        # no rotation: the store + attend pair
+])
+def test_decode_rope_store_equals_the_four_calls(fa, H, G, d, n_ctx, n_rot, neox, ff):
+    """rope on q, rope on the new K row, kv_store_ind, flash_attention_decode_ind (reference
+    call sites: src/model_gpu.cu:277-282) against the one call that stands for them: same cache
+    bytes and same output bit for bit, q and k_new untouched, eager and replayed from a graph."""
+    import torch
+    scale = float(1.0 / np.sqrt(d))
+    theta = 1.0e6 if neox else 5.0e5
+    rng = np.random.default_rng(H * 7 + n_ctx + n_rot)
+    base_k = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    base_v = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    freq = torch.from_numpy(rng.uniform(0.5, 8.0, max(n_rot // 2, 1)).astype(np.float32)).cuda() if ff else None
+    q = torch.zeros((H, d), device="cuda")
+    k_new = torch.zeros((G, d), device="cuda")
+    v_new = torch.zeros((G, d), device="cuda")
+    dpos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ka, va = torch.from_numpy(base_k).cuda(), torch.from_numpy(base_v).cuda()   # four calls
+    kb, vb = ka.clone(), va.clone()                                             # one call
+    out_a = torch.empty((H, d), device="cuda")
+    out_b = torch.empty((H, d), device="cuda")
+    rope_ind = fa.rope_neox_ind if neox else fa.rope_normal_ind
+
+    angles = torch.zeros((max(n_rot // 2, 1), 2), device="cuda")
+
+    def fused(with_table=False):
+        if with_table and n_rot:   # the angles once per token, as a decode step over many layers would
+            fa.rope_angles_ind(angles, n_rot, theta, dpos, freq)
+        fa.flash_attention_decode_rope_store_ind(q, k_new, v_new, kb, vb, out_b, H, G, d, n_ctx, dpos, scale,
+                                                 n_rot, theta, freq, neox, angles if with_table and n_rot else None)
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            fa.set_stream(torch.cuda.current_stream().cuda_stream)
+            fused()
+    finally:
+        fa.set_stream(torch.cuda.current_stream().cuda_stream)
+    positions = [0, 1, 31, 32, 33, 255, 256, 257, n_ctx // 2 - 1, n_ctx // 2, n_ctx - 2, n_ctx - 1, n_ctx, -1]
+    for i, pos in enumerate(positions):
+        q.copy_(torch.from_numpy(rng.standard_normal((H, d)).astype(np.float32)))
+        k_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        v_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        dpos.fill_(pos)
+        q_rot, k_rot = q.clone(), k_new.clone()
+        q_before, k_before = q.clone(), k_new.clone()
+        if n_rot:
+            rope_ind(q_rot, H, d, n_rot, theta, dpos, freq)
+            rope_ind(k_rot, G, d, n_rot, theta, dpos, freq)
+        fa.kv_store_ind(ka, va, k_rot, v_new, G, d, n_ctx, dpos)
+        fa.flash_attention_decode_ind(q_rot, ka, va, out_a, H, G, d, n_ctx, dpos, scale)
+        if i % 2 == 0:
+            g.replay()
+        else:
+            fused(with_table=(i % 4 == 1))
+        torch.cuda.synchronize()
+        assert torch.equal(q, q_before) and torch.equal(k_new, k_before), pos
+        assert torch.equal(ka, kb) and torch.equal(va, vb), pos
+        assert torch.equal(out_a.view(torch.int32), out_b.view(torch.int32)), pos
+    if n_rot:   # the rotation did something: the rotated row differs from the raw one
+        assert not torch.equal(k_rot, k_new)
+
+
+@pytest.mark.gpu
+def test_decode_rope_store_rejects_what_it_does_not_cover(fa):
+    import torch
+    from orin_llm_amd.kernels import OrinFaError
+    H, G, d, n_ctx = 4, 2, 128, 256
+    q = torch.zeros((H, d), device="cuda")
+    kn = torch.zeros((G, d), device="cuda")
+    kc = torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda")
+    out = torch.empty((H, d), device="cuda")
+    dpos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for n_rot, neox in [(64, True), (130, False), (63, False), (-2, False)]:
+        with pytest.raises(OrinFaError):
+            fa.flash_attention_decode_rope_store_ind(q, kn, kn, kc, kc.clone(), out, H, G, d, n_ctx, dpos, 0.1,
+                                                     n_rot, 1.0e4, None, neox)
+    with pytest.raises(OrinFaError):
+        fa.rope_angles_ind(q, 63, 1.0e4, dpos)
+    with pytest.raises(OrinFaError):
+        fa.flash_attention_decode_rope_store_ind(q, None, kn, kc, kc.clone(), out, H, G, d, n_ctx, dpos, 0.1,
+                                                 128, 1.0e4, None, True)
+
+
+@pytest.mark.gpu
 def test_kv_mutators_reject_bad_arguments(fa):
     import torch
     from orin_llm_amd.kernels import OrinFaError
