@@ -216,6 +216,12 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     FA_STAMP(0);
 
+    // Every kernel argument is asked for here, in one trip to memory: left alone, the compiler
+    // fetches the pointers only where they are first used, behind a wait for the integers.
+    {
+        const void *p0 = a.q, *p1 = a.kc, *p2 = a.vc, *p3 = a.out;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(a.n_head));
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: tile indices live in scalar registers
     const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
@@ -369,13 +375,20 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     if (n_mine > 0) {
         // V buffer 0 receives the diagonal tile, whose rows at or past kv_end are not fetched:
         // clear it first, so that no stale bit pattern meets a zero weight (0 * NaN is not 0).
+        // The buffer is this wave's own: once the wave's LDS writes have completed, the copy
+        // into it may go out -- together with K(1), ahead of the wait for the queries, so that
+        // the second tile's trip to memory runs beside the queries' instead of after it.
 #pragma unroll
         for (int i = 0; i < G::kCopies; ++i)
             *reinterpret_cast<u32x4*>(ws + G::kVOff + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        copy_checked(vdesc, v_buf(0), tile_of(0));
+        copy_checked(kdesc, k_buf(1), tile_of(1));
     }
     FA_STAMP(10);
     // ---- query block -> LDS (fp16) ----
-    if (n_mine > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (G::kCopies & 15) | ((G::kCopies >> 4) << 14)); // vmcnt: the queries are in, K(0) may be in flight
+    constexpr int kInFlight = 3 * G::kCopies; // K(0), V(0), K(1)
+    if (n_mine > 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (kInFlight & 15) | ((kInFlight >> 4) << 14)); // vmcnt: the queries are in, the copies may be in flight
     else __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
     for (int j = 0; j < kQLoads; ++j) {
@@ -384,11 +397,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         for (int e = 0; e < 4; ++e) hv[e] = (_Float16)(__uint_as_float(qraw[j][e]) * qmul[j]);
         *reinterpret_cast<h4*>(smem + G::kQOff + qcol[j] * G::kQStride + (lane % (D / 4)) * 8) = hv;
     }
-    __syncthreads(); // (also orders the clearing of V buffer 0 before the copy into it)
-    if (n_mine > 0) {
-        copy_checked(vdesc, v_buf(0), tile_of(0));
-        copy_checked(kdesc, k_buf(1), tile_of(1));
-    }
+    __syncthreads();
     int limit[NCB];
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) {
