@@ -138,9 +138,25 @@ def cpu_baseline_prefill(ref, layers_qkv, H, G, d, n_ctx, P, B, scale, budget_s=
         dt += time.perf_counter() - t0
         if dt > budget_s:
             break
+    # Beside it, separately labelled: the same restatement spread over the host's cores (the
+    # reference's CPU backend has no threading), one (token, head) row per task, fp16 cache.
+    threads = ref.max_threads()
+    rows = np.array([(t, h) for t in range(B) for h in range(H)], np.int32)
+    mt_flops, mt_dt, mt_layers = 0.0, 0.0, 0
+    for q, k, v in layers_qkv:
+        t0 = time.perf_counter()
+        ref.flash_attention_rows(q, k, v, rows, H, G, d, n_ctx, P, np.float32(scale), threads=threads)
+        mt_dt += time.perf_counter() - t0
+        mt_flops += prefill_flops(H, d, P, B)
+        mt_layers += 1
+        if mt_dt > budget_s / 3:
+            break
     return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=1, kind="port",
                 sample=f"{done} query tokens x {H} heads at depth {P} from the first {used} layer(s) "
-                       f"({flops / 1e9:.2f} GFLOP in {dt:.1f} s), reference loop order, fp32 cache")
+                       f"({flops / 1e9:.2f} GFLOP in {dt:.1f} s), reference loop order, fp32 cache",
+                all_cores=dict(value=mt_flops / mt_dt / 1e12, unit="TFLOP/s", cores=threads,
+                               sample=f"every (token, head) row of {mt_layers} layer(s) at depth {P} in {mt_dt:.1f} s, "
+                                      f"rows spread over {threads} OpenMP threads, fp16 cache"))
 
 
 def cpu_baseline_decode(ref, q, k, v, H, G, d, n_ctx, L, scale):
@@ -154,8 +170,21 @@ def cpu_baseline_decode(ref, q, k, v, H, G, d, n_ctx, L, scale):
             break
     dt = time.perf_counter() - t0
     # the CPU backend keeps an fp32 cache; the bytes counted are the fp16 bytes of the same positions
+    threads = min(ref.max_threads(), H)
+    rows = np.array([(0, h) for h in range(H)], np.int32)
+    mt_reps, t0 = 0, time.perf_counter()
+    while True:
+        ref.flash_attention_rows(q[None], k, v, rows, H, G, d, n_ctx, L - 1, np.float32(scale), threads=threads)
+        mt_reps += 1
+        if time.perf_counter() - t0 > 3.0 or mt_reps >= 64:
+            break
+    mt_dt = time.perf_counter() - t0
+    # the CPU backend keeps an fp32 cache; the bytes counted are the fp16 bytes of the same positions
     return dict(value=decode_bytes(H, G, d, L) * reps / dt / 1e9, unit="GB/s", cores=1, kind="port",
-                sample=f"{reps} decode steps of layer 0 at L={L} in {dt:.1f} s, reference loop order, fp32 cache")
+                sample=f"{reps} decode steps of layer 0 at L={L} in {dt:.1f} s, reference loop order, fp32 cache",
+                all_cores=dict(value=decode_bytes(H, G, d, L) * mt_reps / mt_dt / 1e9, unit="GB/s", cores=threads,
+                               sample=f"{mt_reps} decode steps of layer 0 at L={L} in {mt_dt:.1f} s, one head per "
+                                      f"OpenMP thread, fp16 cache"))
 
 
 def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
@@ -251,8 +280,8 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
         parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="sampled, layer 0, vs CPU oracle"),
     )
     if with_cpu:
-        sample = ((ql.cpu().numpy(), kl.view(torch.uint16).cpu().numpy(), vl.view(torch.uint16).cpu().numpy())
-                  for ql, kl, vl, _ in stacks[dom][:6])
+        sample = [(ql.cpu().numpy(), kl.view(torch.uint16).cpu().numpy(), vl.view(torch.uint16).cpu().numpy())
+                  for ql, kl, vl, _ in stacks[dom][:6]]
         res["cpu_baseline"] = cpu_baseline_prefill(ref, sample, H, G, d, n_ctx, P, B, scale)
     return res
 
