@@ -43,6 +43,7 @@ WORKLOADS = {
     # name: (shape, kind, n_ctx, list of (P, B) for prefill | L for decode)
     "qwen1.5b-prefill512": ("qwen1.5b", "prefill", 4096, [(0, 512), (3584, 512)]),
     "qwen1.5b-prefill512-d3584": ("qwen1.5b", "prefill", 4096, [(3584, 512)]),  # the default workload's second chunk alone
+    "qwen1.5b-prefill512-d32256": ("qwen1.5b", "prefill", 32768, [(32256, 512)]),  # the last chunk of a full 32k context
     "llama8b-prefill512-d4096": ("llama8b", "prefill", 8192, [(4096, 512)]),
     "llama8b-prefill512-d0": ("llama8b", "prefill", 8192, [(0, 512)]),
     "llama8b-prefill512-d7680": ("llama8b", "prefill", 8192, [(7680, 512)]),
@@ -78,7 +79,7 @@ TRAFFIC = {
     "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
 }
 ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k", "qwen1.5b-decode-store-32k",
-        "qwen1.5b-decode-rope-store-32k",
+        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256",
         "llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
 
 

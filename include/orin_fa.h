@@ -52,7 +52,10 @@ void orin_fa_set_stream(void* stream);
  * (reference: src/kernels.h:11-12, src/kernels.cu:1753-1776): the bytes of device
  * scratch the decode path needs for its split-KV partial results, and the call that
  * points the library at a caller-owned block of at least that size (256-byte
- * aligned).  Optional: orin_fa_init already allocates a block of this size. */
+ * aligned).  Optional: orin_fa_init already allocates a block of this size.
+ * orin_fa_prefill uses the same block when it cuts a long context's KV rows among
+ * workgroups (few query heads, 5120 rows or more): launches that use the block must
+ * not overlap, which one stream guarantees. */
 size_t orin_fa_workspace_bytes(void);
 int orin_fa_set_workspace(void* dev_ptr, size_t bytes);
 

@@ -125,7 +125,7 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
     a.r = n_head / n_kv;
     a.n_splits = 1;
     set_scale(a, scale);
-    return hip_code(prefill_launch(a, head_dim, g_state.cu_count, g_state.stream));
+    return hip_code(prefill_launch(a, head_dim, g_state.cu_count, g_state.stream, g_state.ws, g_state.ws_bytes));
 }
 
 namespace {

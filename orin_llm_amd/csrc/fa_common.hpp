@@ -52,12 +52,16 @@ struct FaArgs {
     int tq_magic;      // prefill: 65536 / tq + 1 (division of a column index by tq as multiply and shift)
     int heads_per_group; // prefill: query heads per head group
     int n_splits;      // decode: KV splits
+    int kv_split_shift; // prefill: log2 of the number of KV splits a token tile's rows are shared among (0: none);
+                        // with splits, part_o [split][batch][n_head][D] and part_ml [split][batch][n_head] (log-sum-exp, log2
+                        // units) receive what the combine kernel turns into out
     float c;           // |scale| * log2(e), clamped away from zero
     float qsign;       // sign of scale, folded into Q
 };
 
 // Launchers (defined next to their kernels).  All return hipError_t of the launch.
-hipError_t prefill_launch(const FaArgs& args, int head_dim, int cu_count, hipStream_t stream);
+hipError_t prefill_launch(const FaArgs& args, int head_dim, int cu_count, hipStream_t stream, void* workspace,
+                          size_t workspace_bytes);
 hipError_t prefill_allow_lds();
 // mid, when not null, is recorded between the split kernel and the combine kernel (timing only).
 hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream, hipEvent_t mid = nullptr);

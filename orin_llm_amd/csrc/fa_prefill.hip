@@ -227,7 +227,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
     const int hh = lane >> 5;  // lane-half: 8-wide k slice of an operand, rows 8q + 4*hh + 0..3 of an accumulator
 
-    const int kvh = __builtin_amdgcn_readfirstlane(blockIdx.x), hg = __builtin_amdgcn_readfirstlane(blockIdx.y); // (the KV head varies fastest in dispatch order)
+    const int kvh = __builtin_amdgcn_readfirstlane(blockIdx.x); // (the KV head varies fastest in dispatch order)
+    // blockIdx.y = head group * splits + KV split (splits: a power of two, 1 unless the launcher found the grid too small)
+    const int hg = __builtin_amdgcn_readfirstlane(blockIdx.y) >> a.kv_split_shift;
+    const int split = __builtin_amdgcn_readfirstlane(blockIdx.y) & ((1 << a.kv_split_shift) - 1);
     const int n_past = a.n_past, batch = a.batch, tq = a.tq;
     const int t0 = (a.n_ttiles - 1 - __builtin_amdgcn_readfirstlane(blockIdx.z)) * tq; // longest rows first
     const int head_lo = hg * a.heads_per_group;
@@ -245,16 +248,22 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // keeps the common order: its steps are long enough to cover the trip, and it measured 2-4 %
     // slower with any stagger.  (The order of the tiles does not matter to the result.)
     // Steps past the end map to negative tiles, for which the copies fetch a tile nobody reads.
-    const int n_mine = n_tiles > wave ? (n_tiles - 1 - wave) / kWaves + 1 : 0;
+    // With KV splits, split s of S takes the tiles w + 4*(s + S*i): runs of four tiles (one per
+    // wave) go to the splits in turn, so the tiles at the diagonal, the ones that can need the
+    // mask, are still each the highest tile of the wave that owns them.
+    const int t_base = wave + kWaves * split;   // this wave's lowest tile
+    const int t_shift = 2 + a.kv_split_shift;   // log2 of the distance between its tiles
+    static_assert(kWaves == 4, "tile distance as a shift");
+    const int n_mine = n_tiles > t_base ? ((n_tiles - 1 - t_base) >> t_shift) + 1 : 0;
     const int n_rest = n_mine - 1;
     const int rot = (NCB == 1 && n_rest > 1)
                         ? (int)((((unsigned)__builtin_amdgcn_readfirstlane(blockIdx.z) * 0x9E3779B1u) >> 8) % (unsigned)n_rest) : 0;
     auto tile_of = [&](int j) {
-        if (j == 0) return wave + kWaves * n_rest;
+        if (j == 0) return t_base + (n_rest << t_shift);
         if (j > n_rest) return -1;
         int k = j - 1 + rot;
         k = k >= n_rest ? k - n_rest : k;
-        return wave + kWaves * (n_rest - 1 - k);
+        return t_base + ((n_rest - 1 - k) << t_shift);
     };
     // column c of the block -> (token, head of the group); columns past the group's heads are padding
     auto col_valid = [&](int c, int& tok, int& hl) {
@@ -780,13 +789,21 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         for (int w = 0; w < kWaves; ++w) m_all = fmaxf(m_all, mw[w]);
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            wgt[w] = fast_exp2(mw[w] - m_all); // the wave that holds the column's diagonal has a finite m
+            // (the wave that holds the column's diagonal has a finite m; with KV splits a split may
+            // hold no visible row of a column at all)
+            wgt[w] = m_all > -INFINITY ? fast_exp2(mw[w] - m_all) : 0.0f;
             l_all += lw[w] * wgt[w];
         }
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) wgt[w] *= inv;
-        float* const dst = a.out + ((size_t)tok * a.n_head + kvh * a.r + hl) * D;
+        const size_t orow = (size_t)tok * a.n_head + kvh * a.r + hl;
+        float* dst = a.out + orow * D;
+        if (a.kv_split_shift > 0) { // this split's normalised share and its log-sum-exp, for the combine kernel
+            const size_t prow = (size_t)split * batch * a.n_head + orow;
+            dst = a.part_o + prow * D;
+            if (part == 0) a.part_ml[prow] = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : -INFINITY;
+        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             f4 acc[kHalfJ];
@@ -806,6 +823,40 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     FA_STAMP(8);
 }
 
+// out = sum over the KV splits of their normalised outputs, weighted by 2^(lse_s - max lse) and
+// divided by the weights' sum.  One thread per 16 bytes of out; rows = batch * n_head.
+template <int D>
+__global__ __launch_bounds__(256) void fa_prefill_combine_kernel(const float* part_o, const float* part_lse, float* out,
+                                                                 int rows, int splits) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int row = idx / (D / 4), piece = idx % (D / 4);
+    if (row >= rows) return;
+    constexpr int kMaxS = 4;
+    float lse[kMaxS];
+    f4 x[kMaxS];
+#pragma unroll
+    for (int s = 0; s < kMaxS; ++s)
+        if (s < splits) {
+            lse[s] = part_lse[(size_t)s * rows + row];
+            x[s] = *reinterpret_cast<const f4*>(part_o + ((size_t)s * rows + row) * D + piece * 4);
+        }
+    float m = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kMaxS; ++s)
+        if (s < splits) m = fmaxf(m, lse[s]);
+    float wsum = 0.0f;
+    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < kMaxS; ++s)
+        if (s < splits) {
+            const float w = lse[s] > -INFINITY ? fast_exp2(lse[s] - m) : 0.0f; // (a split without a visible row of this column)
+            wsum += w;
+            acc += x[s] * w;
+        }
+    const float inv = wsum > 0.0f ? 1.0f / wsum : 0.0f;
+    *reinterpret_cast<f4*>(out + (size_t)row * D + piece * 4) = acc * inv;
+}
+
 template <int D, int NCB>
 hipError_t launch_kernel(const FaArgs& a, dim3 grid, hipStream_t stream) {
     constexpr int lds = PGeom<D, NCB>::kLdsB;
@@ -820,8 +871,17 @@ hipError_t allow_lds() {
                                PGeom<D, NCB>::kLdsB);
 }
 
+// Rows of context from which cutting a token tile's rows among several workgroups pays for the
+// second launch and the partial results' trip through memory (Qwen2.5-1.5B heads, 512-token
+// chunk: 35.1 -> 33.2 us at 6144 rows, 106 -> 71 us at 16896, 304 -> 121 us at 32768; slower
+// below about 4600 rows).
+#ifndef ORIN_FA_SPLIT_MIN_ROWS
+#define ORIN_FA_SPLIT_MIN_ROWS 5120
+#endif
+constexpr int kSplitMinRows = ORIN_FA_SPLIT_MIN_ROWS;
+
 template <int D>
-hipError_t launch(FaArgs a, int cu_count, hipStream_t stream) {
+hipError_t launch(FaArgs a, int cu_count, hipStream_t stream, void* workspace, size_t workspace_bytes) {
     // Column packing: a workgroup's columns are (heads of the group) x (tq tokens), 64 of them
     // (two 32-column blocks) or 32.  GQA ratios up to 8 are one group; larger ratios are cut
     // into groups of 8 heads that each re-read the KV head.
@@ -832,21 +892,45 @@ hipError_t launch(FaArgs a, int cu_count, hipStream_t stream) {
     a.tq = 64 / a.heads_per_group;
     // A workgroup occupies a whole CU and the kernel lasts as long as its longest workgroup, so
     // a grid that would leave half the CUs idle is cut finer: 32 columns per workgroup.
-    if (2 * a.n_kv * a.n_hgroups * ((a.batch + a.tq - 1) / a.tq) <= cu_count) {
-        ncb = 1;
-        a.tq = 32 / a.heads_per_group;
+    // On a long context the better cut is along the KV rows: the workgroup keeps its 64 columns
+    // (a step's K and V tiles then serve twice the columns: in the 32-column shape the step is
+    // bound by what the CU's vector memory path delivers, 64 bytes a clock, not by the matrix
+    // pipe) and 2 or 4 workgroups share a token tile's rows; a second, small kernel merges their
+    // results.  Needs room for the partial results in the workspace.
+    a.kv_split_shift = 0;
+    const int wgs64 = a.n_kv * a.n_hgroups * ((a.batch + a.tq - 1) / a.tq);
+    if (2 * wgs64 <= cu_count) {
+        const int shift = 4 * wgs64 <= cu_count ? 2 : 1;
+        const size_t rows = (size_t)a.batch * a.n_head;
+        const size_t need = (rows << shift) * (D + 1) * sizeof(float);
+        if (a.n_past + a.batch >= kSplitMinRows && workspace && need <= workspace_bytes) {
+            a.kv_split_shift = shift;
+            a.part_o = static_cast<float*>(workspace);
+            a.part_ml = a.part_o + (rows << shift) * D;
+        } else {
+            ncb = 1;
+            a.tq = 32 / a.heads_per_group;
+        }
     }
     a.n_ttiles = (a.batch + a.tq - 1) / a.tq;
     a.tq_magic = 65536 / a.tq + 1;
-    if (a.n_hgroups > 65535 || a.n_ttiles > 65535) return hipErrorInvalidValue;
-    const dim3 grid(a.n_kv, a.n_hgroups, a.n_ttiles);
-    return ncb == 2 ? launch_kernel<D, 2>(a, grid, stream) : launch_kernel<D, 1>(a, grid, stream);
+    if ((a.n_hgroups << a.kv_split_shift) > 65535 || a.n_ttiles > 65535) return hipErrorInvalidValue;
+    const dim3 grid(a.n_kv, a.n_hgroups << a.kv_split_shift, a.n_ttiles);
+    const hipError_t e = ncb == 2 ? launch_kernel<D, 2>(a, grid, stream) : launch_kernel<D, 1>(a, grid, stream);
+    if (e != hipSuccess || a.kv_split_shift == 0) return e;
+    const int rows = a.batch * a.n_head;
+    const unsigned blocks = (unsigned)(((size_t)rows * (D / 4) + 255) / 256);
+    hipLaunchKernelGGL(fa_prefill_combine_kernel<D>, dim3(blocks), dim3(256), 0, stream, a.part_o, a.part_ml, a.out, rows,
+                       1 << a.kv_split_shift);
+    return hipGetLastError();
 }
 
 } // namespace
 
-hipError_t prefill_launch(const FaArgs& a, int head_dim, int cu_count, hipStream_t stream) {
-    return head_dim == 128 ? launch<128>(a, cu_count, stream) : launch<64>(a, cu_count, stream);
+hipError_t prefill_launch(const FaArgs& a, int head_dim, int cu_count, hipStream_t stream, void* workspace,
+                          size_t workspace_bytes) {
+    return head_dim == 128 ? launch<128>(a, cu_count, stream, workspace, workspace_bytes)
+                           : launch<64>(a, cu_count, stream, workspace, workspace_bytes);
 }
 
 // The kernels use more than 64 KB of dynamic LDS; the opt-in is set once per kernel at init.

@@ -161,6 +161,29 @@ def test_prefill_wide_blocks(fa, d, r):
     check(got[rows[:, 0], rows[:, 1]], want, f"prefill wide d{d} r{r}")
 
 
+@pytest.mark.parametrize("H,G,d,n_past,batch,scale", [
+    (12, 2, 128, 4608, 512, 0.0883883),   # Qwen2.5-1.5B heads: two workgroups share a token tile's rows
+    (12, 2, 128, 7680, 512, 0.0883883),
+    (2, 1, 128, 4100, 1100, 0.0883883),   # four workgroups per token tile
+    (1, 1, 64, 0, 5200, 0.125),           # from an empty cache: early token tiles leave splits without a row
+    (8, 1, 64, 4900, 300, -0.3),          # a ragged end, negative scale (the rescaling path on most tiles)
+    (3, 1, 128, 5200, 1, 0.0883883),      # one token
+])
+def test_prefill_kv_splits(fa, H, G, d, n_past, batch, scale):
+    """Few query columns on a long context: the launcher cuts a token tile's KV rows among 2 or
+    4 workgroups and a second kernel merges their results.  Same oracle, same tolerance; every
+    element of out is written (the buffer starts as a sentinel value)."""
+    n_ctx = n_past + batch + 7
+    q, kc, vc = make_case(900 + H + n_past, H, G, d, n_ctx, n_past + batch, batch, outliers=2, poison_tail=True)
+    toks = sorted({0, 1, 4, 5, 9, 10, 31, 32, 63, 64, 127, 128, 129, 255, 256, 511, batch // 2, batch - 2, batch - 1}
+                  & set(range(batch)))
+    rows = np.array([(t, h) for t in toks for h in range(H)], np.int32)
+    want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, n_past, np.float32(scale))
+    got = gpu_prefill(fa, q, kc, vc, H, G, d, n_ctx, n_past, batch, scale)
+    assert np.isfinite(got).all() and (got != 12345.0).all()
+    check(got[rows[:, 0], rows[:, 1]], want, f"prefill kv splits H{H} G{G} d{d} P{n_past} B{batch}")
+
+
 @pytest.mark.parametrize("scale", [1.0, 0.35, -0.0883883])
 @pytest.mark.parametrize("H,G,batch", [(4, 2, 96), (32, 8, 600)])
 def test_prefill_moving_reference(fa, scale, H, G, batch):
