@@ -54,7 +54,7 @@ void orin_fa_set_stream(void* stream);
  * points the library at a caller-owned block of at least that size (256-byte
  * aligned).  Optional: orin_fa_init already allocates a block of this size.
  * orin_fa_prefill uses the same block when it cuts a long context's KV rows among
- * workgroups (few query heads, 5120 rows or more): launches that use the block must
+ * workgroups (few query columns, 3072 rows or more): launches that use the block must
  * not overlap, which one stream guarantees. */
 size_t orin_fa_workspace_bytes(void);
 int orin_fa_set_workspace(void* dev_ptr, size_t bytes);

@@ -167,11 +167,13 @@ def test_prefill_wide_blocks(fa, d, r):
     (2, 1, 128, 4100, 1100, 0.0883883),   # four workgroups per token tile
     (1, 1, 64, 0, 5200, 0.125),           # from an empty cache: early token tiles leave splits without a row
     (8, 1, 64, 4900, 300, -0.3),          # a ragged end, negative scale (the rescaling path on most tiles)
-    (3, 1, 128, 5200, 1, 0.0883883),      # one token
+    (3, 1, 128, 5200, 1, 0.0883883),      # one token: sixteen workgroups share its rows
+    (12, 2, 128, 9000, 45, 0.0883883),    # a short last chunk of a long prompt: sixteen workgroups per token tile
+    (12, 2, 128, 3100, 200, 0.0883883),   # four workgroups per token tile, from 3072 rows
 ])
 def test_prefill_kv_splits(fa, H, G, d, n_past, batch, scale):
-    """Few query columns on a long context: the launcher cuts a token tile's KV rows among 2 or
-    4 workgroups and a second kernel merges their results.  Same oracle, same tolerance; every
+    """Few query columns on a long context: the launcher cuts a token tile's KV rows among 2 to
+    16 workgroups and a second kernel merges their results.  Same oracle, same tolerance; every
     element of out is written (the buffer starts as a sentinel value)."""
     n_ctx = n_past + batch + 7
     q, kc, vc = make_case(900 + H + n_past, H, G, d, n_ctx, n_past + batch, batch, outliers=2, poison_tail=True)
