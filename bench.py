@@ -470,6 +470,38 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
     return res
 
 
+def time_eager_and_graph(torch, kernels, one_step, steps, warmup):
+    """Times `steps` passes of one_step launched eagerly and again replayed as one HIP graph
+    (small launches are otherwise priced by the host's launch rate, not by the GPU).  Returns
+    (wall seconds, device milliseconds) of the faster form and both forms' ms per step."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, e0.elapsed_time(e1)
+
+    wall_e, dev_e = timed(one_step)
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            one_step()
+    finally:
+        kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+    wall_g, dev_g = timed(g.replay)
+    forms = dict(eager=dict(ms_per_step=wall_e / steps * 1e3, device_ms_per_step=dev_e / steps),
+                 graph=dict(ms_per_step=wall_g / steps * 1e3, device_ms_per_step=dev_g / steps))
+    return min(wall_e, wall_g), min(dev_e, dev_g), forms
+
+
 def run_kv_store(torch, kernels, name, steps, warmup, with_cpu):
     """One step = kv_store_batch of a 512-token chunk into every layer's cache (fp32 in, fp16 out)."""
     from oracle import ref
@@ -487,18 +519,8 @@ def run_kv_store(torch, kernels, name, steps, warmup, with_cpu):
         for kc, vc, k, v in stack:
             kernels.kv_store_batch(kc, vc, k, v, G, d, n_ctx, P, B)
 
-    for _ in range(warmup):
-        one_step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        one_step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+    wall, dev_ms, forms = time_eager_and_graph(torch, kernels, one_step, steps, warmup)
+    us = dev_ms * 1e3 / (steps * layers)
     nbytes = 2.0 * B * G * d * (4 + 2)  # K and V: fp32 read, fp16 written
     kc, vc, k, v = stack[0]
     wk = np.zeros((G, n_ctx, d), np.uint16)
@@ -512,7 +534,7 @@ def run_kv_store(torch, kernels, name, steps, warmup, with_cpu):
                               frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None, kernel="kv_store_kernel<8, false>",
                               launch_us=us, bytes_per_launch=nbytes,
                               note="3 MB per launch: bound by the launch, not by HBM"),
-                parity=dict(bit_exact=exact, rows="layer 0, whole cache, vs CPU oracle"))
+                parity=dict(bit_exact=exact, rows="layer 0, whole cache, vs CPU oracle"), **forms)
 
 
 def run_rope(torch, kernels, name, steps, warmup, with_cpu):
@@ -540,27 +562,17 @@ def run_rope(torch, kernels, name, steps, warmup, with_cpu):
             kernels.rope_normal_batch(q, B * H, d, d, theta, P, H)
             kernels.rope_normal_batch(k, B * G, d, d, theta, P, G)
 
-    for _ in range(warmup):
-        one_step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        one_step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    us = e0.elapsed_time(e1) * 1e3 / (steps * layers)
+    wall, dev_ms, forms = time_eager_and_graph(torch, kernels, one_step, steps, warmup)
+    us = dev_ms * 1e3 / (steps * layers)
     nbytes = 2.0 * B * (H + G) * d * 4
     return dict(value=nbytes * layers * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
                 config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_past=P, batch=B, n_rot=d,
                             bytes_per_step=nbytes * layers),
                 roofline=dict(bound="hbm", achieved=nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
                               frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None,
-                              kernel="rope_kernel<false, false>, Q rows then K rows", launch_us=us,
+                              kernel="rope4_kernel<false, false>, Q rows then K rows", launch_us=us,
                               bytes_per_launch=nbytes, note="launch_us and bytes cover the two launches of a layer"),
-                parity=dict(max_rel_to_tensor_max=err, rows="layer 0, all rows, vs CPU oracle"))
+                parity=dict(max_rel_to_tensor_max=err, rows="layer 0, all rows, vs CPU oracle"), **forms)
 
 
 def run_kv_shift(torch, kernels, name, steps, warmup, with_cpu):

@@ -7,7 +7,9 @@
 // with i + n_rot/2, "normal" pairs 2i with 2i + 1; elements at or past n_rot are left alone.
 // pos = n_past + row / heads (batch form) or *d_pos (single-token form, read on the device).
 //
-// Every head of a token shares the token's angles, so one thread owns (token, pair, group of up
+// Two kernels: rope4_kernel for the shapes models have (n_rot a multiple of 8, 16-byte aligned
+// rows), all 128-bit accesses, and rope_kernel for any even n_rot.  In rope_kernel,
+// every head of a token shares the token's angles, so one thread owns (token, pair, group of up
 // to 8 heads): the block's first threads compute the frequency of each pair once into LDS, each
 // thread forms its angle and one sine/cosine, then rotates its heads; all loads are issued
 // before any of that arithmetic -- where the reference spends a power, a sine and a cosine per
@@ -73,6 +75,68 @@ __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int hea
         }
 }
 
+// The same rotation for the common shapes (n_rot a multiple of 8, rows 16-byte aligned), moved in
+// 16-byte pieces: a thread owns four adjacent pairs of (token, group of up to 4 heads) -- "neox":
+// elements 4j..4j+3 and the four n_rot/2 further on; "normal": elements 8j..8j+7 -- so every
+// load and store is a full 128-bit access that a wave makes on whole cache lines, all of a
+// thread's loads are in flight before its four sines and cosines are formed, and an angle is
+// computed once per four heads.  The frequencies come from a table the block's first n_rot/2
+// threads fill.  Arithmetic per element as in rope_kernel.
+constexpr int kHeadsPerThread4 = 4;
+
+template <bool NEOX, bool IND>
+__global__ __launch_bounds__(256) void rope4_kernel(float* x, int tokens, int heads, int head_dim, int n_rot,
+                                                    float theta, int n_past, const int* d_pos,
+                                                    const float* freq_factors) {
+#pragma clang fp contract(off)
+    __shared__ float sh_freq[256];
+    const int half = n_rot / 2, quads = half / 4;
+    const int n_hgroups = (heads + kHeadsPerThread4 - 1) / kHeadsPerThread4;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    const bool active = t < (long long)tokens * n_hgroups * quads;
+    const int qi = (int)(t % quads);
+    const long long th = t / quads;
+    const int hgroup = (int)(th % n_hgroups), token = (int)(th / n_hgroups);
+    const int h0 = hgroup * kHeadsPerThread4;
+    float* row = x + ((size_t)token * heads + h0) * head_dim;
+    const int o0 = NEOX ? 4 * qi : 8 * qi, o1 = NEOX ? 4 * qi + half : 8 * qi + 4;
+    float4 a[kHeadsPerThread4], b[kHeadsPerThread4];
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread4; ++u)
+        if (active && h0 + u < heads) {
+            a[u] = *reinterpret_cast<const float4*>(row + (size_t)u * head_dim + o0);
+            b[u] = *reinterpret_cast<const float4*>(row + (size_t)u * head_dim + o1);
+        }
+    const int pos = IND ? *d_pos : n_past + token;
+    if ((int)threadIdx.x < half) sh_freq[threadIdx.x] = rope_freq(threadIdx.x, n_rot, theta, freq_factors);
+    __syncthreads();
+    if (!active) return;
+    float c[4], sn[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float ang = (float)pos * sh_freq[4 * qi + e];
+        c[e] = cosf(ang);
+        sn[e] = sinf(ang);
+    }
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread4; ++u)
+        if (h0 + u < heads) {
+            if (NEOX) {
+                rope_rotate(a[u].x, b[u].x, c[0], sn[0]);
+                rope_rotate(a[u].y, b[u].y, c[1], sn[1]);
+                rope_rotate(a[u].z, b[u].z, c[2], sn[2]);
+                rope_rotate(a[u].w, b[u].w, c[3], sn[3]);
+            } else {
+                rope_rotate(a[u].x, a[u].y, c[0], sn[0]);
+                rope_rotate(a[u].z, a[u].w, c[1], sn[1]);
+                rope_rotate(b[u].x, b[u].y, c[2], sn[2]);
+                rope_rotate(b[u].z, b[u].w, c[3], sn[3]);
+            }
+            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o0) = a[u];
+            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o1) = b[u];
+        }
+}
+
 // (cos, sin) of every pair at the position *d_pos: what each thread of rope_kernel forms for
 // itself, written out once for callers that rotate several rows of one token (every layer of a
 // decode step rotates by the same angles).
@@ -101,6 +165,19 @@ hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta,
     // batch form: rows = tokens * heads; single-token form: every row belongs to the one token
     const int tokens = d_pos ? 1 : rows / heads;
     const int heads_per_token = d_pos ? rows : heads;
+    if (n_rot % 8 == 0 && n_rot / 2 <= 256 && head_dim % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+        const int n_hgroups4 = (heads_per_token + kHeadsPerThread4 - 1) / kHeadsPerThread4;
+        const long long threads4 = (long long)tokens * n_hgroups4 * (n_rot / 8);
+        const unsigned grid4 = (unsigned)((threads4 + 255) / 256);
+        if (grid4 == 0) return hipSuccess;
+#define ORIN_ROPE4_LAUNCH(NEOX, IND) \
+    hipLaunchKernelGGL((rope4_kernel<NEOX, IND>), dim3(grid4), dim3(256), 0, stream, x, tokens, heads_per_token, \
+                       head_dim, n_rot, theta, n_past, d_pos, freq_factors)
+        if (neox) { if (d_pos) ORIN_ROPE4_LAUNCH(true, true); else ORIN_ROPE4_LAUNCH(true, false); }
+        else      { if (d_pos) ORIN_ROPE4_LAUNCH(false, true); else ORIN_ROPE4_LAUNCH(false, false); }
+#undef ORIN_ROPE4_LAUNCH
+        return hipGetLastError();
+    }
     const int n_hgroups = (heads_per_token + kHeadsPerThread - 1) / kHeadsPerThread;
     const long long threads = (long long)tokens * n_hgroups * (n_rot / 2);
     const unsigned grid = (unsigned)((threads + 255) / 256);
