@@ -564,6 +564,26 @@ def run_rope(torch, kernels, name, steps, warmup, with_cpu):
 
     wall, dev_ms, forms = time_eager_and_graph(torch, kernels, one_step, steps, warmup)
     us = dev_ms * 1e3 / (steps * layers)
+    # beside it: the chunk's whole way into the cache -- rope on Q, rope on K, kv_store_batch -- as the three
+    # calls of the reference and as the one call that stands for them
+    vv = torch.randn((B * G, d), generator=g, device="cuda")
+    caches = [(torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda"),
+               torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda")) for _ in range(layers)]
+
+    def three_calls():
+        for (q, k), (kc, vc) in zip(stack, caches):
+            kernels.rope_normal_batch(q, B * H, d, d, theta, P, H)
+            kernels.rope_normal_batch(k, B * G, d, d, theta, P, G)
+            kernels.kv_store_batch(kc, vc, k, vv, G, d, n_ctx, P, B)
+
+    def one_call():
+        for (q, k), (kc, vc) in zip(stack, caches):
+            kernels.rope_store_batch(q, k, vv, kc, vc, B, H, G, d, n_ctx, P, d, theta, None, False)
+
+    _, dev3, _ = time_eager_and_graph(torch, kernels, three_calls, steps, warmup)
+    _, dev1, _ = time_eager_and_graph(torch, kernels, one_call, steps, warmup)
+    forms["into_the_cache"] = dict(three_calls_us=dev3 * 1e3 / (steps * layers), one_call_us=dev1 * 1e3 / (steps * layers),
+                                   note="rope on Q + rope on K + kv_store_batch per layer; one_call: orin_fa_rope_store_batch")
     nbytes = 2.0 * B * (H + G) * d * 4
     return dict(value=nbytes * layers * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
                 config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_past=P, batch=B, n_rot=d,

@@ -90,6 +90,17 @@ int orin_fa_rope_batch(float* x, int rows, int head_dim, int n_rot, float theta,
 int orin_fa_rope_ind(float* x, int rows, int head_dim, int n_rot, float theta, const int* d_pos,
                      const float* freq_factors, int neox);
 
+/* The three calls a prefill layer makes ahead of its attention -- rope_*_batch on the Q rows,
+ * rope_*_batch on the K rows, kv_store_batch (reference call sites: src/model_gpu.cu:378-382)
+ * -- as one call; no counterpart in the reference.  q [batch][n_head][head_dim] and
+ * k [batch][n_kv][head_dim] are rotated in place, k and v [batch][n_kv][head_dim] go to cache
+ * positions [n_past, n_past + batch): memory ends up exactly as after the three calls.  One
+ * launch when n_rot = head_dim (a multiple of 8) and all pointers are 16-byte aligned, else
+ * the three launches. */
+int orin_fa_rope_store_batch(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc, int batch, int n_head,
+                             int n_kv, int head_dim, int n_ctx, int n_past, int n_rot, float theta,
+                             const float* freq_factors, int neox);
+
 /* Replaces llm::cuda::kv_store_batch (reference: src/kernels.h:66-67, src/kernels.cu:1659-1678,
  * 2079-2083; CPU statement src/model_cpu.cpp:276-279): rounds the fp32 K and V rows of `batch`
  * tokens (k, v: [batch][heads][head_dim]) to binary16, nearest-even, into cache positions

@@ -270,6 +270,30 @@ int orin_fa_rope_ind(float* x, int rows, int head_dim, int n_rot, float theta, c
     return hip_code(rope_launch(x, rows, head_dim, n_rot, theta, 0, rows, d_pos, freq_factors, neox != 0, g_state.stream));
 }
 
+int orin_fa_rope_store_batch(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc, int batch, int n_head,
+                             int n_kv, int head_dim, int n_ctx, int n_past, int n_rot, float theta,
+                             const float* freq_factors, int neox) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!q || !k || !v || !kc || !vc) return ORIN_FA_E_INVALID;
+    if (batch < 0 || n_head <= 0 || n_kv <= 0 || head_dim <= 0 || n_ctx <= 0 || n_past < 0) return ORIN_FA_E_INVALID;
+    if (n_rot < 0 || n_rot > head_dim || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    if ((long long)n_past + batch > n_ctx) return ORIN_FA_E_INVALID;
+    if (batch == 0) return ORIN_FA_OK;
+    if (rope_store_fused_ok(q, k, v, kc, vc, head_dim, n_rot))
+        return hip_code(rope_store_launch(q, k, v, kc, vc, batch, n_head, n_kv, head_dim, n_ctx, n_past, theta,
+                                          freq_factors, neox != 0, g_state.stream));
+    // any other shape: the three launches this call stands for
+    if (n_rot > 0) {
+        hipError_t e = rope_launch(q, batch * n_head, head_dim, n_rot, theta, n_past, n_head, nullptr, freq_factors,
+                                   neox != 0, g_state.stream);
+        if (e != hipSuccess) return hip_code(e);
+        e = rope_launch(k, batch * n_kv, head_dim, n_rot, theta, n_past, n_kv, nullptr, freq_factors, neox != 0,
+                        g_state.stream);
+        if (e != hipSuccess) return hip_code(e);
+    }
+    return hip_code(kv_store_launch(kc, vc, k, v, n_kv, head_dim, n_ctx, n_past, batch, nullptr, g_state.stream));
+}
+
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return 0;
     if (head_dim != 64 && head_dim != 128) return 0;

@@ -77,6 +77,11 @@ hipError_t kv_shift_launch(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, in
 // Rotary embedding (rope.hip).  d_pos not null selects the single-token form.
 hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
                        const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream);
+bool rope_store_fused_ok(const float* q, const float* k, const float* v, const uint16_t* kc, const uint16_t* vc,
+                         int head_dim, int n_rot);
+hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc, int tokens, int n_head,
+                             int n_kv, int head_dim, int n_ctx, int n_past, float theta, const float* freq_factors,
+                             bool neox, hipStream_t stream);
 hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
                               hipStream_t stream);
 

@@ -137,6 +137,94 @@ __global__ __launch_bounds__(256) void rope4_kernel(float* x, int tokens, int he
         }
 }
 
+// The three launches a prefill layer makes ahead of its attention (reference call sites:
+// src/model_gpu.cu:378-382) in one: blocks [0, nbq) rotate the Q rows as rope4_kernel does,
+// blocks [nbq, nbq + nbk) rotate the K rows, write them back and store them to the cache as
+// fp16 (rounded from the rotated fp32 value, as the store kernel rounds what the rotary kernel
+// wrote), the remaining blocks store the V rows.  n_rot = head_dim, a multiple of 8.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+template <bool NEOX>
+__global__ __launch_bounds__(256) void rope_store_kernel(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc,
+                                                         int tokens, int n_head, int n_kv, int head_dim, int n_ctx,
+                                                         int n_past, float theta, const float* freq_factors,
+                                                         unsigned nbq, unsigned nbk) {
+#pragma clang fp contract(off)
+    __shared__ float sh_freq[256];
+    if (blockIdx.x >= nbq + nbk) { // ---- V rows -> cache ----
+        const int per_row = head_dim / 8;
+        const long long j = (long long)(blockIdx.x - nbq - nbk) * 256 + threadIdx.x;
+        if (j >= (long long)tokens * n_kv * per_row) return;
+        const long long row = j / per_row; // = token * n_kv + head
+        const int piece = (int)(j % per_row), head = (int)(row % n_kv), pos = n_past + (int)(row / n_kv);
+        const float* src = v + row * head_dim + piece * 8;
+        const float4 x0 = *reinterpret_cast<const float4*>(src);
+        const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
+        half8_t h;
+        h[0] = (_Float16)x0.x; h[1] = (_Float16)x0.y; h[2] = (_Float16)x0.z; h[3] = (_Float16)x0.w;
+        h[4] = (_Float16)x1.x; h[5] = (_Float16)x1.y; h[6] = (_Float16)x1.z; h[7] = (_Float16)x1.w;
+        *reinterpret_cast<half8_t*>(vc + ((size_t)head * n_ctx + pos) * head_dim + piece * 8) = h;
+        return;
+    }
+    const bool is_k = blockIdx.x >= nbq;
+    float* const x = is_k ? k : q;
+    const int heads = is_k ? n_kv : n_head;
+    const int n_rot = head_dim, half = n_rot / 2, quads = half / 4;
+    const int n_hgroups = (heads + kHeadsPerThread4 - 1) / kHeadsPerThread4;
+    const long long t = (long long)(blockIdx.x - (is_k ? nbq : 0u)) * 256 + threadIdx.x;
+    const bool active = t < (long long)tokens * n_hgroups * quads;
+    const int qi = (int)(t % quads);
+    const long long th = t / quads;
+    const int hgroup = (int)(th % n_hgroups), token = (int)(th / n_hgroups);
+    const int h0 = hgroup * kHeadsPerThread4;
+    float* row = x + ((size_t)token * heads + h0) * head_dim;
+    const int o0 = NEOX ? 4 * qi : 8 * qi, o1 = NEOX ? 4 * qi + half : 8 * qi + 4;
+    float4 a[kHeadsPerThread4], b[kHeadsPerThread4];
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread4; ++u)
+        if (active && h0 + u < heads) {
+            a[u] = *reinterpret_cast<const float4*>(row + (size_t)u * head_dim + o0);
+            b[u] = *reinterpret_cast<const float4*>(row + (size_t)u * head_dim + o1);
+        }
+    const int pos = n_past + token;
+    if ((int)threadIdx.x < half) sh_freq[threadIdx.x] = rope_freq(threadIdx.x, n_rot, theta, freq_factors);
+    __syncthreads();
+    if (!active) return;
+    float c[4], sn[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float ang = (float)pos * sh_freq[4 * qi + e];
+        c[e] = cosf(ang);
+        sn[e] = sinf(ang);
+    }
+#pragma unroll
+    for (int u = 0; u < kHeadsPerThread4; ++u)
+        if (h0 + u < heads) {
+            if (NEOX) {
+                rope_rotate(a[u].x, b[u].x, c[0], sn[0]);
+                rope_rotate(a[u].y, b[u].y, c[1], sn[1]);
+                rope_rotate(a[u].z, b[u].z, c[2], sn[2]);
+                rope_rotate(a[u].w, b[u].w, c[3], sn[3]);
+            } else {
+                rope_rotate(a[u].x, a[u].y, c[0], sn[0]);
+                rope_rotate(a[u].z, a[u].w, c[1], sn[1]);
+                rope_rotate(b[u].x, b[u].y, c[2], sn[2]);
+                rope_rotate(b[u].z, b[u].w, c[3], sn[3]);
+            }
+            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o0) = a[u];
+            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o1) = b[u];
+            if (is_k) {
+                uint16_t* dst = kc + ((size_t)(h0 + u) * n_ctx + pos) * head_dim;
+                half4_t ha, hb;
+                ha[0] = (_Float16)a[u].x; ha[1] = (_Float16)a[u].y; ha[2] = (_Float16)a[u].z; ha[3] = (_Float16)a[u].w;
+                hb[0] = (_Float16)b[u].x; hb[1] = (_Float16)b[u].y; hb[2] = (_Float16)b[u].z; hb[3] = (_Float16)b[u].w;
+                *reinterpret_cast<half4_t*>(dst + o0) = ha;
+                *reinterpret_cast<half4_t*>(dst + o1) = hb;
+            }
+        }
+}
+
 // (cos, sin) of every pair at the position *d_pos: what each thread of rope_kernel forms for
 // itself, written out once for callers that rotate several rows of one token (every layer of a
 // decode step rotates by the same angles).
@@ -157,6 +245,31 @@ hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* 
     const unsigned grid = (unsigned)((n_rot / 2 + 63) / 64);
     if (grid == 0) return hipSuccess;
     hipLaunchKernelGGL(rope_angles_kernel, dim3(grid), dim3(64), 0, stream, angles, n_rot, theta, d_pos, freq_factors);
+    return hipGetLastError();
+}
+
+bool rope_store_fused_ok(const float* q, const float* k, const float* v, const uint16_t* kc, const uint16_t* vc,
+                         int head_dim, int n_rot) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                           reinterpret_cast<uintptr_t>(kc) | reinterpret_cast<uintptr_t>(vc);
+    return n_rot == head_dim && head_dim % 8 == 0 && head_dim / 2 <= 256 && (bits & 15u) == 0;
+}
+
+hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc, int tokens, int n_head,
+                             int n_kv, int head_dim, int n_ctx, int n_past, float theta, const float* freq_factors,
+                             bool neox, hipStream_t stream) {
+    const int quads = head_dim / 8;
+    auto blocks = [](long long threads) { return (unsigned)((threads + 255) / 256); };
+    const unsigned nbq = blocks((long long)tokens * ((n_head + kHeadsPerThread4 - 1) / kHeadsPerThread4) * quads);
+    const unsigned nbk = blocks((long long)tokens * ((n_kv + kHeadsPerThread4 - 1) / kHeadsPerThread4) * quads);
+    const unsigned nbv = blocks((long long)tokens * n_kv * (head_dim / 8));
+    if (nbq + nbk + nbv == 0) return hipSuccess;
+    if (neox)
+        hipLaunchKernelGGL(rope_store_kernel<true>, dim3(nbq + nbk + nbv), dim3(256), 0, stream, q, k, v, kc, vc, tokens,
+                           n_head, n_kv, head_dim, n_ctx, n_past, theta, freq_factors, nbq, nbk);
+    else
+        hipLaunchKernelGGL(rope_store_kernel<false>, dim3(nbq + nbk + nbv), dim3(256), 0, stream, q, k, v, kc, vc, tokens,
+                           n_head, n_kv, head_dim, n_ctx, n_past, theta, freq_factors, nbq, nbk);
     return hipGetLastError();
 }
 

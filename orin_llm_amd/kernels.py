@@ -47,6 +47,8 @@ def lib():
         L.orin_fa_decode_store_ind.restype = _int
         L.orin_fa_decode_rope_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
                                                     _int, _flt, _vp, _int, _vp]
+        L.orin_fa_rope_store_batch.argtypes = [_vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _flt, _vp, _int]
+        L.orin_fa_rope_store_batch.restype = _int
         L.orin_fa_rope_angles_ind.argtypes = [_vp, _int, _flt, _vp, _vp]
         L.orin_fa_rope_angles_ind.restype = _int
         L.orin_fa_decode_rope_store_ind.restype = _int
@@ -140,6 +142,15 @@ def flash_attention_decode_rope_store_ind(q, k_new, v_new, kc, vc, out, n_head, 
                                              n_rot, theta, _ptr(freq_factors), 1 if neox else 0, _ptr(angles))
     if rc != 0:
         raise OrinFaError("flash_attention_decode_rope_store_ind", rc)
+
+
+def rope_store_batch(q, k, v, kc, vc, batch, n_head, n_kv, head_dim, n_ctx, n_past, n_rot, theta, freq_factors=None,
+                     neox=True):
+    """rope_*_batch on the Q rows and on the K rows, then kv_store_batch, as one call (no counterpart in the reference)."""
+    rc = lib().orin_fa_rope_store_batch(_ptr(q), _ptr(k), _ptr(v), _ptr(kc), _ptr(vc), batch, n_head, n_kv, head_dim,
+                                        n_ctx, n_past, n_rot, theta, _ptr(freq_factors), 1 if neox else 0)
+    if rc != 0:
+        raise OrinFaError("rope_store_batch", rc)
 
 
 def rope_angles_ind(angles, n_rot, theta, d_pos, freq_factors=None):

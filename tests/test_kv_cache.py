@@ -284,6 +284,45 @@ def test_decode_rope_store_equals_the_four_calls(fa, H, G, d, n_ctx, n_rot, neox
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,n_ctx,n_past,batch,n_rot,neox,ff", [
+    (12, 2, 128, 4096, 3584, 512, 128, True, False),   # Qwen2.5-1.5B chunk
+    (32, 8, 128, 1024, 100, 300, 128, False, True),    # Llama-3 ("normal" pairing, frequency factors)
+    (6, 3, 64, 300, 0, 37, 64, True, True),            # ragged head groups (6 and 3 heads by fours)
+    (5, 1, 128, 64, 63, 1, 128, False, False),         # one token at the last position
+    (8, 2, 128, 512, 7, 45, 64, True, False),          # partial rotation: the three launches
+    (4, 4, 96, 200, 10, 20, 32, False, True),          # head_dim 96
+    (4, 2, 128, 256, 0, 16, 0, True, False),           # no rotation
+])
+def test_rope_store_batch_equals_the_three_calls(fa, H, G, d, n_ctx, n_past, batch, n_rot, neox, ff):
+    """rope on the Q rows, rope on the K rows, kv_store_batch (reference call sites:
+    src/model_gpu.cu:378-382) against the one call that stands for them: q, k and both caches
+    bit for bit."""
+    import torch
+    theta = 1.0e6 if neox else 5.0e5
+    rng = np.random.default_rng(H + d + batch)
+    q = torch.from_numpy(rng.standard_normal((batch, H, d)).astype(np.float32) * 2.0).cuda()
+    k = torch.from_numpy(rng.standard_normal((batch, G, d)).astype(np.float32) * 2.0).cuda()
+    v = torch.from_numpy(rng.standard_normal((batch, G, d)).astype(np.float32) * 2.0).cuda()
+    freq = torch.from_numpy(rng.uniform(0.5, 8.0, max(n_rot // 2, 1)).astype(np.float32)).cuda() if ff else None
+    base = torch.from_numpy(rng.integers(0, 30000, (G, n_ctx, d)).astype(np.int16)).cuda()
+    ka, va, kb, vb = base.clone(), base.clone(), base.clone(), base.clone()
+    qa, kra, qb, krb = q.clone(), k.clone(), q.clone(), k.clone()
+    rope = fa.rope_neox_batch if neox else fa.rope_normal_batch
+    if n_rot:
+        rope(qa, batch * H, d, n_rot, theta, n_past, H, freq)
+        rope(kra, batch * G, d, n_rot, theta, n_past, G, freq)
+    fa.kv_store_batch(ka, va, kra, v, G, d, n_ctx, n_past, batch)
+    fa.rope_store_batch(qb, krb, v, kb, vb, batch, H, G, d, n_ctx, n_past, n_rot, theta, freq, neox)
+    torch.cuda.synchronize()
+    assert torch.equal(qa.view(torch.int32), qb.view(torch.int32))
+    assert torch.equal(kra.view(torch.int32), krb.view(torch.int32))
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    if n_rot and n_past + batch > 1:
+        assert not torch.equal(qb, q)
+    assert torch.equal(kb[:, :n_past], base[:, :n_past]) and torch.equal(kb[:, n_past + batch:], base[:, n_past + batch:])
+
+
+@pytest.mark.gpu
 def test_decode_rope_store_rejects_what_it_does_not_cover(fa):
     import torch
     from orin_llm_amd.kernels import OrinFaError
