@@ -704,7 +704,8 @@ def main():
             r = run(torch, kernels, name, max(3, min(args.steps, 10)), min(args.warmup, 2), False)
             also.append(dict(workload=name, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
                              roofline=r["roofline"], parity=r["parity"],
-                             **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {})))
+                             **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {}),
+                             **({"into_the_cache": r["into_the_cache"]} if "into_the_cache" in r else {})))
         line["also"] = also
     print(json.dumps(line))
 
