@@ -143,7 +143,17 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
     const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
-    if (id * kWaves >= n_tiles) return; // inactive split: the combine kernel never reads it
+    if (id * kWaves >= n_tiles) {
+        // Inactive split: it leaves "no row seen" for its heads, so that the combine kernel can tell
+        // without reading the position itself (one more trip to memory on its short critical path);
+        // the partial outputs are left as they are and get weight zero.
+        if (threadIdx.x < 16 && hg * 16 + (int)threadIdx.x < a.r) {
+            const size_t pi = (size_t)id * a.n_head + kvh * a.r + hg * 16 + threadIdx.x;
+            a.part_ml[pi * 2 + 0] = -INFINITY;
+            a.part_ml[pi * 2 + 1] = 0.0f;
+        }
+        return;
+    }
 
     // The new row, requested by the one wave whose tiles include the row's (its last one, so the
     // row has long arrived when it is wanted) in as few loads as will do.  K: elements 4*lane ..
@@ -435,10 +445,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 }
 
 // Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
-// head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the
-// position, the (m, l) pairs and this thread's share of the partial outputs -- is issued
-// before anything is waited on, so the kernel is one memory round trip deep.  Slots of
-// splits that were inactive for this position hold stale data and are masked after the load.
+// head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the (m, l)
+// pairs and this thread's share of the partial outputs -- is issued before anything is waited
+// on, and nothing else is read (not even the position: splits that were inactive for it have
+// said so in their (m, l)), so the kernel is one memory round trip deep behind its arguments.
+// Partial outputs of such splits hold stale data and are never multiplied.
 template <int D>
 __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) {
     constexpr int kSlices = D / 32;
@@ -470,18 +481,8 @@ __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) 
         const int s = sg + j * kGroups;
         x[j] = s < n_splits ? po[s * stride] : 0.0f;
     }
-    int p = *a.d_pos;
-    p = p < 0 ? 0 : p;
-    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1;
-    const int n_tiles = (npos + kTile - 1) / kTile;
-    const int by_tiles = (n_tiles + kDecodeWaves - 1) / kDecodeWaves;
-    const int n_active = by_tiles < n_splits ? by_tiles : n_splits;
-
-    // weights w_s = 2^(m_s - max m) and the total row sum
-    if (s_mine >= n_active) {
-        m_s = -INFINITY;
-        l_s = 0.0f;
-    }
+    // weights w_s = 2^(m_s - max m) and the total row sum (a split that was inactive for this
+    // position has left m = -inf, l = 0: weight 0)
     float m_all = m_s;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, off));
@@ -501,7 +502,8 @@ __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) 
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
         const int s = sg + j * kGroups;
-        if (s < n_active) acc = __builtin_fmaf(x[j], sh_w[s], acc);
+        const float ws = s < n_splits ? sh_w[s] : 0.0f;
+        if (ws > 0.0f) acc = __builtin_fmaf(x[j], ws, acc); // (what a weightless split left behind may be anything)
     }
     sh_red[sg][threadIdx.x & 31] = acc;
     __syncthreads();
