@@ -55,6 +55,8 @@ WORKLOADS = {
     "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
     # the decode layer's call pair (store the token's K/V rows, then attend; reference src/model_gpu.cu:281-282)
     # through the entry point that does both in the attention launches; the two calls are timed beside it
+    "qwen1.5b-decode-8k": ("qwen1.5b", "decode", 32768, 8192),     # earlier positions of the same 32k cache
+    "qwen1.5b-decode-1k": ("qwen1.5b", "decode", 32768, 1024),
     "qwen1.5b-decode-store-32k": ("qwen1.5b", "decode_store", 32768, 32768),
     "qwen1.5b-decode-rope-store-32k": ("qwen1.5b", "decode_rope_store", 32768, 32768),
     # the two mutators of the cache (byte movers; value = bytes read + written per second)

@@ -16,10 +16,11 @@
 //     over K and V.  The matrix pipe is idle most of the time here, so Q and P are carried as
 //     fp16 hi + lo pairs and the result is accurate to fp32 rounding.
 //   * The position is read on the device; the launch shape depends only on by-value arguments,
-//     so the launch can be captured in a graph and replayed after the position changes.  Every
-//     wave requests its first tile before the position has arrived (one memory round trip less
-//     on the critical path): the loads are bounded by n_ctx, which is always safe, and rows at
-//     or past the position are masked (K) or zeroed on their way into LDS (V) afterwards.
+//     so the launch can be captured in a graph and replayed after the position changes.  The
+//     position and the query heads are requested together, first thing; a split that the
+//     position leaves without a tile exits without having touched the cache (at a short
+//     position in a long cache that is nearly all of them).  Tiles are fetched whole: rows at
+//     or past the position are masked (K) or zeroed on their way into LDS (V).
 //   * Partials (reference maximum, row sum, O) of the 8 waves are merged through LDS and
 //     written per split; the combine kernel merges the splits that were active.
 #include "fa_common.hpp"
@@ -67,6 +68,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     FA_STAMP(0);
 
+    // Every kernel argument the first loads need is asked for here, in one trip to memory: left
+    // alone, the compiler fetches them where they are first used, one wait behind the other, and
+    // the position, whose address is one of them, a third trip later.
+    {
+        const void *p0 = a.q, *p1 = a.kc, *p2 = a.vc, *p3 = a.d_pos;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(a.n_ctx), "s"(a.n_splits), "s"(a.r), "s"(a.qsign));
+    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = lane & 15; // MFMA column (query head of the group) / row (KV row or head_dim index) of the lane
@@ -129,13 +137,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     }
     __builtin_amdgcn_sched_barrier(0); // the small loads first: they return first, and nothing that needs them waits for a tile
 
-    int tile = tile_first;
-    fetch_k(tile); // in flight while the position is loaded
-    fetch_v(tile);
-    // Every load above is used only behind the early return below, and left alone the compiler
-    // moves them all there: position, then query, then the query's conversion, and only then the
-    // first tile -- three memory latencies one after another.  A statement that may write memory
-    // keeps them on this side of the branch, where they overlap the load of the position.
+    // The query loads above are used only behind the early return below, and left alone the
+    // compiler moves them there, behind the wait for the position.  A statement that may write
+    // memory keeps them on this side of the branch, where they overlap the load of the position.
+    // The first tile is NOT requested here: a workgroup that turns out to be inactive would pull
+    // 128 KB of cache rows for nothing -- at a short position in a long cache, all of them but a
+    // few, tens of megabytes per launch that the active ones then queue behind.
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
@@ -143,6 +150,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
     const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
+    int tile = tile_first;
+    if (id * kWaves < n_tiles) {
+        fetch_k(tile);
+        fetch_v(tile);
+        asm volatile("" ::: "memory"); // (as above: ahead of the conversions that follow, not behind them)
+        __builtin_amdgcn_sched_barrier(0);
+    }
     if (id * kWaves >= n_tiles) {
         // Inactive split: it leaves "no row seen" for its heads, so that the combine kernel can tell
         // without reading the position itself (one more trip to memory on its short critical path);
