@@ -6,7 +6,8 @@
 //
 //   * The visible cache rows [0, *d_pos] of one KV head are cut into 32-row tiles.  Workgroup
 //     (KV head, split s) is 8 wave64s; wave w takes tile s*8 + w and then every
-//     (8 * n_splits)-th tile after it, so at 32k context each wave streams one or two tiles and
+//     (8 * n_splits)-th tile after it (runs shorter than 8 at a short position in a long cache,
+//     see the kernel), so at 32k context each wave streams one or two tiles and
 //     every byte of K and V is fetched exactly once, by 128-bit loads with the non-temporal hint.
 //   * K rows go straight from memory into MFMA A-operand order (lane (col, grp) takes row col,
 //     bytes (kk*4 + grp)*16): the score product needs no LDS round trip.  V rows are loaded
@@ -87,8 +88,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     const int hg = id % a.n_hgroups;
     id /= a.n_hgroups; // = split
 
-    const int tile_first = id * kWaves + wave;
-    const int tile_step = kWaves * a.n_splits;
     unsigned char* const vs = smem + wave * G::kWaveB;
     const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
     const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
@@ -150,14 +149,24 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
     const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
+    // Tiles go to the splits in runs of `wu` consecutive tiles, one per wave: eight when there are
+    // enough tiles to keep every wave of every split busy (runs of 128 KB of K and of V), fewer
+    // at a short position in a long cache, whose few tiles then spread over as many workgroups
+    // (CUs, each with its own 64 B/clk into the vector cache) as there are instead of filling a
+    // few workgroups' eight waves.  (Interleaving single tiles among the splits at every length
+    // cost 8 % at full length on Qwen2.5-7B: neighbouring 8 KB pieces then alternate between XCDs.)
+    int wu = (n_tiles + a.n_splits - 1) / a.n_splits;
+    wu = wu > kWaves ? kWaves : wu;
+    const int tile_first = wave < wu ? id * wu + wave : n_tiles; // (n_tiles: none)
+    const int tile_step = wu * a.n_splits;
     int tile = tile_first;
-    if (id * kWaves < n_tiles) {
+    if (id * wu < n_tiles) {
         fetch_k(tile);
         fetch_v(tile);
         asm volatile("" ::: "memory"); // (as above: ahead of the conversions that follow, not behind them)
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (id * kWaves >= n_tiles) {
+    if (id * wu >= n_tiles) {
         // Inactive split: it leaves "no row seen" for its heads, so that the combine kernel can tell
         // without reading the position itself (one more trip to memory on its short critical path);
         // the partial outputs are left as they are and get weight zero.
