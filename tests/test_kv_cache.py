@@ -344,6 +344,25 @@ def test_decode_rope_store_rejects_what_it_does_not_cover(fa):
 
 
 @pytest.mark.gpu
+def test_rope_store_batch_rejects_bad_arguments(fa):
+    import torch
+    from orin_llm_amd.kernels import OrinFaError
+    H, G, d, n_ctx = 4, 2, 128, 64
+    q = torch.zeros((8, H, d), device="cuda")
+    k = torch.zeros((8, G, d), device="cuda")
+    kc = torch.zeros((G, n_ctx, d), dtype=torch.int16, device="cuda")
+    vc = kc.clone()
+    for n_past, batch, n_rot in [(60, 8, 128), (-1, 8, 128), (0, 8, 130), (0, 8, 63)]:   # past n_ctx, negative, n_rot > d, odd
+        with pytest.raises(OrinFaError):
+            fa.rope_store_batch(q, k, k, kc, vc, batch, H, G, d, n_ctx, n_past, n_rot, 1.0e4, None, True)
+    with pytest.raises(OrinFaError):
+        fa.rope_store_batch(q, None, k, kc, vc, 8, H, G, d, n_ctx, 0, 128, 1.0e4, None, True)
+    fa.rope_store_batch(q, k, k, kc, vc, 0, H, G, d, n_ctx, 0, 128, 1.0e4, None, True)        # an empty chunk is a no-op
+    torch.cuda.synchronize()
+    assert not kc.any()
+
+
+@pytest.mark.gpu
 def test_kv_mutators_reject_bad_arguments(fa):
     import torch
     from orin_llm_amd.kernels import OrinFaError
