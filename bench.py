@@ -44,6 +44,7 @@ WORKLOADS = {
     "qwen1.5b-prefill512": ("qwen1.5b", "prefill", 4096, [(0, 512), (3584, 512)]),
     "qwen1.5b-prefill512-d3584": ("qwen1.5b", "prefill", 4096, [(3584, 512)]),  # the default workload's second chunk alone
     "qwen1.5b-prefill512-d32256": ("qwen1.5b", "prefill", 32768, [(32256, 512)]),  # the last chunk of a full 32k context
+    "qwen1.5b-prefill45-d32000": ("qwen1.5b", "prefill", 32768, [(32000, 45)]),    # a short last piece of a long prompt
     "llama8b-prefill512-d4096": ("llama8b", "prefill", 8192, [(4096, 512)]),
     "llama8b-prefill512-d0": ("llama8b", "prefill", 8192, [(0, 512)]),
     "llama8b-prefill512-d7680": ("llama8b", "prefill", 8192, [(7680, 512)]),
