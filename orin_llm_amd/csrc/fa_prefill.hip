@@ -34,6 +34,11 @@
 // arithmetic) in an XOR-swizzled layout that both the 1 KB copy bursts and the operand reads
 // hit conflict-free.  Each wave walks its tiles from the diagonal backwards, so the only tile
 // that can need the causal mask is handled in the prologue and the steady state is mask-free.
+//
+// Few query columns on a long context (a model with few heads, or a short chunk): the launcher
+// lets 2 to 16 workgroups share a token tile's KV rows (runs of four tiles go to the splits in
+// turn); each writes its normalised output and log-sum-exp to the workspace and
+// fa_prefill_combine_kernel merges them into `out`.
 #include "fa_common.hpp"
 
 // Cycle-counter stamps for profiling builds (defined by a prefix header there); nothing otherwise.
