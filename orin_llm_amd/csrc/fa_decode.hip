@@ -468,72 +468,73 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 }
 
 // Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
-// head_dim); 8 lane-groups of 32 take the splits round-robin.  Every global load -- the (m, l)
-// pairs and this thread's share of the partial outputs -- is issued before anything is waited
-// on, and nothing else is read (not even the position: splits that were inactive for it have
-// said so in their (m, l)), so the kernel is one memory round trip deep behind its arguments.
-// Partial outputs of such splits hold stale data and are never multiplied.
-template <int D>
+// head_dim); 8 lane-groups of 32 take the splits round-robin.  A thread loads the (m, l) pair
+// and its element of the partial output for each of its splits -- every load issued before
+// anything is waited on, and nothing else is read (not even the position: splits that were
+// inactive for it have said so in their (m, l)) -- merges them on its own, relative to the
+// largest m it has seen, and the 8 groups' results meet in LDS behind the kernel's only
+// barrier.  No cross-lane step: the (m, l) pairs are read redundantly by the 32 threads of a
+// group (one address, one broadcast), which costs less than reductions across lanes would on a
+// kernel that is little more than one trip to memory.  Partial outputs of inactive splits hold
+// stale data and are never multiplied.
+// PER: splits per thread (n_splits <= 8 * PER; the launcher picks the smallest that fits).
+template <int D, int PER>
 __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) {
     constexpr int kSlices = D / 32;
     constexpr int kGroups = 8;
-    constexpr int kPer = kMaxSplits / kGroups; // partial-output loads per thread, at most
-    __shared__ float sh_w[kMaxSplits];
-    __shared__ float sh_red[kGroups][32];
-    __shared__ float sh_wave[4][2];
+    constexpr int kPer = PER;
+    static_assert(kGroups * PER <= kMaxSplits, "more slots than splits can be");
+    __shared__ float sh_acc[kGroups][32];
+    __shared__ float sh_m[kGroups], sh_l[kGroups];
     const int head = blockIdx.x / kSlices;
-    const int d = (blockIdx.x % kSlices) * 32 + (threadIdx.x & 31);
+    const int dl = threadIdx.x & 31;
+    const int d = (blockIdx.x % kSlices) * 32 + dl;
     const int sg = threadIdx.x >> 5;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
     const int n_splits = a.n_splits;
 
-    // loads first
-    const int s_mine = threadIdx.x; // kMaxSplits == 256 == blockDim.x
-    float m_s = -INFINITY, l_s = 0.0f;
-    if (s_mine < n_splits) {
-        const float2 ml = *reinterpret_cast<const float2*>(a.part_ml + ((size_t)s_mine * a.n_head + head) * 2);
-        m_s = ml.x;
-        l_s = ml.y;
-    }
+    float2 ml[kPer];
     float x[kPer];
     const float* po = a.part_o + (size_t)head * D + d;
-    const size_t stride = (size_t)a.n_head * D;
+    const float* pm = a.part_ml + (size_t)head * 2;
+    const size_t stride = (size_t)a.n_head * D, stride_ml = (size_t)a.n_head * 2;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-        const int s = sg + j * kGroups;
-        x[j] = s < n_splits ? po[s * stride] : 0.0f;
+        // (slots past n_splits read split 0 again and are voided below: a load under a branch
+        // would make the compiler wait for the loads before it where the branch ends)
+        const int s = sg + j * kGroups, sc = s < n_splits ? s : 0;
+        ml[j] = *reinterpret_cast<const float2*>(pm + sc * stride_ml);
+        x[j] = po[sc * stride];
     }
-    // weights w_s = 2^(m_s - max m) and the total row sum (a split that was inactive for this
-    // position has left m = -inf, l = 0: weight 0)
-    float m_all = m_s;
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) m_all = fmaxf(m_all, __shfl_xor(m_all, off));
-    if (lane == 0) sh_wave[wave][0] = m_all;
-    __syncthreads();
-    m_all = fmaxf(fmaxf(sh_wave[0][0], sh_wave[1][0]), fmaxf(sh_wave[2][0], sh_wave[3][0]));
-    const float w = fast_exp2(m_s - m_all); // every active split has seen a visible row, so m_all is finite
-    sh_w[s_mine] = w;                       // 0 for inactive slots
-    float l_all = w * l_s;
+    for (int j = 0; j < kPer; ++j)
+        if (sg + j * kGroups >= n_splits) ml[j] = float2{-INFINITY, 0.0f};
+    float m_loc = -INFINITY;
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) l_all += __shfl_xor(l_all, off);
-    if (lane == 0) sh_wave[wave][1] = l_all;
-    __syncthreads();
-    l_all = (sh_wave[0][1] + sh_wave[1][1]) + (sh_wave[2][1] + sh_wave[3][1]);
-
-    float acc = 0.0f;
+    for (int j = 0; j < kPer; ++j) m_loc = fmaxf(m_loc, ml[j].x);
+    float l_loc = 0.0f, acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-        const int s = sg + j * kGroups;
-        const float ws = s < n_splits ? sh_w[s] : 0.0f;
-        if (ws > 0.0f) acc = __builtin_fmaf(x[j], ws, acc); // (what a weightless split left behind may be anything)
+        const float w = ml[j].x > -INFINITY ? fast_exp2(ml[j].x - m_loc) : 0.0f;
+        l_loc = __builtin_fmaf(ml[j].y, w, l_loc);
+        if (w > 0.0f) acc = __builtin_fmaf(x[j], w, acc); // (what a weightless split left behind may be anything)
     }
-    sh_red[sg][threadIdx.x & 31] = acc;
+    sh_acc[sg][dl] = acc;
+    if (dl == 0) {
+        sh_m[sg] = m_loc;
+        sh_l[sg] = l_loc;
+    }
     __syncthreads();
     if (sg == 0) {
-        float tot = 0.0f;
+        float m_all = -INFINITY;
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) tot += sh_red[g][threadIdx.x];
+        for (int g = 0; g < kGroups; ++g) m_all = fmaxf(m_all, sh_m[g]);
+        float tot = 0.0f, l_all = 0.0f;
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) {
+            const float w = sh_m[g] > -INFINITY ? fast_exp2(sh_m[g] - m_all) : 0.0f;
+            l_all = __builtin_fmaf(sh_l[g], w, l_all);
+            tot = __builtin_fmaf(sh_acc[g][dl], w, tot);
+        }
         a.out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
     }
 }
@@ -548,7 +549,11 @@ hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
-    hipLaunchKernelGGL(fa_decode_combine_kernel<D>, dim3(a.n_head * (D / 32)), dim3(256), 0, stream, a);
+    const dim3 cgrid(a.n_head * (D / 32));
+    if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, a);
+    else if (a.n_splits <= 64) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 8>), cgrid, dim3(256), 0, stream, a);
+    else if (a.n_splits <= 128) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 16>), cgrid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((fa_decode_combine_kernel<D, 32>), cgrid, dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
