@@ -178,21 +178,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         return;
     }
 
-    // The new row, requested by the one wave whose tiles include the row's (its last one, so the
-    // row has long arrived when it is wanted) in as few loads as will do.  K: elements 4*lane ..
-    // 4*lane+3 (the lanes hand each other the pieces they hold of a K row through LDS then); V:
-    // piece lane % (D/8), which is what the lane holds of a V row.  The other waves make the same
-    // loads from the query, which their cache holds: no branch, so no wait where one would end.
-    float4 k_raw = float4{0.f, 0.f, 0.f, 0.f}, v_raw[2] = {k_raw, k_raw};
-    if constexpr (STORE) {
-        const int pt = pos / kTile;
-        const bool owner = store && pt >= tile_first && (pt - tile_first) % tile_step == 0;
-        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : a.q) + (lane % (D / 4)) * 4;
-        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : a.q) + (lane % G::kChunksPerRow) * 8;
-        k_raw = *reinterpret_cast<const float4*>(kp4);
-        v_raw[0] = *reinterpret_cast<const float4*>(vp8);
-        v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
-    }
     FA_STAMP(1);
     float qf[G::kSteps][8]; // this lane's 8 elements of every k-step: head_dim indices kk*32 + grp*8 + 0..7
 #pragma unroll
@@ -261,6 +246,25 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         }
     }
 
+    __builtin_amdgcn_sched_barrier(0);
+    // The new row, requested by the one wave whose tiles include the row's (its last one, so the
+    // row has long arrived when it is wanted) in as few loads as will do -- and only now, behind
+    // the query's conversion: while a CU's tiles stream in, every further load a wave issues
+    // holds it up for a few hundred cycles, which the conversion can do without.  K: elements 4*lane ..
+    // 4*lane+3 (the lanes hand each other the pieces they hold of a K row through LDS then); V:
+    // piece lane % (D/8), which is what the lane holds of a V row.  The other waves make the same
+    // loads from the query, which their cache holds: no branch, so no wait where one would end.
+    float4 k_raw = float4{0.f, 0.f, 0.f, 0.f}, v_raw[2] = {k_raw, k_raw};
+    if constexpr (STORE) {
+        const int pt = pos / kTile;
+        const bool owner = store && pt >= tile_first && (pt - tile_first) % tile_step == 0;
+        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : a.q) + (lane % (D / 4)) * 4;
+        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : a.q) + (lane % G::kChunksPerRow) * 8;
+        k_raw = *reinterpret_cast<const float4*>(kp4);
+        v_raw[0] = *reinterpret_cast<const float4*>(vp8);
+        v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     FA_STAMP(2);
     // m_ref: reference maximum of the raw scores (before the scale); l_run: this lane's share of
     // the row sum; o: O^T accumulators, lane (col, grp) holds head_dim rows db*16 + grp*4 + i.
