@@ -763,10 +763,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     __syncthreads();
     FA_STAMP(7);
 
-    // Four threads per column: the weights are computed once, then each thread merges and stores
-    // a quarter of the column's head_dim in 16-byte pieces (the four pieces of a step are one
-    // contiguous 64 bytes of the output row).
-    const int cm = threadIdx.x >> 2, part = threadIdx.x & 3;
+    // Four threads per column (eight in the 32-column shape, so that no thread idles): the weights
+    // are computed once, then each thread merges and stores its share of the column's head_dim in
+    // 16-byte pieces (the pieces of a step are one contiguous 64 or 128 bytes of the output row).
+    constexpr int kParts = (kWaves * 64) / G::kCols; // threads per column: 4 with 64 columns, 8 with 32
+    const int cm = threadIdx.x / kParts, part = threadIdx.x % kParts;
     int tok, hl;
     if (cm < G::kCols && col_valid(cm, tok, hl)) {
         // every LDS read first (the partial outputs in two halves of 16 reads), so that their
@@ -777,14 +778,14 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             mw[w] = ml[(w * G::kCols + cm) * 2 + 0];
             lw[w] = ml[(w * G::kCols + cm) * 2 + 1];
         }
-        constexpr int kHalfJ = D / 32;
+        constexpr int kHalfJ = D / (8 * kParts); // 16-byte pieces per thread and half
         f4 x[kHalfJ][kWaves];
         auto load_half = [&](int j0) {
 #pragma unroll
             for (int j = 0; j < kHalfJ; ++j)
 #pragma unroll
                 for (int w = 0; w < kWaves; ++w)
-                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((j0 + j) * 4 + part) * 4) * 4);
+                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((j0 + j) * kParts + part) * 4) * 4);
         };
         load_half(0);
         __builtin_amdgcn_sched_barrier(0);
@@ -822,7 +823,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
             if (h == 0) load_half(kHalfJ);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j = 0; j < kHalfJ; ++j) *reinterpret_cast<f4*>(dst + ((h * kHalfJ + j) * 4 + part) * 4) = acc[j];
+            for (int j = 0; j < kHalfJ; ++j) *reinterpret_cast<f4*>(dst + ((h * kHalfJ + j) * kParts + part) * 4) = acc[j];
         }
     }
     FA_STAMP(8);
