@@ -13,6 +13,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-exceptions",
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the leading scalar arguments of a kernel arrive in registers when a wave starts, instead of
+    # behind a trip to memory (the attention kernels put what their first loads need there)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
 ]
 
 

@@ -62,20 +62,19 @@ struct DGeom {
 // head_dim 64) further on.  Same arithmetic as the rotary kernel, so again bit for bit what the
 // separate launches give, four launches in the place of seven.
 template <int D, int MODE>
-__global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(const FaArgs a) {
+__global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
+    // What the first loads need comes first, as scalars: the leading kernel arguments are handed
+    // to a wave in registers when it starts (kernel-argument preload), so the position and the
+    // query can be requested at once instead of behind a trip to memory for their addresses.
+    const int* __restrict__ d_pos, const float* __restrict__ q, const uint16_t* kc, const uint16_t* vc,
+    const int n_ctx, const int n_splits, const int r, const float qsign, const int n_kv, const int n_hgroups,
+    const FaArgs a) {
     using G = DGeom<D>;
     constexpr int kWaves = kDecodeWaves;
     constexpr int kThreads = kWaves * 64;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     FA_STAMP(0);
 
-    // Every kernel argument the first loads need is asked for here, in one trip to memory: left
-    // alone, the compiler fetches them where they are first used, one wait behind the other, and
-    // the position, whose address is one of them, a third trip later.
-    {
-        const void *p0 = a.q, *p1 = a.kc, *p2 = a.vc, *p3 = a.d_pos;
-        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(a.n_ctx), "s"(a.n_splits), "s"(a.r), "s"(a.qsign));
-    }
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int col = lane & 15; // MFMA column (query head of the group) / row (KV row or head_dim index) of the lane
@@ -83,14 +82,14 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 
     // Workgroup id -> (KV head, head group, split).  The KV head varies fastest.
     int id = blockIdx.x;
-    const int kvh = id % a.n_kv;
-    id /= a.n_kv;
-    const int hg = id % a.n_hgroups;
-    id /= a.n_hgroups; // = split
+    const int kvh = id % n_kv;
+    id /= n_kv;
+    const int hg = id % n_hgroups;
+    id /= n_hgroups; // = split
 
     unsigned char* const vs = smem + wave * G::kWaveB;
-    const __amdgpu_buffer_rsrc_t krs = make_rsrc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
-    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)a.n_ctx * D * 2);
+    const __amdgpu_buffer_rsrc_t krs = make_rsrc(kc + (size_t)kvh * n_ctx * D, (unsigned)n_ctx * D * 2);
+    const __amdgpu_buffer_rsrc_t vrs = make_rsrc(vc + (size_t)kvh * n_ctx * D, (unsigned)n_ctx * D * 2);
 
     u32x4 kreg[2 * G::kSteps], vreg[G::kLoads];
     auto fetch_k = [&](int tile) {
@@ -108,11 +107,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     };
     // ---- query heads: requested before the first tile, so that they arrive before it (a wave's
     // loads complete in order) and the score product can start while V is still on its way ----
-    const int pos = *a.d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
+    const int pos = *d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
     const int hl = hg * 16 + col;
-    const bool valid = hl < a.r;
-    const float* qp = a.q + (size_t)(valid ? kvh * a.r + hl : 0) * D;
-    const float qmul = valid ? a.qsign : 0.0f;
+    const bool valid = hl < r;
+    const float* qp = q + (size_t)(valid ? kvh * r + hl : 0) * D;
+    const float qmul = valid ? qsign : 0.0f;
     float4 qx[2 * G::kSteps];
 #pragma unroll
     for (int kk = 0; kk < G::kSteps; ++kk) {
@@ -129,8 +128,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     float ff_given = 1.0f;
     if constexpr (ROPE) {
         const int pi = min(lane, a.n_rot / 2 - 1);
-        const float* anp = a.rope_angles ? a.rope_angles + 2 * pi : a.q;
-        const float* ffp = a.freq_factors ? a.freq_factors + pi : a.q;
+        const float* anp = a.rope_angles ? a.rope_angles + 2 * pi : q;
+        const float* ffp = a.freq_factors ? a.freq_factors + pi : q;
         cs_given = *reinterpret_cast<const float2*>(anp);
         ff_given = *ffp;
     }
@@ -146,8 +145,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     __builtin_amdgcn_sched_barrier(0);
 
     int p = pos < 0 ? 0 : pos;
-    const int npos = (p > a.n_ctx - 1 ? a.n_ctx - 1 : p) + 1; // rows [0, npos) are visible
-    const bool store = STORE && pos >= 0 && pos < a.n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
+    const int npos = (p > n_ctx - 1 ? n_ctx - 1 : p) + 1; // rows [0, npos) are visible
+    const bool store = STORE && pos >= 0 && pos < n_ctx;   // (a position outside the cache stores nothing, as the store kernel)
     const int n_tiles = (npos + kTile - 1) / kTile;
     // Tiles go to the splits in runs of `wu` consecutive tiles, one per wave: eight when there are
     // enough tiles to keep every wave of every split busy (runs of 128 KB of K and of V), fewer
@@ -155,10 +154,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     // (CUs, each with its own 64 B/clk into the vector cache) as there are instead of filling a
     // few workgroups' eight waves.  (Interleaving single tiles among the splits at every length
     // cost 8 % at full length on Qwen2.5-7B: neighbouring 8 KB pieces then alternate between XCDs.)
-    int wu = (n_tiles + a.n_splits - 1) / a.n_splits;
+    int wu = (n_tiles + n_splits - 1) / n_splits;
     wu = wu > kWaves ? kWaves : wu;
     const int tile_first = wave < wu ? id * wu + wave : n_tiles; // (n_tiles: none)
-    const int tile_step = wu * a.n_splits;
+    const int tile_step = wu * n_splits;
     int tile = tile_first;
     if (id * wu < n_tiles) {
         fetch_k(tile);
@@ -170,8 +169,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         // Inactive split: it leaves "no row seen" for its heads, so that the combine kernel can tell
         // without reading the position itself (one more trip to memory on its short critical path);
         // the partial outputs are left as they are and get weight zero.
-        if (threadIdx.x < 16 && hg * 16 + (int)threadIdx.x < a.r) {
-            const size_t pi = (size_t)id * a.n_head + kvh * a.r + hg * 16 + threadIdx.x;
+        if (threadIdx.x < 16 && hg * 16 + (int)threadIdx.x < r) {
+            const size_t pi = (size_t)id * a.n_head + kvh * r + hg * 16 + threadIdx.x;
             a.part_ml[pi * 2 + 0] = -INFINITY;
             a.part_ml[pi * 2 + 1] = 0.0f;
         }
@@ -258,8 +257,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
     if constexpr (STORE) {
         const int pt = pos / kTile;
         const bool owner = store && pt >= tile_first && (pt - tile_first) % tile_step == 0;
-        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : a.q) + (lane % (D / 4)) * 4;
-        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : a.q) + (lane % G::kChunksPerRow) * 8;
+        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : q) + (lane % (D / 4)) * 4;
+        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : q) + (lane % G::kChunksPerRow) * 8;
         k_raw = *reinterpret_cast<const float4*>(kp4);
         v_raw[0] = *reinterpret_cast<const float4*>(vp8);
         v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
@@ -279,7 +278,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         if constexpr (STORE) {
             if (store && tile == pos / kTile) { // the tile of the new row (the last visible one)
                 const int row = pos % kTile;
-                const size_t row_off = ((size_t)kvh * a.n_ctx + pos) * D;
+                const size_t row_off = ((size_t)kvh * n_ctx + pos) * D;
                 // (Nothing below may be started ahead of this branch: the compiler would otherwise
                 // convert the new row before the loop, in every wave, and wait there for the row's
                 // loads -- the last ones issued, so for the whole first tile.)
@@ -294,7 +293,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
                 auto put_k = [&](int kk, u32x4 piece) { // into the operand registers and (one head group's wave) the cache
                     if (col == row % 16) {
                         kreg[(row / 16) * G::kSteps + kk] = piece;
-                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.kc) + row_off + (kk * 4 + grp) * 8) = piece;
+                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(kc) + row_off + (kk * 4 + grp) * 8) = piece;
                     }
                 };
                 {
@@ -334,7 +333,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
                 for (int i = 0; i < G::kLoads; ++i) {
                     if ((i * 64 + lane) / G::kChunksPerRow == row) {
                         vreg[i] = v_new16;
-                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.vc) + row_off + (lane % G::kChunksPerRow) * 8) = v_new16;
+                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(vc) + row_off + (lane % G::kChunksPerRow) * 8) = v_new16;
                     }
                 }
             }
@@ -438,7 +437,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
         const int c = idx / (D / 4);
         const int d4 = (idx % (D / 4)) * 4;
         const int h_local = hg * 16 + c;
-        if (h_local >= a.r) continue;
+        if (h_local >= r) continue;
         float mw[kWaves], lw[kWaves];
         float m_all = -INFINITY;
 #pragma unroll
@@ -455,8 +454,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
             l_all += lw[w] * wgt;
             acc += *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)c * G::kOStride + d4) * 4) * wgt;
         }
-        const int head = kvh * a.r + h_local;
-        if (a.n_splits > 1) {
+        const int head = kvh * r + h_local;
+        if (n_splits > 1) {
             const size_t pi = (size_t)id * a.n_head + head;
             *reinterpret_cast<f4*>(a.part_o + pi * D + d4) = acc;
             if (d4 == 0) {
@@ -483,7 +482,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(cons
 // stale data and are never multiplied.
 // PER: splits per thread (n_splits <= 8 * PER; the launcher picks the smallest that fits).
 template <int D, int PER>
-__global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) {
+__global__ __launch_bounds__(256) void fa_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                                 float* __restrict__ out, const int n_splits, const int n_head) {
     constexpr int kSlices = D / 32;
     constexpr int kGroups = 8;
     constexpr int kPer = PER;
@@ -494,13 +494,12 @@ __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) 
     const int dl = threadIdx.x & 31;
     const int d = (blockIdx.x % kSlices) * 32 + dl;
     const int sg = threadIdx.x >> 5;
-    const int n_splits = a.n_splits;
 
     float2 ml[kPer];
     float x[kPer];
-    const float* po = a.part_o + (size_t)head * D + d;
-    const float* pm = a.part_ml + (size_t)head * 2;
-    const size_t stride = (size_t)a.n_head * D, stride_ml = (size_t)a.n_head * 2;
+    const float* po = part_o + (size_t)head * D + d;
+    const float* pm = part_ml + (size_t)head * 2;
+    const size_t stride = (size_t)n_head * D, stride_ml = (size_t)n_head * 2;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
         // (slots past n_splits read split 0 again and are voided below: a load under a branch
@@ -539,7 +538,7 @@ __global__ __launch_bounds__(256) void fa_decode_combine_kernel(const FaArgs a) 
             l_all = __builtin_fmaf(sh_l[g], w, l_all);
             tot = __builtin_fmaf(sh_acc[g][dl], w, tot);
         }
-        a.out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
+        out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
     }
 }
 
@@ -547,17 +546,22 @@ template <int D>
 hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     const int grid = a.n_kv * a.n_hgroups * a.n_splits;
     constexpr int lds = DGeom<D>::kLdsB;
-    if (a.k_new && a.n_rot > 0) hipLaunchKernelGGL((fa_decode_split_kernel<D, 2>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
-    else if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, 1>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
-    else hipLaunchKernelGGL((fa_decode_split_kernel<D, 0>), dim3(grid), dim3(kDecodeWaves * 64), lds, stream, a);
+    const dim3 g(grid), b(kDecodeWaves * 64);
+#define ORIN_FA_SPLIT_ARGS a.d_pos, a.q, a.kc, a.vc, a.n_ctx, a.n_splits, a.r, a.qsign, a.n_kv, a.n_hgroups, a
+    if (a.k_new && a.n_rot > 0) hipLaunchKernelGGL((fa_decode_split_kernel<D, 2>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
+    else if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, 1>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
+    else hipLaunchKernelGGL((fa_decode_split_kernel<D, 0>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
+#undef ORIN_FA_SPLIT_ARGS
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
     const dim3 cgrid(a.n_head * (D / 32));
-    if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, a);
-    else if (a.n_splits <= 64) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 8>), cgrid, dim3(256), 0, stream, a);
-    else if (a.n_splits <= 128) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 16>), cgrid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL((fa_decode_combine_kernel<D, 32>), cgrid, dim3(256), 0, stream, a);
+#define ORIN_FA_COMBINE_ARGS a.part_o, a.part_ml, a.out, a.n_splits, a.n_head
+    if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else if (a.n_splits <= 64) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 8>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else if (a.n_splits <= 128) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 16>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else hipLaunchKernelGGL((fa_decode_combine_kernel<D, 32>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
+#undef ORIN_FA_COMBINE_ARGS
     return hipGetLastError();
 }
 
@@ -572,7 +576,7 @@ hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream, hipE
 namespace {
 template <int D, int MODE>
 hipError_t allow_lds() {
-    void (*const kernel)(const FaArgs) = fa_decode_split_kernel<D, MODE>;
+    const auto kernel = fa_decode_split_kernel<D, MODE>;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                DGeom<D>::kLdsB);
 }

@@ -215,18 +215,20 @@ constexpr ItemTable kItemsOfBlock = make_items();
 constexpr int kItemsPerBlock = 48;
 
 template <int D, int NCB>
-__global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const FaArgs a) {
+__global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
+    // What the prologue's loads need comes first, as scalars: the leading kernel arguments are
+    // handed to a wave in registers when it starts (kernel-argument preload), so the query block
+    // and the first tiles are requested at once, not behind a trip to memory for their addresses.
+    // packed: heads_per_group | kv_split_shift << 4 | tq << 8 | tq_magic << 16.
+    const float* __restrict__ q_in, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, const int n_ctx,
+    const int n_past, const int batch, const int n_head, const int r_heads, const int n_ttiles, const unsigned packed,
+    const float qsign, const FaArgs a) {
     using G = PGeom<D, NCB>;
     constexpr int kWaves = kPrefillWaves;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     FA_STAMP(0);
-
-    // Every kernel argument is asked for here, in one trip to memory: left alone, the compiler
-    // fetches the pointers only where they are first used, behind a wait for the integers.
-    {
-        const void *p0 = a.q, *p1 = a.kc, *p2 = a.vc, *p3 = a.out;
-        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(a.n_head));
-    }
+    const int heads_per_group = packed & 15, kv_split_shift = (packed >> 4) & 15, tq = (packed >> 8) & 255;
+    const int tq_magic = packed >> 16;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // uniform: tile indices live in scalar registers
     const int c32 = lane & 31; // MFMA column (query column of a block) / row (KV row or head_dim index) of the lane
@@ -234,11 +236,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
 
     const int kvh = __builtin_amdgcn_readfirstlane(blockIdx.x); // (the KV head varies fastest in dispatch order)
     // blockIdx.y = head group * splits + KV split (splits: a power of two, 1 unless the launcher found the grid too small)
-    const int hg = __builtin_amdgcn_readfirstlane(blockIdx.y) >> a.kv_split_shift;
-    const int split = __builtin_amdgcn_readfirstlane(blockIdx.y) & ((1 << a.kv_split_shift) - 1);
-    const int n_past = a.n_past, batch = a.batch, tq = a.tq;
-    const int t0 = (a.n_ttiles - 1 - __builtin_amdgcn_readfirstlane(blockIdx.z)) * tq; // longest rows first
-    const int head_lo = hg * a.heads_per_group;
+    const int hg = __builtin_amdgcn_readfirstlane(blockIdx.y) >> kv_split_shift;
+    const int split = __builtin_amdgcn_readfirstlane(blockIdx.y) & ((1 << kv_split_shift) - 1);
+    const int t0 = (n_ttiles - 1 - __builtin_amdgcn_readfirstlane(blockIdx.z)) * tq; // longest rows first
+    const int head_lo = hg * heads_per_group;
     const int tok_hi = (t0 + tq < batch) ? t0 + tq : batch;
     const int kv_end = n_past + tok_hi;   // the workgroup's columns see rows [0, kv_end) at most
     const int full_end = n_past + t0 + 1; // rows below this are visible to every column
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     // wave) go to the splits in turn, so the tiles at the diagonal, the ones that can need the
     // mask, are still each the highest tile of the wave that owns them.
     const int t_base = wave + kWaves * split;   // this wave's lowest tile
-    const int t_shift = 2 + a.kv_split_shift;   // log2 of the distance between its tiles
+    const int t_shift = 2 + kv_split_shift;   // log2 of the distance between its tiles
     static_assert(kWaves == 4, "tile distance as a shift");
     const int n_mine = n_tiles > t_base ? ((n_tiles - 1 - t_base) >> t_shift) + 1 : 0;
     const int n_rest = n_mine - 1;
@@ -272,17 +273,17 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     };
     // column c of the block -> (token, head of the group); columns past the group's heads are padding
     auto col_valid = [&](int c, int& tok, int& hl) {
-        const int hq = (c * a.tq_magic) >> 16; // = c / tq for the c < 64 that occur (tq_magic = 65536 / tq + 1)
+        const int hq = (c * tq_magic) >> 16; // = c / tq for the c < 64 that occur (tq_magic = 65536 / tq + 1)
         tok = t0 + c - hq * tq;
         hl = head_lo + hq;
-        return hq < a.heads_per_group && hl < a.r && tok < batch;
+        return hq < heads_per_group && hl < r_heads && tok < batch;
     };
 
     unsigned char* const ws = smem + wave * G::kWaveB; // this wave's LDS slice
     const unsigned ws_addr = __builtin_amdgcn_readfirstlane(
         (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)ws);
-    const i32x4 kdesc = make_desc(a.kc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
-    const i32x4 vdesc = make_desc(a.vc + (size_t)kvh * a.n_ctx * D, (unsigned)kv_end * D * 2);
+    const i32x4 kdesc = make_desc(kc + (size_t)kvh * n_ctx * D, (unsigned)kv_end * D * 2);
+    const i32x4 vdesc = make_desc(vc + (size_t)kvh * n_ctx * D, (unsigned)kv_end * D * 2);
 
     // ---- per-lane offsets ----
     // Copy: lane l of copy i lands at LDS byte i*1024 + l*16 = row i*R + l/C, physical chunk l%C,
@@ -357,15 +358,15 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
     float qmul[kQLoads];
     int qcol[kQLoads];
     {
-        const i32x4 qdesc = make_desc(a.q, (unsigned)batch * a.n_head * D * 4);
+        const i32x4 qdesc = make_desc(q_in, (unsigned)batch * n_head * D * 4);
         static_for<0, kQLoads>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int c = wave * (G::kCols / 4) + j * kColsPerLoad + lane / (D / 4);
             int tok, hl;
             const bool valid = col_valid(c, tok, hl);
             qcol[j] = c;
-            qmul[j] = valid ? a.qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
-            const int q_off = valid ? ((tok * a.n_head + kvh * a.r + hl) * D + (lane % (D / 4)) * 4) * 4 : 0;
+            qmul[j] = valid ? qsign : 0.0f; // c > 0 multiplies the scores; the sign of the scale goes here
+            const int q_off = valid ? ((tok * n_head + kvh * r_heads + hl) * D + (lane % (D / 4)) * 4) * 4 : 0;
             reg_load16<0>(qraw[j], qdesc, q_off, 0);
         });
     }
@@ -803,10 +804,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(const Fa
         const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) wgt[w] *= inv;
-        const size_t orow = (size_t)tok * a.n_head + kvh * a.r + hl;
+        const size_t orow = (size_t)tok * n_head + kvh * r_heads + hl;
         float* dst = a.out + orow * D;
-        if (a.kv_split_shift > 0) { // this split's normalised share and its log-sum-exp, for the combine kernel
-            const size_t prow = (size_t)split * batch * a.n_head + orow;
+        if (kv_split_shift > 0) { // this split's normalised share and its log-sum-exp, for the combine kernel
+            const size_t prow = (size_t)split * batch * n_head + orow;
             dst = a.part_o + prow * D;
             if (part == 0) a.part_ml[prow] = l_all > 0.0f ? m_all + __builtin_amdgcn_logf(l_all) : -INFINITY;
         }
@@ -874,13 +875,15 @@ __global__ __launch_bounds__(256) void fa_prefill_combine_kernel(const float* pa
 template <int D, int NCB>
 hipError_t launch_kernel(const FaArgs& a, dim3 grid, hipStream_t stream) {
     constexpr int lds = PGeom<D, NCB>::kLdsB;
-    hipLaunchKernelGGL((fa_prefill_kernel<D, NCB>), grid, dim3(kPrefillWaves * 64), lds, stream, a);
+    const unsigned packed = (unsigned)a.heads_per_group | (unsigned)a.kv_split_shift << 4 | (unsigned)a.tq << 8 | (unsigned)a.tq_magic << 16;
+    hipLaunchKernelGGL((fa_prefill_kernel<D, NCB>), grid, dim3(kPrefillWaves * 64), lds, stream, a.q, a.kc, a.vc, a.n_ctx, a.n_past,
+                       a.batch, a.n_head, a.r, a.n_ttiles, packed, a.qsign, a);
     return hipGetLastError();
 }
 
 template <int D, int NCB>
 hipError_t allow_lds() {
-    void (*const kernel)(const FaArgs) = fa_prefill_kernel<D, NCB>;
+    const auto kernel = fa_prefill_kernel<D, NCB>;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                PGeom<D, NCB>::kLdsB);
 }
