@@ -14,14 +14,18 @@
 namespace orin_fa {
 namespace {
 
+constexpr int kMaxDevices = 16;
+
 struct State {
     bool ready = false;
     int device = 0;
     int cu_count = 0;
     hipStream_t stream = nullptr;
-    void* own_ws = nullptr; // allocated by init
+    void* own_ws = nullptr; // allocated by init, on device own_ws_device
+    int own_ws_device = -1;
     void* ws = nullptr;     // active workspace
     size_t ws_bytes = 0;
+    bool ws_is_own = false;
 };
 State g_state;
 
@@ -36,6 +40,8 @@ inline void set_scale(FaArgs& a, float scale) {
     if (!(a.c >= 1e-30f)) a.c = 1e-30f;
 }
 
+size_t decode_bytes_per_split(int n_head, int head_dim) { return (size_t)n_head * (head_dim + 2) * sizeof(float); }
+
 int decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     const int r = n_head / n_kv;
     const int n_hgroups = (r + 15) / 16;
@@ -44,7 +50,7 @@ int decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     const int by_ctx = (n_ctx + kDecodeWaves * kTile - 1) / (kDecodeWaves * kTile);
     if (s > by_ctx) s = by_ctx;
     if (s > kMaxSplits) s = kMaxSplits;
-    const size_t per_split = (size_t)n_head * (head_dim + 2) * sizeof(float);
+    const size_t per_split = decode_bytes_per_split(n_head, head_dim);
     const size_t ws = g_state.ws ? g_state.ws_bytes : kWorkspaceBytes;
     if ((size_t)s * per_split > ws) s = (int)(ws / per_split);
     return s < 1 ? 1 : s;
@@ -79,17 +85,34 @@ int orin_fa_init(int device) {
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, device);
     if (e != hipSuccess) return hip_code(e);
+    if (device < 0 || device >= kMaxDevices) return ORIN_FA_E_INVALID;
+    g_state.ready = false;
     g_state.device = device;
     g_state.cu_count = prop.multiProcessorCount;
     if ((e = prefill_allow_lds()) != hipSuccess) return hip_code(e);
     if ((e = decode_allow_lds()) != hipSuccess) return hip_code(e);
+    // The library's own workspace lives on the device it was last initialised for: a second init
+    // on another device moves it there (the old block is released; graphs captured with it must
+    // not be replayed any more, as after any change of workspace).
+    if (g_state.own_ws && g_state.own_ws_device != device) {
+        const bool active = g_state.ws_is_own;
+        if (hipSetDevice(g_state.own_ws_device) == hipSuccess) (void)hipFree(g_state.own_ws);
+        if ((e = hipSetDevice(device)) != hipSuccess) return hip_code(e);
+        g_state.own_ws = nullptr;
+        if (active) {
+            g_state.ws = nullptr;
+            g_state.ws_bytes = 0;
+        }
+    }
     if (!g_state.own_ws) {
         e = hipMalloc(&g_state.own_ws, kWorkspaceBytes);
         if (e != hipSuccess) return hip_code(e);
+        g_state.own_ws_device = device;
     }
     if (!g_state.ws) {
         g_state.ws = g_state.own_ws;
         g_state.ws_bytes = kWorkspaceBytes;
+        g_state.ws_is_own = true;
     }
     g_state.ready = true;
     return ORIN_FA_OK;
@@ -103,12 +126,14 @@ int orin_fa_set_workspace(void* dev_ptr, size_t bytes) {
     if (!dev_ptr) { // back to the library's own block
         g_state.ws = g_state.own_ws;
         g_state.ws_bytes = g_state.own_ws ? kWorkspaceBytes : 0;
+        g_state.ws_is_own = true;
         return ORIN_FA_OK;
     }
     if ((reinterpret_cast<uintptr_t>(dev_ptr) & 255u) != 0) return ORIN_FA_E_INVALID;
     if (bytes < kWorkspaceBytes) return ORIN_FA_E_WORKSPACE;
     g_state.ws = dev_ptr;
     g_state.ws_bytes = bytes;
+    g_state.ws_is_own = false;
     return ORIN_FA_OK;
 }
 
@@ -154,7 +179,8 @@ int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_
 }
 
 int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* freq_factors, const int* d_pos) {
-    if (!angles || !d_pos || n_rot <= 0 || (n_rot & 1)) return ORIN_FA_E_INVALID;
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!angles || !d_pos || n_rot <= 0 || (n_rot & 1) || n_rot > 128) return ORIN_FA_E_INVALID; // (head_dim <= 128)
     if (reinterpret_cast<uintptr_t>(angles) & 7u) return ORIN_FA_E_INVALID;
     return hip_code(rope_angles_launch(angles, n_rot, theta, d_pos, freq_factors, g_state.stream));
 }

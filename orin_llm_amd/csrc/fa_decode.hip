@@ -66,7 +66,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // What the first loads need comes first, as scalars: the leading kernel arguments are handed
     // to a wave in registers when it starts (kernel-argument preload), so the position and the
     // query can be requested at once instead of behind a trip to memory for their addresses.
-    const int* __restrict__ d_pos, const float* __restrict__ q, const uint16_t* kc, const uint16_t* vc,
+    // (no __restrict__ on these: loads the compiler knows to be invariant are free to sink past
+    // the statements below that hold them in place)
+    const int* d_pos, const float* q, const uint16_t* kc, const uint16_t* vc,
     const int n_ctx, const int n_splits, const int r, const float qsign, const int n_kv, const int n_hgroups,
     const FaArgs a) {
     using G = DGeom<D>;
@@ -142,6 +144,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // 128 KB of cache rows for nothing -- at a short position in a long cache, all of them but a
     // few, tens of megabytes per launch that the active ones then queue behind.
     asm volatile("" ::: "memory");
+    // The arguments that did not arrive in registers are fetched here, in the trip to memory that
+    // brings the position: left alone, the compiler fetches each where it is first used -- the
+    // scale behind the first tile's arrival, the partials' addresses behind the last product.
+    {
+        const void *p0 = a.part_o, *p1 = a.part_ml, *p2 = a.out;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(a.c), "s"(a.n_head), "s"(pos));
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     int p = pos < 0 ? 0 : pos;

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
     // handed to a wave in registers when it starts (kernel-argument preload), so the query block
     // and the first tiles are requested at once, not behind a trip to memory for their addresses.
     // packed: heads_per_group | kv_split_shift << 4 | tq << 8 | tq_magic << 16.
-    const float* __restrict__ q_in, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, const int n_ctx,
+    const float* q_in, const uint16_t* kc, const uint16_t* vc, const int n_ctx,
     const int n_past, const int batch, const int n_head, const int r_heads, const int n_ttiles, const unsigned packed,
     const float qsign, const FaArgs a) {
     using G = PGeom<D, NCB>;
@@ -371,6 +371,12 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         });
     }
     if (n_mine > 0) copy_checked(kdesc, k_buf(0), tile_of(0));
+    // The arguments that did not arrive in registers are fetched now, beside the first loads: left
+    // alone, the compiler fetches each where it is first used, behind the first products.
+    {
+        const void *p0 = a.out, *p1 = a.part_o, *p2 = a.part_ml;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(a.c));
+    }
     FA_STAMP(9);
     // O = 0: a matrix instruction with a zero addend writes the accumulation registers without
     // touching memory.
