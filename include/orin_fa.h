@@ -77,6 +77,20 @@ int orin_fa_prefill(const float* q, const uint16_t* kc, const uint16_t* vc, floa
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
 
+/* orin_fa_decode_ind for callers that cannot allocate and cannot hand over a workspace (code
+ * under HIP graph capture that never saw orin_fa_set_workspace, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical output, but the split-KV partial results live in a fixed block inside the
+ * library's own device data (orin_fa_static_scratch_bytes() = 2 MiB per GPU, held until the
+ * process ends) instead of the workspace.  The call allocates and frees nothing.  A shape whose
+ * partial results (splits x n_head x (head_dim + 2) x 4 bytes, splits = orin_fa_decode_splits)
+ * exceed the block returns ORIN_FA_E_WORKSPACE with a message on stderr and launches nothing.
+ * Every call on a GPU shares that GPU's block: calls that overlap on one GPU (two streams) race;
+ * calls on one stream do not.  Nothing in the block has to start at zero. */
+int orin_fa_decode_ind_static(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                              int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale);
+size_t orin_fa_static_scratch_bytes(void);
+
 /* Replace llm::cuda::rope_neox_batch / rope_normal_batch (neox != 0 / == 0) and rope_neox_ind /
  * rope_normal_ind (reference: src/kernels.h:55-62, src/kernels.cu:1619-1657, 2059-2075; CPU statement
  * src/model_cpu.cpp:179-203): rotary position embedding in place on fp32 rows x[rows][head_dim].

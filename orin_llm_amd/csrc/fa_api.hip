@@ -14,7 +14,13 @@
 namespace orin_fa {
 namespace {
 
+// Split-KV partial results for orin_fa_decode_ind_static, the entry point that allocates nothing:
+// a fixed block in the library's own device data.  Every GPU the library runs on holds its own
+// copy at its own address until the process ends; that address is looked up once per device in
+// orin_fa_init (the array's name is only a host-side handle: it is never passed to a kernel).
+constexpr size_t kStaticScratchBytes = 2u << 20;
 constexpr int kMaxDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 struct State {
     bool ready = false;
@@ -26,6 +32,7 @@ struct State {
     void* ws = nullptr;     // active workspace
     size_t ws_bytes = 0;
     bool ws_is_own = false;
+    void* static_ws[kMaxDevices] = {}; // device address of `scratch`, per device
 };
 State g_state;
 
@@ -114,6 +121,17 @@ int orin_fa_init(int device) {
         g_state.ws_bytes = kWorkspaceBytes;
         g_state.ws_is_own = true;
     }
+    // This device's copy of the static scratch block: its address, once per device, with the
+    // device current (each GPU holds the array at an address of its own).
+    if (!g_state.static_ws[device]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            fprintf(stderr, "[orin_fa] hipGetSymbolAddress(scratch) failed on device %d: %s\n", device, hipGetErrorString(e));
+            return hip_code(e);
+        }
+        g_state.static_ws[device] = ptr;
+    }
     g_state.ready = true;
     return ORIN_FA_OK;
 }
@@ -161,15 +179,26 @@ struct RopeArgs {
     int neox;
     const float* angles;
 };
+// partials: null = the active workspace; else a block of kStaticScratchBytes (the static scratch)
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
                 int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
-                const float* k_new, const float* v_new, const RopeArgs* rope = nullptr);
+                const float* k_new, const float* v_new, const RopeArgs* rope = nullptr, void* partials = nullptr);
 }
 
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
     return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr);
 }
+
+int orin_fa_decode_ind_static(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                              int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    void* const block = g_state.static_ws[g_state.device]; // looked up in orin_fa_init; never the array's name
+    if (!block) return ORIN_FA_E_NOT_INIT;
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr, nullptr, block);
+}
+
+size_t orin_fa_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_new, uint16_t* kc, uint16_t* vc,
                              float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
@@ -224,7 +253,7 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
 namespace {
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
                 int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
-                const float* k_new, const float* v_new, const RopeArgs* rope) {
+                const float* k_new, const float* v_new, const RopeArgs* rope, void* partials) {
     int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
     if (rc != ORIN_FA_OK) return rc;
     if (!d_pos) return ORIN_FA_E_INVALID;
@@ -240,8 +269,18 @@ int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* o
     a.n_hgroups = (a.r + 15) / 16;
     a.n_splits = decode_splits(n_head, n_kv, head_dim, n_ctx);
     if (a.n_splits > 1) {
-        if (!g_state.ws) return ORIN_FA_E_WORKSPACE;
-        a.part_o = static_cast<float*>(g_state.ws);
+        if (partials) {
+            // the fixed block takes the shape's usual number of splits or nothing: no quiet change of the launch
+            if ((size_t)a.n_splits * decode_bytes_per_split(n_head, head_dim) > kStaticScratchBytes) {
+                fprintf(stderr, "[orin_fa] orin_fa_decode_ind_static: %d splits x %d heads x head_dim %d need %zu bytes of "
+                                "partial results, the static block holds %zu\n", a.n_splits, n_head, head_dim,
+                        (size_t)a.n_splits * decode_bytes_per_split(n_head, head_dim), kStaticScratchBytes);
+                return ORIN_FA_E_WORKSPACE;
+            }
+        } else if (!g_state.ws) {
+            return ORIN_FA_E_WORKSPACE;
+        }
+        a.part_o = static_cast<float*>(partials ? partials : g_state.ws);
         a.part_ml = a.part_o + (size_t)a.n_splits * n_head * head_dim;
     }
     set_scale(a, scale);

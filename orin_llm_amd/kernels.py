@@ -43,6 +43,10 @@ def lib():
         L.orin_fa_prefill.restype = _int
         L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_decode_ind_static.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
+        L.orin_fa_decode_ind_static.restype = _int
+        L.orin_fa_static_scratch_bytes.argtypes = []
+        L.orin_fa_static_scratch_bytes.restype = ctypes.c_size_t
         L.orin_fa_decode_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
         L.orin_fa_decode_store_ind.restype = _int
         L.orin_fa_decode_rope_store_ind.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
@@ -121,6 +125,19 @@ def flash_attention_decode_ind(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_
                                   _ptr(d_pos), scale)
     if rc != 0:
         raise OrinFaError("flash_attention_decode_ind", rc)
+
+
+def flash_attention_decode_ind_static(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):
+    """flash_attention_decode_ind with its partial results in the library's fixed device block: allocates
+    nothing and needs no workspace (no counterpart in the reference)."""
+    rc = lib().orin_fa_decode_ind_static(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), n_head, n_kv, head_dim, n_ctx,
+                                         _ptr(d_pos), scale)
+    if rc != 0:
+        raise OrinFaError("flash_attention_decode_ind_static", rc)
+
+
+def static_scratch_bytes():
+    return int(lib().orin_fa_static_scratch_bytes())
 
 
 def flash_attention_decode_store_ind(q, k_new, v_new, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):

@@ -33,7 +33,7 @@ def lib():
 def test_header_declares_the_expected_entry_points():
     assert _declared_c_functions() == sorted([
         "orin_fa_init", "orin_fa_set_stream", "orin_fa_workspace_bytes", "orin_fa_set_workspace",
-        "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_store_ind", "orin_fa_decode_rope_store_ind", "orin_fa_rope_angles_ind", "orin_fa_rope_store_batch", "orin_fa_decode_ind_timed", "orin_fa_decode_splits",
+        "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_ind_static", "orin_fa_static_scratch_bytes", "orin_fa_decode_store_ind", "orin_fa_decode_rope_store_ind", "orin_fa_rope_angles_ind", "orin_fa_rope_store_batch", "orin_fa_decode_ind_timed", "orin_fa_decode_splits",
         "orin_fa_kv_store_batch", "orin_fa_kv_store_ind", "orin_fa_kv_shift", "orin_fa_rope_batch", "orin_fa_rope_ind", "orin_fa_cu_count",
         "orin_fa_error_string"])
 
