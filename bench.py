@@ -49,15 +49,13 @@ WORKLOADS = {
     "llama8b-prefill512-d0": ("llama8b", "prefill", 8192, [(0, 512)]),
     "llama8b-prefill512-d7680": ("llama8b", "prefill", 8192, [(7680, 512)]),
     "qwen7b-prefill512-d32256": ("qwen7b", "prefill", 32768, [(32256, 512)]),
-    "qwen1.5b-decode-1k": ("qwen1.5b", "decode", 32768, 1024),
+    "qwen1.5b-decode-1k": ("qwen1.5b", "decode", 32768, 1024),     # earlier positions of the same 32k cache
     "qwen1.5b-decode-8k": ("qwen1.5b", "decode", 32768, 8192),
     "qwen1.5b-decode-32k": ("qwen1.5b", "decode", 32768, 32768),
     "llama8b-decode-8k": ("llama8b", "decode", 8192, 8192),
     "qwen7b-decode-32k": ("qwen7b", "decode", 32768, 32767),
     # the decode layer's call pair (store the token's K/V rows, then attend; reference src/model_gpu.cu:281-282)
     # through the entry point that does both in the attention launches; the two calls are timed beside it
-    "qwen1.5b-decode-8k": ("qwen1.5b", "decode", 32768, 8192),     # earlier positions of the same 32k cache
-    "qwen1.5b-decode-1k": ("qwen1.5b", "decode", 32768, 1024),
     "qwen1.5b-decode-store-32k": ("qwen1.5b", "decode_store", 32768, 32768),
     "qwen1.5b-decode-rope-store-32k": ("qwen1.5b", "decode_rope_store", 32768, 32768),
     # the two mutators of the cache (byte movers; value = bytes read + written per second)
@@ -68,22 +66,33 @@ WORKLOADS = {
     # not part of the path: a plain device copy of known size, the yardstick that the HBM
     # counters (FETCH_SIZE / WRITE_SIZE) and the achievable streaming rate are scaled by
     "hbm-copy-256MiB": (None, "copy", 0, 256 << 20),
+    # not part of the path either: a kernel that only reads, as many bytes per launch as one decode layer's
+    # cache (32 MiB: Qwen2.5-1.5B at 32k and Llama-3-8B at 8k; 64 MiB: Qwen2.5-7B at 32k), launched back to
+    # back over rotating buffers that no cache holds -- what such a launch costs when nothing is computed
+    "hbm-read-32MiB": (None, "read", 0, 32 << 20),
+    "hbm-read-64MiB": (None, "read", 0, 64 << 20),
 }
 # HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
-# WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy.  These are
-# recorded measurements (a counter pass cannot run inside the timed benchmark); None where not taken.
-TRAFFIC = {
-    # (2 KV heads over 8 XCDs: each of the 4 L2s that serve a head fetches that head's K and V itself,
-    # 4 x 4.19 MB, mostly from the Infinity Cache; Q 3.15 MB in, 3.15 MB out)
-    "qwen1.5b-prefill512": 20.12e6 + 3.15e6,
-    "qwen1.5b-prefill512-d3584": 20.12e6 + 3.15e6,
-    "llama8b-prefill512-d4096": 27.53e6 + 8.39e6,
-    "qwen1.5b-decode-32k": 33.68e6 + 0.80e6 + 0.97e6 + 0.006e6,
-    "qwen7b-decode-32k": 67.35e6 + 0.94e6 + 1.12e6 + 0.014e6,
-}
-ALSO = ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k", "llama8b-decode-8k", "qwen1.5b-decode-store-32k",
-        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256",
-        "llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k"]
+# WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy: recorded
+# measurements (a counter pass cannot run inside the timed benchmark), kept with the commit they were
+# taken at in profiles/traffic.json; None where not taken.
+def _load_traffic():
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            doc = json.load(f)
+        return {k: v["bytes_per_launch"] for k, v in doc["workloads"].items()}, doc.get("measured_at_commit")
+    except (OSError, ValueError, KeyError):
+        return {}, None
+
+
+TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
+# Run after the default workload and reported under "also"; the cases the targets are stated on come last, and
+# "targets" at the very end of the line repeats their figures in a few hundred characters.
+ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
+        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k", "hbm-read-32MiB",
+        "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+TARGETS = ["hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
 
 
 def prefill_flops(H, d, P, B):
@@ -111,16 +120,28 @@ def make_layer(torch, seed, H, G, d, n_ctx, n_filled, batch, outliers):
     return q, k.view(torch.int16), v.view(torch.int16)
 
 
-def parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, n_past, batch, scale, n_rows=48):
-    rng = np.random.default_rng(0)
-    toks = sorted({0, batch - 1, *(int(x) for x in rng.integers(0, batch, size=6))})
+def parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, n_past, batch, scale, n_rows=48, seed=0):
+    rng = np.random.default_rng(seed)
+    n_tok = max(1, min(8, n_rows // 4))
+    toks = sorted({0, batch - 1, *(int(x) for x in rng.integers(0, batch, size=max(0, n_tok - 2)))})
     rows = np.array([(t, h) for t in toks for h in rng.choice(H, size=min(H, max(1, n_rows // len(toks))),
                                                               replace=False)], np.int32)
     want = ref.flash_attention_rows(q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
                                     v.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, n_past,
-                                    np.float32(scale))
+                                    np.float32(scale), threads=ref.max_threads())
     got = out.cpu().numpy()[rows[:, 0], rows[:, 1]]
     return rel_err(got, want)
+
+
+def parity_stack(torch, ref, rel_err, stack, H, G, d, n_ctx, n_past, batch, scale, rows_first=48, rows_other=12):
+    """Sampled (token, head) rows of EVERY layer of a timed stack against the CPU oracle (layer 0 more
+    densely); returns the worst figures over the layers."""
+    worst = [0.0, 0.0, 0.0]
+    for l, (q, k, v, out) in enumerate(stack):
+        e = parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, n_past, batch, scale,
+                        n_rows=rows_first if l == 0 else rows_other, seed=l)
+        worst = [max(a, b) for a, b in zip(worst, e)]
+    return worst
 
 
 def cpu_baseline_prefill(ref, layers_qkv, H, G, d, n_ctx, P, B, scale, budget_s=15.0):
@@ -265,8 +286,8 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
         f = prefill_flops(H, d, P, B)
         per_chunk.append(dict(P=P, B=B, launch_us=ms * 1e3, tflops=f / (ms * 1e-3) / 1e12,
                               frac=f / (ms * 1e-3) / PEAK_FLOPS))
-    q, k, v, out = stacks[dom][0]
-    err = parity_rows(torch, ref, rel_err, q, k, v, out, H, G, d, n_ctx, P, B, scale)
+    errs = [parity_stack(torch, ref, rel_err, stacks[ci], H, G, d, n_ctx, Pc, Bc, scale) for ci, (Pc, Bc) in enumerate(chunks)]
+    err = [max(e[i] for e in errs) for i in range(3)]
     res = dict(
         value=flops_step * steps / wall / 1e12, unit="TFLOP/s", ms_per_step=wall / steps * 1e3,
         config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=layers, n_ctx=n_ctx,
@@ -281,8 +302,10 @@ def run_prefill(torch, kernels, name, steps, warmup, with_cpu):
                            "launch_us_back_to_back: stack average including launch gaps"),
         per_chunk=per_chunk,
         eager=dict(ms_per_step=wall_eager / steps * 1e3), graph=dict(ms_per_step=wall_graph / steps * 1e3),
-        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="sampled, layer 0, vs CPU oracle"),
+        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2],
+                    rows=f"worst over sampled rows of all {layers} layers of every chunk, vs CPU oracle"),
     )
+    res["config"]["launch"] = "graph" if wall_graph <= wall_eager else "eager"
     if with_cpu:
         sample = [(ql.cpu().numpy(), kl.view(torch.uint16).cpu().numpy(), vl.view(torch.uint16).cpu().numpy())
                   for ql, kl, vl, _ in stacks[dom][:6]]
@@ -427,15 +450,18 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
         one_stack((steps - 1) % n_stacks)
         torch.cuda.synchronize()
     q, k, v, out = stacks[(steps - 1) % n_stacks][0]
-    if rope:  # the oracle attends with the rotated query; the cache already holds the rotated row
-        q = q.clone()
-        kernels.rope_neox_ind(q, H, d, d, theta, dpos)
-        torch.cuda.synchronize()
     rows = np.array([(0, h) for h in range(H)], np.int32)
-    want = ref.flash_attention_rows(q.cpu().numpy()[None], k.view(torch.uint16).cpu().numpy(),
-                                    v.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, L - 1,
-                                    np.float32(scale))
-    err = rel_err(out.cpu().numpy(), want)
+    q_rot = q  # layer 0's query as the oracle wants it
+    err = [0.0, 0.0, 0.0]
+    for ql, kl, vl, outl in stacks[(steps - 1) % n_stacks]:  # every head of every layer of the stack that ran last
+        if rope:
+            ql = ql.clone()
+            kernels.rope_neox_ind(ql, H, d, d, theta, dpos)
+            torch.cuda.synchronize()
+        want = ref.flash_attention_rows(ql.cpu().numpy()[None], kl.view(torch.uint16).cpu().numpy(),
+                                        vl.view(torch.uint16).cpu().numpy(), rows, H, G, d, n_ctx, L - 1,
+                                        np.float32(scale), threads=ref.max_threads())
+        err = [max(a, b) for a, b in zip(err, rel_err(outl.cpu().numpy(), want))]
     wall = min(wall_graph, wall_eager)
     launch_us = min(dev_graph_ms, dev_eager_ms) * 1e3 / (steps * layers)
     res = dict(
@@ -453,7 +479,7 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
                            "kernel alone, which include about 2 us of dispatch latency each"),
         eager=dict(ms_per_step=wall_eager / steps * 1e3, device_ms_per_step=dev_eager_ms / steps),
         graph=dict(ms_per_step=wall_graph / steps * 1e3, device_ms_per_step=dev_graph_ms / steps),
-        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows="all heads, layer 0, vs CPU oracle"),
+        parity=dict(err_row=err[0], err_floor1pct=err[1], rel_l2=err[2], rows=f"all heads of all {layers} layers, vs CPU oracle"),
     )
     if store:
         mode = "rotate + store" if rope else "store"
@@ -466,6 +492,10 @@ def run_decode(torch, kernels, name, steps, warmup, with_cpu):
                else "kv_store_ind + flash_attention_decode_ind")
         res["roofline"]["note"] += f"; launch_us_separate_calls: {sep} per layer, back to back, eager and replayed from a graph"
     if with_cpu:
+        if rope:  # the oracle attends with the rotated query; the cache already holds the rotated row
+            q = q.clone()
+            kernels.rope_neox_ind(q, H, d, d, theta, dpos)
+            torch.cuda.synchronize()
         res["cpu_baseline"] = cpu_baseline_decode(ref, q.cpu().numpy(), k.view(torch.uint16).cpu().numpy(),
                                                   v.view(torch.uint16).cpu().numpy(), H, G, d, n_ctx, L, scale)
     del stacks, graphs
@@ -663,9 +693,73 @@ def run_copy(torch, kernels, name, steps, warmup, with_cpu):
                 parity=None)
 
 
+def run_read(torch, kernels, name, steps, warmup, with_cpu):
+    """A kernel that only reads: `nbytes` per launch, launched back to back over buffers that rotate through
+    more memory than the last-level cache holds; the best of three load shapes is reported, all are listed.
+    One step = 28 launches (a decode stack's worth).  Beside it, the launch-to-launch time of a one-wave kernel."""
+    nbytes = WORKLOADS[name][3]
+    launches = 28
+    n_buf = max(launches, int(np.ceil(1.2e9 / nbytes)))
+    pool = torch.empty(n_buf * nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    bufs = [pool[i * nbytes:(i + 1) * nbytes] for i in range(n_buf)]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    shapes, wall_best = {}, None
+    for per in (16, 4, 2):
+        k = 0
+
+        def one_step():
+            nonlocal k
+            for _ in range(launches):
+                kernels.bench_hbm_read(bufs[k % n_buf], nbytes, per)
+                k += 1
+
+        for _ in range(warmup):
+            one_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            one_step()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        us = e0.elapsed_time(e1) * 1e3 / (steps * launches)
+        shapes[f"{per}_loads_per_thread"] = us
+        if wall_best is None or us < best_us:
+            best_us, wall_best = us, wall
+    # launch-to-launch time of a one-wave kernel, replayed from a graph so that the host's own pace does not count
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            for _ in range(200):
+                kernels.bench_tiny_launch()
+    finally:
+        kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+    g.replay()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(5):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    tiny_us = e0.elapsed_time(e1) * 1e3 / 1000
+    del g
+    del bufs, pool
+    torch.cuda.empty_cache()
+    return dict(value=nbytes * launches * steps / wall_best / 1e9, unit="GB/s", ms_per_step=wall_best / steps * 1e3,
+                config=dict(workload=name, bytes_per_launch=nbytes, launches_per_step=launches, buffers_rotated=n_buf),
+                roofline=dict(bound="hbm", achieved=nbytes / (best_us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (best_us * 1e-6) / PEAK_BYTES, traffic=float(nbytes),
+                              kernel="hbm_read_kernel (plain streaming read, not part of the path)", launch_us=best_us,
+                              launch_us_by_shape=shapes, tiny_kernel_launch_to_launch_us=tiny_us,
+                              bytes_per_launch=nbytes),
+                parity=None)
+
+
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
@@ -699,17 +793,38 @@ def main():
         dtype="f16", data="synthetic",
     )
     line.update(main_res)
+    if TRAFFIC_COMMIT:
+        line["roofline"]["traffic_measured_at_commit"] = TRAFFIC_COMMIT
     if not args.no_also:
         also = []
         for name in ALSO:
             if name == args.workload:
                 continue
-            r = run(torch, kernels, name, max(3, min(args.steps, 10)), min(args.warmup, 2), False)
+            r = run(torch, kernels, name, max(3, min(args.steps, 10)), min(args.warmup, 2),
+                    name in ALSO_CPU and not args.no_cpu)
+            r["roofline"].pop("note", None)
             also.append(dict(workload=name, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
                              roofline=r["roofline"], parity=r["parity"],
                              **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {}),
-                             **({"into_the_cache": r["into_the_cache"]} if "into_the_cache" in r else {})))
+                             **({"into_the_cache": r["into_the_cache"]} if "into_the_cache" in r else {}),
+                             **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})))
         line["also"] = also
+        # The figures the targets are stated on, once more and briefly, as the last thing on the line.
+        targets = {}
+        for a in also:
+            if a["workload"] in TARGETS:
+                rf = a["roofline"]
+                t = dict(frac=round(rf["frac"], 4), achieved=round(rf["achieved"], 1), unit=rf["unit"],
+                         launch_us=round(rf["launch_us"], 2))
+                if a["parity"]:
+                    t["err_row"] = float(f"{a['parity']['err_row']:.2e}")
+                    t["err_floor1pct"] = float(f"{a['parity']['err_floor1pct']:.2e}")
+                if "tiny_kernel_launch_to_launch_us" in rf:
+                    t["tiny_launch_us"] = round(rf["tiny_kernel_launch_to_launch_us"], 2)
+                if "cpu_baseline" in a:
+                    t["cpu_GBps_1core"] = round(a["cpu_baseline"]["value"], 3)
+                targets[a["workload"]] = t
+        line["targets"] = targets
     print(json.dumps(line))
 
 

@@ -169,14 +169,6 @@ int orin_fa_decode_rope_store_ind(const float* q, const float* k_new, const floa
  * (src/kernels.cu:1619-1657); for orin_fa_decode_rope_store_ind, once per token. */
 int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* freq_factors, const int* d_pos);
 
-/* Measurement aid with no counterpart in the reference: orin_fa_decode_ind with HIP events
- * recorded before, between and after its two kernels on the library's stream.  Synchronises
- * on the last event and returns the elapsed time of the split kernel and of the combine
- * kernel in microseconds (the latter 0 when the shape needs no split).  Not capture-safe. */
-int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
-                             int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
-                             float* us_split, float* us_combine);
-
 /* Introspection for tests and benchmarks: the number of KV splits a decode launch
  * with these shapes uses (0 if the shape is rejected), and the CU count seen at init. */
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx);

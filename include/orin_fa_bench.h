@@ -1,0 +1,38 @@
+/*
+ * orin_fa_bench -- measurement aids exported by liborin_fa.so beside the product ABI of
+ * include/orin_fa.h.  None of them has a counterpart in the reference and none is part of the
+ * attention path: bench.py uses them for the yardsticks its figures are read against.  An
+ * engine has no reason to call them.
+ */
+#ifndef ORIN_FA_BENCH_H
+#define ORIN_FA_BENCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* orin_fa_decode_ind with HIP events recorded before, between and after its two kernels on the
+ * library's stream.  Synchronises on the last event and returns the elapsed time of the split
+ * kernel and of the combine kernel in microseconds (the latter 0 when the shape needs no
+ * split).  Not capture-safe. */
+int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+                             int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
+                             float* us_split, float* us_combine);
+
+/* One launch, on the library's stream, of a kernel that does nothing but read `bytes` bytes at
+ * src (device, 16-byte aligned) once with streaming 128-bit loads spread over every CU:
+ * loads_per_thread (2, 4, 8 or 16) 16-byte loads per thread of 512-thread workgroups.  What a
+ * decode step's cache read costs when nothing else is done with the bytes.  Asynchronous. */
+int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread);
+
+/* One launch, on the library's stream, of a one-wave kernel that reads one word: the cost of
+ * a launch as such, when timed back to back.  Asynchronous. */
+int orin_fa_bench_tiny_launch(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "liborin_fa.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
-           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
+           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-exceptions",

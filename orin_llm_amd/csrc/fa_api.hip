@@ -10,6 +10,7 @@
 #include <stdio.h>
 
 #include "../../include/orin_fa.h"
+#include "../../include/orin_fa_bench.h"
 
 namespace orin_fa {
 namespace {
@@ -357,6 +358,22 @@ int orin_fa_rope_store_batch(float* q, float* k, const float* v, uint16_t* kc, u
         if (e != hipSuccess) return hip_code(e);
     }
     return hip_code(kv_store_launch(kc, vc, k, v, n_kv, head_dim, n_ctx, n_past, batch, nullptr, g_state.stream));
+}
+
+// ---- measurement aids (include/orin_fa_bench.h) ----
+int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!src || (reinterpret_cast<uintptr_t>(src) & 15u)) return ORIN_FA_E_INVALID;
+    // (the word that is never written lives in the library's own workspace block)
+    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
+    return hip_code(hbm_read_launch(src, bytes, loads_per_thread, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
+}
+
+int orin_fa_bench_tiny_launch(void) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
+    unsigned* const w = static_cast<unsigned*>(g_state.own_ws);
+    return hip_code(tiny_launch(w, w + 64, g_state.stream));
 }
 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {

@@ -85,6 +85,10 @@ hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, u
 hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
                               hipStream_t stream);
 
+// Measurement aids (bench_aids.hip).
+hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream);
+hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream);
+
 template <int N>
 struct IntC {
     static constexpr int value = N;

@@ -69,6 +69,10 @@ def lib():
         L.orin_fa_decode_ind_timed.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
                                                ctypes.POINTER(_flt), ctypes.POINTER(_flt)]
         L.orin_fa_decode_ind_timed.restype = _int
+        L.orin_fa_bench_hbm_read.argtypes = [_vp, ctypes.c_size_t, _int]
+        L.orin_fa_bench_hbm_read.restype = _int
+        L.orin_fa_bench_tiny_launch.argtypes = []
+        L.orin_fa_bench_tiny_launch.restype = _int
         L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
         L.orin_fa_decode_splits.restype = _int
         L.orin_fa_cu_count.argtypes = []
@@ -236,3 +240,17 @@ def decode_splits(n_head, n_kv, head_dim, n_ctx):
 
 def cu_count():
     return int(lib().orin_fa_cu_count())
+
+
+def bench_hbm_read(src, nbytes, loads_per_thread=16):
+    """Measurement aid: one launch of a plain streaming read of nbytes at src."""
+    rc = lib().orin_fa_bench_hbm_read(_ptr(src), int(nbytes), int(loads_per_thread))
+    if rc != 0:
+        raise OrinFaError("bench_hbm_read", rc)
+
+
+def bench_tiny_launch():
+    """Measurement aid: one launch of a one-wave kernel."""
+    rc = lib().orin_fa_bench_tiny_launch()
+    if rc != 0:
+        raise OrinFaError("bench_tiny_launch", rc)

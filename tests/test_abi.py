@@ -9,6 +9,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "orin_llm_amd", "liborin_fa.so")
 HDR = os.path.join(ROOT, "include", "orin_fa.h")
+BENCH_HDR = os.path.join(ROOT, "include", "orin_fa_bench.h")
 SHIM_HDR = os.path.join(ROOT, "include", "orin_llm_amd", "kernels.h")
 REF_HDR = "/root/reference/src/kernels.h"
 
@@ -18,8 +19,8 @@ def _strip_comments(text):
     return re.sub(r"//[^\n]*", " ", text)
 
 
-def _declared_c_functions():
-    body = _strip_comments(open(HDR).read())
+def _declared_c_functions(header=HDR):
+    body = _strip_comments(open(header).read())
     return sorted(set(re.findall(r"\b(orin_fa_[a-z_]+)\s*\(", body)))
 
 
@@ -33,14 +34,19 @@ def lib():
 def test_header_declares_the_expected_entry_points():
     assert _declared_c_functions() == sorted([
         "orin_fa_init", "orin_fa_set_stream", "orin_fa_workspace_bytes", "orin_fa_set_workspace",
-        "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_ind_static", "orin_fa_static_scratch_bytes", "orin_fa_decode_store_ind", "orin_fa_decode_rope_store_ind", "orin_fa_rope_angles_ind", "orin_fa_rope_store_batch", "orin_fa_decode_ind_timed", "orin_fa_decode_splits",
+        "orin_fa_prefill", "orin_fa_decode_ind", "orin_fa_decode_ind_static", "orin_fa_static_scratch_bytes", "orin_fa_decode_store_ind", "orin_fa_decode_rope_store_ind", "orin_fa_rope_angles_ind", "orin_fa_rope_store_batch", "orin_fa_decode_splits",
         "orin_fa_kv_store_batch", "orin_fa_kv_store_ind", "orin_fa_kv_shift", "orin_fa_rope_batch", "orin_fa_rope_ind", "orin_fa_cu_count",
         "orin_fa_error_string"])
 
 
+def test_measurement_aids_sit_in_their_own_header():
+    assert _declared_c_functions(BENCH_HDR) == sorted(["orin_fa_decode_ind_timed", "orin_fa_bench_hbm_read",
+                                                       "orin_fa_bench_tiny_launch"])
+
+
 def test_library_exports_every_declared_symbol(lib):
-    for name in _declared_c_functions():
-        assert hasattr(lib, name), f"{name} declared in include/orin_fa.h but not exported"
+    for name in _declared_c_functions() + _declared_c_functions(BENCH_HDR):
+        assert hasattr(lib, name), f"{name} declared in a header but not exported"
 
 
 def test_calls_that_need_no_device(lib):

@@ -30,7 +30,7 @@ def test_decode_bytes_counts_k_and_v_once_plus_q_and_out():
 def test_workload_table_is_consistent():
     assert bench.WORKLOADS["qwen1.5b-prefill512"][3] == [(0, 512), (3584, 512)]   # the configuration the metric is quoted on
     for name, (shape, kind, n_ctx, spec) in bench.WORKLOADS.items():
-        assert kind in ("prefill", "decode", "decode_store", "decode_rope_store", "copy", "kv_store", "kv_shift", "rope"), name
+        assert kind in ("prefill", "decode", "decode_store", "decode_rope_store", "copy", "read", "kv_store", "kv_shift", "rope"), name
         if kind == "prefill":
             assert all(P + B <= n_ctx for P, B in spec), name
         if kind in ("decode", "decode_store"):
@@ -39,6 +39,10 @@ def test_workload_table_is_consistent():
             s = bench.SHAPES[shape]
             assert s["H"] % s["G"] == 0 and s["d"] in (64, 128), name
     assert set(bench.ALSO) <= set(bench.WORKLOADS) and set(bench.TRAFFIC) <= set(bench.WORKLOADS)
+    # the cases the targets are stated on close the line, and the recorded traffic names its commit
+    assert bench.ALSO[-3:] == ["llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+    assert set(bench.TARGETS) <= set(bench.ALSO) and bench.ALSO_CPU <= set(bench.ALSO)
+    assert bench.TRAFFIC and bench.TRAFFIC_COMMIT
     assert bench.PEAK_FLOPS == 2.5e15 and bench.PEAK_BYTES == 8.0e12
 
 
