@@ -1,14 +1,15 @@
 """GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
 
-Tolerance (written once, used everywhere): util.TOL = 2e-3 on util.rel_err()[0], the
-maximum error of any fp32 output element relative to the largest magnitude in its own
-(token, head) row.
+Tolerance (written once, in util.py, used everywhere): TOL = 2e-3 on rel_err()[0], the maximum
+error of any fp32 output element relative to the largest magnitude in its own (token, head)
+row; and on rel_err()[1], the element-wise error with a floor of 1 % of the row maximum,
+FLOOR_DECODE = 2e-3 for decode and the bound FLOOR_PREFILL = 5e-2 for prefill.
 """
 import numpy as np
 import pytest
 
 from oracle import ref
-from util import TOL, make_case, rel_err
+from util import FLOOR_DECODE, FLOOR_FP32_KV, FLOOR_PREFILL, TOL, make_case, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -61,11 +62,12 @@ def gpu_decode(fa, q, kc, vc, n_head, n_kv, d, n_ctx, pos, scale, dk=None, dv=No
     return o[:n_head]
 
 
-def check(got, want, what, tol=TOL):
+def check(got, want, what, tol=TOL, floor=FLOOR_PREFILL):
     row, floor1pct, l2 = rel_err(got, want)
-    print(f"{what}: err_row {row:.3e} (gate {tol:g})  floor1pct {floor1pct:.3e}  l2 {l2:.3e}", flush=True)
+    print(f"{what}: err_row {row:.3e} (gate {tol:g})  floor1pct {floor1pct:.3e} (gate {floor:g})  l2 {l2:.3e}", flush=True)
     assert np.isfinite(got).all(), what
     assert row < tol, (what, row, floor1pct, l2)
+    assert floor1pct < floor, (what, row, floor1pct, l2)
 
 
 # ---------------------------------------------------------------- config 1 (golden)
@@ -87,13 +89,13 @@ def test_cfg1_golden_prefill_then_decode(fa, cfg1):
         lg = c["logits_" + variant]
         want = (lg[:, :-1] / lg[:, -1:]).reshape(n_tok, H, d)
         got = gpu_prefill(fa, q[:n_pre], kc, vc, H, G, d, n_ctx, 0, n_pre, scale)
-        check(got, want[:n_pre], f"cfg1{variant} prefill")
+        check(got, want[:n_pre], f"cfg1{variant} prefill", floor=FLOOR_FP32_KV if variant == "a" else FLOOR_PREFILL)
         import torch
 
         dk, dv = _dev(kc), _dev(vc)
         dec = np.stack([gpu_decode(fa, q[t], None, None, H, G, d, n_ctx, t, scale, dk=dk, dv=dv)
                         for t in range(n_pre, n_tok)])
-        check(dec, want[n_pre:], f"cfg1{variant} decode")
+        check(dec, want[n_pre:], f"cfg1{variant} decode", floor=FLOOR_FP32_KV if variant == "a" else FLOOR_DECODE)
         del torch
 
 
@@ -113,7 +115,7 @@ def test_decode_small(fa, d, r):
     for npos in (1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 260, 384):
         want = ref.flash_attention_decode_ind(q[0], kc, vc, H, G, d, n_ctx, npos - 1, np.float32(scale))
         got = gpu_decode(fa, q[0], None, None, H, G, d, n_ctx, npos - 1, scale, dk=dk, dv=dv)
-        check(got, want, f"decode d{d} r{r} npos{npos}")
+        check(got, want, f"decode d{d} r{r} npos{npos}", floor=FLOOR_DECODE)
     del torch
 
 
@@ -216,7 +218,7 @@ def test_prefill_row_equals_decode_and_chunk_split(fa):
     check(np.concatenate([a, b]), whole, "chunk split", tol=1e-3)
     for t in (0, 76, 199):
         dec = gpu_decode(fa, q[t], kc, vc, H, G, d, n_ctx, n_past + t, scale)
-        check(dec, whole[t], f"prefill row {t} vs decode", tol=1e-3)
+        check(dec, whole[t], f"prefill row {t} vs decode", tol=1e-3)  # (prefill against decode: the prefill bound)
 
 
 def test_decode_ignores_cache_tail_and_position_is_read_on_device(fa):
@@ -235,7 +237,7 @@ def test_decode_ignores_cache_tail_and_position_is_read_on_device(fa):
         fa.flash_attention_decode_ind(dq, dk, dv, out, H, G, d, n_ctx, dpos, float(scale))
         torch.cuda.synchronize()
         want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, pos, np.float32(scale))
-        check(out.cpu().numpy(), want, f"decode pos {pos}")
+        check(out.cpu().numpy(), want, f"decode pos {pos}", floor=FLOOR_DECODE)
 
 
 def test_decode_graph_capture_replay(fa):
@@ -272,7 +274,7 @@ def test_decode_graph_capture_replay(fa):
         for l in range(n_layer):
             want = ref.flash_attention_rows(cases[l][0], cases[l][1], cases[l][2], rows, H, G, d, n_ctx, pos,
                                             np.float32(scale))
-            check(outs[l].cpu().numpy(), want, f"graph replay pos {pos} layer {l}")
+            check(outs[l].cpu().numpy(), want, f"graph replay pos {pos} layer {l}", floor=FLOOR_DECODE)
 
 
 # ---------------------------------------------------------------- BASELINE configs at full size (row-sampled oracle)
@@ -322,7 +324,27 @@ def test_decode_full_configs(fa, name, H, G, n_ctx, L, outliers):
         q, kc, vc = make_case(2000 + 13 * layer + L, H, G, d, n_ctx, L, 1, outliers=outliers, poison_tail=True)
         want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, L - 1, np.float32(scale))
         got = gpu_decode(fa, q[0], kc, vc, H, G, d, n_ctx, L - 1, scale)
-        check(got, want, f"{name} layer {layer}")
+        check(got, want, f"{name} layer {layer}", floor=FLOOR_DECODE)
+
+
+def test_cfg2_full_stack_28_layers(fa):
+    """Config 2 as written: the full 28-layer stack with independent seeds per layer, both chunks
+    (cache start positions 0 and 3584), sampled rows of every layer against the oracle."""
+    H, G, d, n_ctx, batch, layers = 12, 2, 128, 4096, 512, 28
+    scale = 1.0 / np.sqrt(d)
+    worst = 0.0
+    for n_past in (0, 3584):
+        for layer in range(layers):
+            q, kc, vc = make_case(50000 + 100 * layer + (n_past > 0), H, G, d, n_ctx, n_past + batch, batch,
+                                  outliers=4, poison_tail=True)
+            rng = np.random.default_rng(layer)
+            toks = sorted({0, batch - 1, *(int(t) for t in rng.integers(0, batch, size=10))})
+            rows = np.array([(t, int(h)) for t in toks for h in rng.choice(H, size=4, replace=False)], np.int32)
+            want = ref.flash_attention_rows(q, kc, vc, rows, H, G, d, n_ctx, n_past, np.float32(scale), threads=ref.max_threads())
+            got = gpu_prefill(fa, q, kc, vc, H, G, d, n_ctx, n_past, batch, scale)
+            check(got[rows[:, 0], rows[:, 1]], want, f"cfg2 P{n_past} layer {layer}")
+            worst = max(worst, rel_err(got[rows[:, 0], rows[:, 1]], want)[0])
+    print(f"cfg2 28 layers x 2 chunks: worst err_row {worst:.3e}", flush=True)
 
 
 # ---------------------------------------------------------------- error behaviour

@@ -14,7 +14,7 @@ import numpy as np
 import pytest
 
 from oracle import ref
-from util import TOL, rel_err
+from util import FLOOR_PREFILL, TOL, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -97,7 +97,8 @@ def test_prefill_layer_through_the_shim(shim):
     assert (stored != kc_ref[:, n_past:n_past + batch]).mean() < 1e-3
     assert np.array_equal(dvc.cpu().numpy().view(np.uint16), vc_ref)
     got = out.cpu().numpy()[rows[:, 0], rows[:, 1]]
-    assert rel_err(got, want)[0] < TOL
+    e = rel_err(got, want)
+    assert e[0] < TOL and e[1] < FLOOR_PREFILL, e
 
 
 def test_decode_steps_through_the_shim_replayed_from_a_graph(shim):
@@ -152,7 +153,8 @@ def test_decode_steps_through_the_shim_replayed_from_a_graph(shim):
             k_ref = ref.rope_batch(k[l], D, D, THETA, pos, G, None, True)
             ref.kv_store_f16(kcs[l], vcs[l], k_ref[None], v[l][None], G, D, n_ctx, pos, 1)
             want = ref.flash_attention_rows(q_ref[None], kcs[l], vcs[l], rows, H, G, D, n_ctx, pos, np.float32(SCALE))
-            assert rel_err(got[l], want)[0] < TOL, (pos, l)
+            e = rel_err(got[l], want)  # (the rotated K row may differ from the oracle's in a last bit: the prefill bound)
+            assert e[0] < TOL and e[1] < FLOOR_PREFILL, (pos, l, e)
         for l in range(n_layer):   # the oracle's caches follow every layer, checked or not
             if l not in (0, 13, n_layer - 1):
                 k_ref = ref.rope_batch(k[l], D, D, THETA, pos, G, None, True)

@@ -1,8 +1,20 @@
 """Shared helpers for the parity tests: input generators and the error metric."""
 import numpy as np
 
-# Gate for GPU-vs-oracle comparisons: max relative error on fp32 outputs (rel_err()[0]).
+# Gates for GPU-vs-oracle comparisons on fp32 outputs (figures of rel_err()).
+#   TOL            err_row < 2e-3, everywhere.
+#   FLOOR_DECODE   err_floor1pct < 2e-3 for decode (fp16 hi + lo operands: fp32-accurate), wherever
+#                  both sides read the same cache values.
+#   FLOOR_PREFILL  err_floor1pct < 5e-2 for prefill: its weights P are single fp16 values (the
+#                  reference GPU kernel's choice too), whose rounding alone costs about
+#                  100 x err_row on this figure; the bound keeps that figure from drifting.
+#   FLOOR_FP32_KV  err_floor1pct < 1e-1 where the reference side kept K/V in fp32 and the GPU
+#                  reads the fp16 cache (config 1, faithful variant): the cache format alone
+#                  scores 4.9e-2 (tests/test_oracle.py::test_fp16_cache_format_error).
 TOL = 2e-3
+FLOOR_DECODE = 2e-3
+FLOOR_PREFILL = 5e-2
+FLOOR_FP32_KV = 1e-1
 
 
 def rel_err(got, ref):
@@ -14,9 +26,10 @@ def rel_err(got, ref):
                      zero, so the error of each element is taken relative to the largest
                      magnitude of its own output row.
       err_floor1pct  max_i |got_i - ref_i| / max(|ref_i|, 0.01 * rowmax): a stricter variant,
-                     reported only.  The fp16 cache format alone (fp32 CPU cache vs the same
-                     values rounded to fp16, no GPU involved) already scores 4.9e-2 on it for
-                     config 1, see tests/test_oracle.py::test_fp16_cache_format_error.
+                     gated at FLOOR_DECODE for decode and bounded by FLOOR_PREFILL for prefill.
+                     The fp16 cache format alone (fp32 CPU cache vs the same values rounded to
+                     fp16, no GPU involved) already scores 4.9e-2 on it for config 1, see
+                     tests/test_oracle.py::test_fp16_cache_format_error.
       rel_l2         ||got - ref|| / ||ref|| over the whole tensor.
     """
     got = np.asarray(got, np.float64)
