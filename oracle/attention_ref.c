@@ -12,8 +12,11 @@
  *   orc_flash_attention*, _rows           composition of the above, checked against the same fixtures
  *   orc_kv_store_*                        exact against numpy astype(float16) at the documented offset
  *   orc_kv_shift_u16                      exact against the slice statement new[keep:n-s] = old[keep+s:], tail 0
- *   orc_rope_*                            float64 rotation by the same fp32 angle; neox == permuted normal, bit for bit;
- *                                         position 0 is the identity; elements past n_rot untouched
+ *   orc_rope_*                            bit-exact logits of the unmodified reference CPU build run with its rotary
+ *                                         embedding on (tests/golden/rope_reference.npz: NeoX and adjacent pairs,
+ *                                         frequency factors, n_rot < head_dim, positions near 0 and near 32768);
+ *                                         float64 rotation by the same fp32 angle; neox == permuted normal, bit for
+ *                                         bit; position 0 is the identity; elements past n_rot untouched
  */
 #include "attention_ref.h"
 

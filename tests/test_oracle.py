@@ -234,3 +234,60 @@ def test_invariants():
     again = ref.flash_attention(qb, kc2, vc, n_head, n_kv, d, n_ctx, 60, 40, scale)
     assert np.array_equal(again[:35].view(np.uint32), whole[:35].view(np.uint32))
     assert not np.array_equal(again[35:], whole[35:])
+
+
+# ---------------------------------------------------------------- rotary embedding, pinned on a reference run
+
+@pytest.fixture(scope="module")
+def rope_golden():
+    """Logits of the unmodified reference CPU build with its rotary embedding on
+    (tests/golden/make_rope_fixture.py)."""
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "rope_reference.npz"))
+    n_head, n_kv, d, n_tok, pos_hi, n_ctx_hi, out_base, n_embd = (int(x) for x in z["meta"])
+    return dict(z=z, n_head=n_head, n_kv=n_kv, d=d, n_tok=n_tok, pos_hi=pos_hi, n_ctx_hi=n_ctx_hi,
+                out_base=out_base, n_embd=n_embd)
+
+
+@pytest.mark.parametrize("where", ["lo", "hi"])
+@pytest.mark.parametrize("name,n_rot,theta,with_ff,neox", [
+    ("neox", 128, 1.0e6, False, True),       # arch qwen2 => NeoX pairing (reference src/model_common.cpp:30-33)
+    ("normal", 128, 5.0e5, True, False),     # arch llama => adjacent pairs, with rope_freqs.weight (:36-41)
+    ("partial", 64, 10000.0, False, False),  # n_rot < head_dim, the reference's default base (:24-25)
+])
+def test_rope_store_attention_reproduce_reference_logits(rope_golden, name, n_rot, theta, with_ff, neox, where):
+    """oracle rope -> cache write -> attention, pushed through the synthetic model's tail, equals the
+    logits of the reference's own rope_neox / rope_normal + attention (src/model_cpu.cpp:179-203,
+    264-295) bit for bit, at small positions and at positions near 32768."""
+    g = rope_golden
+    z, H, G, d, n_tok = g["z"], g["n_head"], g["n_kv"], g["d"], g["n_tok"]
+    pos0, n_ctx = (0, 256) if where == "lo" else (g["pos_hi"], g["n_ctx_hi"])
+    ff = z["factors"][:n_rot // 2] if with_ff else None
+    logits = z[f"logits_{name}_{where}"]
+    kc = np.zeros((G, n_ctx, d), np.float32)  # (the CPU backend's caches start as zeros, rows below pos0 stay so)
+    vc = np.zeros((G, n_ctx, d), np.float32)
+    scale = np.float32(1.0) / np.sqrt(np.float32(d))
+    cfg = dict(n_embd=g["n_embd"], out_base=g["out_base"])
+    for t in range(n_tok):
+        pos = pos0 + t
+        q_rot = ref.rope_batch(z["q"][t].reshape(H, d), d, n_rot, theta, pos, H, ff, neox)
+        k_rot = ref.rope_batch(z["k"][t].reshape(G, d), d, n_rot, theta, pos, G, ff, neox)
+        if n_rot < d:  # elements at or past n_rot are untouched
+            assert np.array_equal(q_rot[:, n_rot:], z["q"][t].reshape(H, d)[:, n_rot:])
+        ref.kv_store_f32(kc, vc, k_rot.reshape(1, G, d), z["v"][t].reshape(1, G, d), G, d, n_ctx, pos, 1)
+        attn = ref.attention_token_f32(q_rot, kc, vc, H, G, d, n_ctx, pos + 1, scale)
+        mine = _tail_logits(cfg, t, attn)
+        assert np.array_equal(mine.view(np.uint32), logits[t].view(np.uint32)), f"{name} {where} token {t}"
+
+
+def test_rope_golden_cases_differ(rope_golden):
+    """The three cases and the two position ranges are really different computations (a fixture in
+    which the rotation had been skipped would make the test above vacuous)."""
+    z = rope_golden["z"]
+    keys = [f"logits_{n}_{w}" for n in ("neox", "normal", "partial") for w in ("lo", "hi")]
+    for i, a in enumerate(keys):
+        for b in keys[i + 1:]:
+            assert not np.allclose(z[a], z[b], rtol=1e-3, atol=1e-3), (a, b)
+    # position 0 rotates by nothing: token 0 of every "lo" run is the same attention (a single key)
+    assert np.array_equal(z["logits_neox_lo"][0], z["logits_normal_lo"][0])
