@@ -19,6 +19,9 @@
  *   kc, vc   IEEE binary16 bit patterns in uint16_t, one layer's cache,
  *            element (kv_head, pos, i) at (kv_head * n_ctx + pos) * head_dim + i
  *   GQA map  query head h reads KV head h / (n_head / n_kv)
+ * Alignment: q, out, kc, vc (and k_new, v_new) of the attention entry points must be 16-byte
+ * aligned (ORIN_FA_E_INVALID otherwise; the reference accepts any alignment of its element
+ * types); the KV-cache mutators and the rotary embedding accept any alignment.
  */
 #ifndef ORIN_FA_H
 #define ORIN_FA_H
@@ -55,7 +58,10 @@ void orin_fa_set_stream(void* stream);
  * aligned).  Optional: orin_fa_init already allocates a block of this size.
  * orin_fa_prefill uses the same block when it cuts a long context's KV rows among
  * workgroups (few query columns, 3072 rows or more): launches that use the block must
- * not overlap, which one stream guarantees. */
+ * not overlap, which one stream guarantees.  The block's address is baked into a captured
+ * graph like every other pointer argument: set the workspace before capturing, keep the
+ * block alive while the graph may be replayed, and capture again after changing it (a second
+ * orin_fa_init on another device releases the library's own block and allocates it there). */
 size_t orin_fa_workspace_bytes(void);
 int orin_fa_set_workspace(void* dev_ptr, size_t bytes);
 

@@ -108,3 +108,39 @@ def test_shim_header_matches_reference_declarations():
     for name in ("flash_attention", "flash_attention_decode_ind", "kv_store_batch", "kv_store_ind", "kv_shift",
                  "rope_neox_batch", "rope_normal_batch", "rope_neox_ind", "rope_normal_ind"):
         assert _decl(ours, name) == _decl(ref, name)
+
+
+def test_caller_built_against_the_reference_header_links_to_the_library(tmp_path):
+    """A translation unit that includes the reference's own src/kernels.h and calls the path's
+    operators the way src/model_gpu.cu does (default freq_factors included) links against
+    liborin_fa.so with nothing unresolved.  Built, never run; needs the reference tree."""
+    if not os.path.exists(REF_HDR):
+        pytest.skip("reference tree not mounted")
+    src = tmp_path / "caller.cpp"
+    src.write_text('''
+#include "kernels.h"
+int main(int argc, char**) {
+    float* q = nullptr; float* out = nullptr; uint16_t* kc = nullptr; uint16_t* vc = nullptr; int* d_pos = nullptr;
+    float* k = nullptr; float* v = nullptr;
+    if (argc > 1000) {  // never taken: the calls only have to resolve
+        llm::cuda::init();
+        llm::cuda::set_stream(nullptr);
+        llm::cuda::rope_neox_batch(q, 512 * 12, 128, 128, 1e6f, 0, 12);
+        llm::cuda::rope_normal_batch(k, 512 * 2, 128, 128, 1e6f, 0, 2);
+        llm::cuda::kv_store_batch(kc, vc, k, v, 2, 128, 4096, 0, 512);
+        llm::cuda::flash_attention(q, kc, vc, out, 12, 2, 128, 4096, 0, 512, 0.088f);
+        llm::cuda::rope_neox_ind(q, 12, 128, 128, 1e6f, d_pos);
+        llm::cuda::rope_normal_ind(k, 2, 128, 128, 1e6f, d_pos);
+        llm::cuda::kv_store_ind(kc, vc, k, v, 2, 128, 4096, d_pos);
+        llm::cuda::flash_attention_decode_ind(q, kc, vc, out, 12, 2, 128, 4096, d_pos, 0.088f);
+        llm::cuda::kv_shift(kc, vc, 28, 2, 128, 4096, 4, 2046);
+    }
+    return 0;
+}
+''')
+    exe = tmp_path / "caller"
+    r = subprocess.run(["g++", "-std=c++17", "-I", os.path.dirname(REF_HDR), "-I", "/root/reference/include", str(src),
+                        "-o", str(exe), "-L", os.path.dirname(LIB), "-lorin_fa", "-Wl,--no-undefined",
+                        "-Wl,--allow-shlib-undefined", "-Wl,-rpath," + os.path.dirname(LIB)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
