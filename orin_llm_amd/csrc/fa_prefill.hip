@@ -170,15 +170,15 @@ __device__ __forceinline__ void reg_load16(u32x4& dst, i32x4 desc, int off, int 
 }
 
 // One such copy, for the main loop, which deals them out between the matrix instructions so
-// that the vector-memory issue queue never backs up.  The LDS base is whatever set_lds_base()
-// put into M0 last: nothing else in the loop touches that register (the compiler has no reason
-// to -- it generates no LDS-directed loads, relative moves or lane reads of its own there).
-__device__ __forceinline__ void set_lds_base(unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %0" : : "s"(lds_base) : "memory", "m0");
-}
+// that the vector-memory issue queue never backs up.  The LDS base is written to M0 inside the
+// same block as the copy that uses it (as lds_copy_4k does), so nothing the compiler may put
+// between two copies can change the destination.
 template <int IMM>
-__device__ __forceinline__ void lds_copy_1k(i32x4 desc, int off, int soff) {
-    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds" : : "v"(off), "s"(desc), "s"(soff), "n"(IMM) : "memory", "m0");
+__device__ __forceinline__ void lds_copy_1k(i32x4 desc, unsigned lds_base, int off, int soff) {
+    asm volatile("s_mov_b32 m0, %4\n\tbuffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds"
+                 :
+                 : "v"(off), "s"(desc), "s"(soff), "n"(IMM), "s"(lds_base)
+                 : "memory", "m0");
 }
 
 // The vector instructions of stage B for one 32x32 score block (16 scores per lane), in issue
@@ -331,8 +331,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
     auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
-        if constexpr (sub == 0) set_lds_base(lds_dst + half * 4096);
-        lds_copy_1k<sub * 1024>(d, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
+        lds_copy_1k<sub * 1024>(d, lds_dst + half * 4096, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
     };
     auto k_buf = [&](int par) { return ws_addr + G::kKOff + par * G::kTileB; };
     auto v_buf = [&](int par) { return ws_addr + G::kVOff + par * G::kTileB; };
