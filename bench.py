@@ -71,6 +71,10 @@ WORKLOADS = {
     # back over rotating buffers that no cache holds -- what such a launch costs when nothing is computed
     "hbm-read-32MiB": (None, "read", 0, 32 << 20),
     "hbm-read-64MiB": (None, "read", 0, 64 << 20),
+    # not part of the path: a stand-in for one split-KV decode step (256 workgroups stream 32 MiB and leave 3 KB
+    # partials), its partials merged by a second kernel, as the library does, or inside the launch by a two-level
+    # last-arriver reduction over write-through stores and relaxed atomics -- what fusing the combine would cost
+    "decode-handoff-mock": (None, "handoff", 0, 32 << 20),
 }
 # HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
 # WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy: recorded
@@ -89,9 +93,9 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 # Run after the default workload and reported under "also"; the cases the targets are stated on come last, and
 # "targets" at the very end of the line repeats their figures in a few hundred characters.
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
-        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k", "hbm-read-32MiB",
-        "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
-TARGETS = ["hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k", "decode-handoff-mock",
+        "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
 
 
@@ -757,9 +761,55 @@ def run_read(torch, kernels, name, steps, warmup, with_cpu):
                 parity=None)
 
 
+def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = 28 launches of the stand-in over rotating cold buffers; value = the two-launch form's rate."""
+    nbytes, scratch_bytes = kernels.bench_handoff_sizes()
+    launches = 28
+    n_buf = max(launches, int(np.ceil(1.2e9 / nbytes)))
+    pool = torch.empty(n_buf * nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    scratch = torch.zeros(scratch_bytes, dtype=torch.uint8, device="cuda")
+    outs = {f: torch.zeros(784, device="cuda") for f in (False, True)}
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    us, walls = {}, {}
+    for fused in (False, True):
+        k = 0
+
+        def one_step():
+            nonlocal k
+            for _ in range(launches):
+                kernels.bench_handoff(pool[(k % n_buf) * nbytes:], fused, scratch, outs[fused])
+                k += 1
+
+        for _ in range(warmup):
+            one_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            one_step()
+        e1.record()
+        torch.cuda.synchronize()
+        walls[fused] = time.perf_counter() - t0
+        us[fused] = e0.elapsed_time(e1) * 1e3 / (steps * launches)
+    want = np.tile(np.array([32896.0, 0.0, 256.0, 384.0], np.float32), 196)
+    want[1::4] = 256.0 * (np.arange(196) & 7)
+    same = bool(np.array_equal(outs[False].cpu().numpy(), want) and np.array_equal(outs[True].cpu().numpy(), want))
+    del pool
+    torch.cuda.empty_cache()
+    return dict(value=nbytes * launches * steps / walls[False] / 1e9, unit="GB/s", ms_per_step=walls[False] / steps * 1e3,
+                config=dict(workload=name, bytes_per_launch=nbytes, launches_per_step=launches, workgroups=256,
+                            partial_floats=784),
+                roofline=dict(bound="hbm", achieved=nbytes / (us[False] * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (us[False] * 1e-6) / PEAK_BYTES, traffic=None,
+                              kernel="handoff_split_kernel<false> + handoff_combine_kernel (stand-in, not part of the path)",
+                              launch_us=us[False], two_launch_us=us[False], fused_two_level_us=us[True],
+                              bytes_per_launch=nbytes),
+                parity=dict(both_forms_give_the_known_sum=same))
+
+
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
@@ -816,7 +866,9 @@ def main():
                 rf = a["roofline"]
                 t = dict(frac=round(rf["frac"], 4), achieved=round(rf["achieved"], 1), unit=rf["unit"],
                          launch_us=round(rf["launch_us"], 2))
-                if a["parity"]:
+                if "fused_two_level_us" in rf:
+                    t = dict(two_launch_us=round(rf["two_launch_us"], 2), fused_two_level_us=round(rf["fused_two_level_us"], 2))
+                elif a["parity"]:
                     t["err_row"] = float(f"{a['parity']['err_row']:.2e}")
                     t["err_floor1pct"] = float(f"{a['parity']['err_floor1pct']:.2e}")
                 if "tiny_kernel_launch_to_launch_us" in rf:

@@ -28,6 +28,18 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
  * decode step's cache read costs when nothing else is done with the bytes.  Asynchronous. */
 int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread);
 
+/* A stand-in for one split-KV decode step, to price the two ways of merging its partial results:
+ * 256 workgroups stream orin_fa_bench_handoff_stream_bytes() (32 MiB) at src and leave 784-float
+ * partial results that are then added up into out[784] -- fused = 0: by a second kernel (two
+ * launches, what the library does); fused = 1: inside the one launch, by a two-level
+ * last-arriver reduction over write-through stores and relaxed agent-scope atomics (no
+ * cache-wide fence).  scratch: orin_fa_bench_handoff_scratch_bytes() of device memory, zeroed
+ * once by the caller before the first call.  out is the same either way (784 floats: element
+ * 4i of every group is the sum of 1..256 = 32896).  Asynchronous, on the library's stream. */
+int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out);
+size_t orin_fa_bench_handoff_scratch_bytes(void);
+size_t orin_fa_bench_handoff_stream_bytes(void);
+
 /* One launch, on the library's stream, of a one-wave kernel that reads one word: the cost of
  * a launch as such, when timed back to back.  Asynchronous. */
 int orin_fa_bench_tiny_launch(void);

@@ -22,6 +22,103 @@ __global__ __launch_bounds__(512) void hbm_read_kernel(const u32x4* __restrict__
     if (acc == 0x9E3779B9u) *sink = acc;
 }
 
+// ---- what a split-KV decode step costs around its stream, two ways ----
+// A stand-in for the decode split kernel: 256 workgroups x 512 threads, each streams 128 KB and
+// leaves a partial result of kPart floats (values that depend on the workgroup only, so that the
+// sum is known).  FUSED = false: the partials are written and a second kernel adds them up
+// (what the library does).  FUSED = true: the partials are merged inside the launch by a
+// two-level "last arriver" reduction -- partials written through to memory (agent scope), one
+// relaxed agent-scope atomic per workgroup on its group's counter, the last of every 16 adds
+// its group's partials up, writes the sum through, arrives at the second counter, and the last
+// of those writes the result; no fence that writes back or invalidates a whole cache.  The last
+// arriver puts the counters back to zero, so launches can follow one another.
+constexpr int kMockWgs = 256, kMockGroup = 16, kPart = 784; // (6 heads x (128 + 2) floats, rounded up to 16 B x 49 x 4)
+constexpr int kPart4 = kPart / 4;
+
+__device__ __forceinline__ f4 ld_agent(const float* base, int idx4) { // 16-byte load that is coherent across the chip
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(base, 0x7fffffff);
+    return __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(r, idx4 * 16, 0, 16));
+}
+__device__ __forceinline__ void st_agent(float* base, int idx4, f4 v) { // 16-byte store written through to memory
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(base, 0x7fffffff);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, idx4 * 16, 0, 16);
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(512) void handoff_split_kernel(const u32x4* __restrict__ src, float* part1, float* part2,
+                                                            float* out, unsigned* ctr) {
+    extern __shared__ unsigned char smem_pad[]; // (as much LDS as the decode kernel: one workgroup per CU)
+    __shared__ unsigned sh_old;
+    const size_t i = (size_t)blockIdx.x * 512 * 16 + threadIdx.x;
+    u32x4 r[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) r[k] = __builtin_nontemporal_load(src + i + k * 512);
+    unsigned acc = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc ^= r[k].x ^ r[k].y ^ r[k].z ^ r[k].w;
+    const float bump = acc == 0x9E3779B9u ? 1.0f : 0.0f; // never: ties the partial to the stream
+    const int t = threadIdx.x;
+    const f4 mine = f4{(float)(blockIdx.x + 1) + bump, (float)(t & 7), 1.0f, (float)(blockIdx.x & 3)};
+    if constexpr (!FUSED) {
+        if (t < kPart4) *reinterpret_cast<f4*>(part1 + ((size_t)blockIdx.x * kPart4 + t) * 4) = mine;
+        return;
+    } else {
+        if (t < kPart4) st_agent(part1, blockIdx.x * kPart4 + t, mine);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the stores have been acknowledged
+        __syncthreads();
+        const int grp = blockIdx.x / kMockGroup;
+        if (t == 0) sh_old = __hip_atomic_fetch_add(&ctr[grp * 32], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (sh_old != kMockGroup - 1) return;
+        if (t == 0) __hip_atomic_store(&ctr[grp * 32], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t < kPart4) {
+            f4 x[kMockGroup];
+#pragma unroll
+            for (int j = 0; j < kMockGroup; ++j) x[j] = ld_agent(part1, (grp * kMockGroup + j) * kPart4 + t);
+            f4 sum = x[0];
+#pragma unroll
+            for (int j = 1; j < kMockGroup; ++j) sum += x[j];
+            st_agent(part2, grp * kPart4 + t, sum);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        constexpr int kGroups = kMockWgs / kMockGroup;
+        if (t == 0) sh_old = __hip_atomic_fetch_add(&ctr[kGroups * 32], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (sh_old != kGroups - 1) return;
+        if (t == 0) __hip_atomic_store(&ctr[kGroups * 32], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t < kPart4) {
+            f4 x[kGroups];
+#pragma unroll
+            for (int j = 0; j < kGroups; ++j) x[j] = ld_agent(part2, j * kPart4 + t);
+            f4 sum = x[0];
+#pragma unroll
+            for (int j = 1; j < kGroups; ++j) sum += x[j];
+            *reinterpret_cast<f4*>(out + t * 4) = sum;
+        }
+    }
+}
+
+// The second launch of the unfused form: 49 workgroups of 4 waves; a wave adds up one 16-byte
+// element of the 256 partials (4 per lane, then across the lanes).
+__global__ __launch_bounds__(256) void handoff_combine_kernel(const float* part1, float* out) {
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    f4 x[kMockWgs / 64];
+#pragma unroll
+    for (int j = 0; j < kMockWgs / 64; ++j) x[j] = *reinterpret_cast<const f4*>(part1 + ((size_t)(lane + 64 * j) * kPart4 + e) * 4);
+    f4 sum = x[0];
+#pragma unroll
+    for (int j = 1; j < kMockWgs / 64; ++j) sum += x[j];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        f4 o;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o[c] = __shfl_xor(sum[c], off);
+        sum += o;
+    }
+    if (lane == 0) *reinterpret_cast<f4*>(out + e * 4) = sum;
+}
+
 // The smallest launch there is: one wave that reads one word.
 __global__ void tiny_kernel(const unsigned* src, unsigned* sink) {
     if (src[threadIdx.x & 1] == 0x9E3779B9u) *sink = 1;
@@ -40,6 +137,32 @@ hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, 
     else if (per == 4) hipLaunchKernelGGL(hbm_read_kernel<4>, dim3(grid), dim3(512), 0, stream, p, sink, n16);
     else if (per == 8) hipLaunchKernelGGL(hbm_read_kernel<8>, dim3(grid), dim3(512), 0, stream, p, sink, n16);
     else hipLaunchKernelGGL(hbm_read_kernel<16>, dim3(grid), dim3(512), 0, stream, p, sink, n16);
+    return hipGetLastError();
+}
+
+// scratch: kHandoffScratchBytes of device memory, zeroed once by the caller (counters at the end).
+hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out, hipStream_t stream) {
+    float* const part1 = static_cast<float*>(scratch);
+    float* const part2 = part1 + (size_t)kMockWgs * kPart;
+    unsigned* const ctr = reinterpret_cast<unsigned*>(part2 + (size_t)(kMockWgs / kMockGroup) * kPart);
+    const u32x4* p = static_cast<const u32x4*>(src);
+    constexpr int lds = 128 * 1024;
+    static bool allowed = false;
+    if (!allowed) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(handoff_split_kernel<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(handoff_split_kernel<true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        allowed = true;
+    }
+    if (fused) {
+        hipLaunchKernelGGL(handoff_split_kernel<true>, dim3(kMockWgs), dim3(512), lds, stream, p, part1, part2, out, ctr);
+    } else {
+        hipLaunchKernelGGL(handoff_split_kernel<false>, dim3(kMockWgs), dim3(512), lds, stream, p, part1, part2, out, ctr);
+        hipLaunchKernelGGL(handoff_combine_kernel, dim3(kPart4 / 4), dim3(256), 0, stream, part1, out);
+    }
     return hipGetLastError();
 }
 

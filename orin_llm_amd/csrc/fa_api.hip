@@ -369,6 +369,17 @@ int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread) 
     return hip_code(hbm_read_launch(src, bytes, loads_per_thread, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
 }
 
+int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!src || !scratch || !out) return ORIN_FA_E_INVALID;
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(scratch) | reinterpret_cast<uintptr_t>(out)) & 15u)
+        return ORIN_FA_E_INVALID;
+    return hip_code(handoff_launch(src, fused, scratch, out, g_state.stream));
+}
+
+size_t orin_fa_bench_handoff_scratch_bytes(void) { return kHandoffScratchBytes; }
+size_t orin_fa_bench_handoff_stream_bytes(void) { return kHandoffStreamBytes; }
+
 int orin_fa_bench_tiny_launch(void) {
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
     if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;

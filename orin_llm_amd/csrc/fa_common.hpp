@@ -88,6 +88,9 @@ hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* 
 // Measurement aids (bench_aids.hip).
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream);
 hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream);
+constexpr size_t kHandoffScratchBytes = 1u << 20; // partials of both levels and the arrival counters
+constexpr size_t kHandoffStreamBytes = (size_t)256 * 512 * 16 * 16; // 32 MiB read per launch
+hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out, hipStream_t stream);
 
 template <int N>
 struct IntC {

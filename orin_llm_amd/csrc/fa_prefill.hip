@@ -61,6 +61,22 @@ struct PGeom {
     static constexpr int kTileB = kTile * kRowB;      // one K or V tile
     static constexpr int kCopies = kTileB / 1024;     // one LDS copy instruction moves 64 lanes x 16 B
     static constexpr int kRowsPerCopy = 1024 / kRowB; // 4 (d=128) or 8 (d=64)
+    static constexpr int kCopyVariants = 16 / kRowsPerCopy; // copies whose rows differ in what the swizzle looks at
+    // The 16-byte chunks of a row sit in LDS in swizzled order: physical chunk p of row r holds
+    // logical chunk p ^ swz(r).  LDS has 64 four-byte banks, i.e. 16 chunk-wide bank groups per
+    // 256 bytes, and two access patterns must each spread over all 16: a K operand read
+    // (ds_read_b128, 16 lanes at a time = 16 consecutive rows, one logical chunk) and a V
+    // transposing read (ds_read_b64_tr_b16, 32 lanes at a time = 4 consecutive rows x 4
+    // consecutive chunks).  d = 128 (a row fills all 16 groups): the row's two low bits go to
+    // chunk bits 3:2, where they separate the 4 rows of a V read, and bits 3:2 of the row to chunk
+    // bits 1:0, which makes 16 consecutive rows distinct.  d = 64 (two rows fill the groups, the
+    // row's lowest bit picks the half): bit 1 of the row goes to chunk bit 2, bits 3:2 to bits
+    // 1:0.  Either way swz(r + 16) = swz(r), and swz(r + 8) differs (second pointer set of the V reads).
+    // (Measured with 4 waves reading: 25.0 instead of 32.1 clocks per K read, 16.3 instead of 32.0 per V read,
+    // where an unconflicted 1 KB read takes 24.7.)
+    __device__ static constexpr int swz(int r) {
+        return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+    }
     static constexpr int kKOff = 0;                   // wave slice: K buffers 0/1, then V buffers 0/1
     static constexpr int kVOff = 2 * kTileB;
     static constexpr int kOStride = D + 4;
@@ -146,15 +162,15 @@ __device__ __forceinline__ i32x4 make_desc(const void* base, unsigned bytes) {
 // part of the range check.  The copies count on the vector-memory counter and complete in
 // issue order; callers wait with s_waitcnt vmcnt(n).  One asm block, so that M0 (the LDS base)
 // cannot change between the copies.
-__device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int off_even, int off_odd, int soff) {
+__device__ __forceinline__ void lds_copy_4k(i32x4 desc, unsigned lds_base, int off0, int off1, int off2, int off3, int soff) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
-        "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
-        "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds\n\t"
-        "buffer_load_dwordx4 %1, %3, %4 offen offset:2048 lds\n\t"
-        "buffer_load_dwordx4 %2, %3, %4 offen offset:3072 lds"
+        "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
+        "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
+        "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
+        "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds"
         :
-        : "s"(lds_base), "v"(off_even), "v"(off_odd), "s"(desc), "s"(soff)
+        : "s"(lds_base), "v"(off0), "v"(off1), "v"(off2), "v"(off3), "s"(desc), "s"(soff)
         : "memory", "m0");
 }
 
@@ -287,42 +303,48 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
 
     // ---- per-lane offsets ----
     // Copy: lane l of copy i lands at LDS byte i*1024 + l*16 = row i*R + l/C, physical chunk l%C,
-    // and physical chunk p of row r holds logical chunk p ^ (r & 7).
-    int g_off[2];
+    // and physical chunk p of row r holds logical chunk p ^ swz(r); copy i is of variant i % kVar.
+    constexpr int kVar = G::kCopyVariants;
+    int g_off[kVar];
     {
         const int r_in = lane / G::kChunks, pc = lane % G::kChunks;
 #pragma unroll
-        for (int par = 0; par < 2; ++par) {
-            const int sw = (par * G::kRowsPerCopy + r_in) & 7;
-            g_off[par] = r_in * G::kRowB + ((pc ^ sw) & (G::kChunks - 1)) * 16;
+        for (int v = 0; v < kVar; ++v) {
+            const int sw = G::swz(v * G::kRowsPerCopy + r_in);
+            g_off[v] = r_in * G::kRowB + ((pc ^ sw) & (G::kChunks - 1)) * 16;
         }
     }
-    constexpr int kOdd = (G::kRowsPerCopy == 4) ? 1 : 0;
     // K operand read: lane (c32, hh) takes row c32, logical chunk ks*2 + hh.  The pointers carry
     // every per-lane term; the buffer parity is an immediate offset.
     const unsigned char* kp[G::kSteps];
 #pragma unroll
-    for (int ks = 0; ks < G::kSteps; ++ks) kp[ks] = ws + G::kKOff + c32 * G::kRowB + (((ks * 2 + hh) ^ (c32 & 7)) * 16);
+    for (int ks = 0; ks < G::kSteps; ++ks) kp[ks] = ws + G::kKOff + c32 * G::kRowB + (((ks * 2 + hh) ^ G::swz(c32)) * 16);
     // V transposing read, per 16-lane group (lane i of the group): addresses row R + i/4, 8-byte
     // column (d0/4 + i%4) and receives rows R..R+3 at head_dim index d0 + i, where d0 = db*32 +
     // 16 * (lane/16 % 2) and R = 16*kh + 4*hh (+8 for the second half of the operand): the
     // operand's k index (hh, j) is KV row 16*kh + 8*(j/4) + 4*hh + j%4, the row that score
     // register 8*kh + j of lane-half hh belongs to.
-    const unsigned char* vp[G::kDBlk];
+    // Rows R + 8 are swizzled differently from rows R (rows R + 16 alike): two pointer sets.
+    const unsigned char* vp[2][G::kDBlk];
     {
         const int i16 = lane & 15, g2 = (lane >> 4) & 1;
-        const int r0 = 4 * hh + (i16 >> 2), sw = r0 & 7;
+        const int r0 = 4 * hh + (i16 >> 2);
 #pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db)
-            vp[db] = ws + G::kVOff + r0 * G::kRowB + (((db * 4 + g2 * 2 + ((i16 & 3) >> 1)) ^ sw) * 16) + (i16 & 1) * 8;
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int db = 0; db < G::kDBlk; ++db)
+                vp[u][db] = ws + G::kVOff + (r0 + 8 * u) * G::kRowB +
+                            (((db * 4 + g2 * 2 + ((i16 & 3) >> 1)) ^ G::swz(r0 + 8 * u)) * 16) + (i16 & 1) * 8;
     }
 
     // Prologue copies: the whole offset is in the (range-checked) vector operand, so rows at or
     // past kv_end of the diagonal tile, and tiles below zero, are not fetched.
     auto copy_checked = [&](const i32x4& desc, unsigned lds_dst, int tile) {
         const int base = tile * G::kTileB;
-        lds_copy_4k(desc, lds_dst, base + g_off[0], base + g_off[kOdd], 0);
-        if (G::kCopies > 4) lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[kOdd], 0);
+        lds_copy_4k(desc, lds_dst, base + g_off[0], base + g_off[1 % kVar], base + g_off[2 % kVar], base + g_off[3 % kVar], 0);
+        if (G::kCopies > 4)
+            lds_copy_4k(desc, lds_dst + 4096, base + 4096 + g_off[0], base + 4096 + g_off[1 % kVar], base + 4096 + g_off[2 % kVar],
+                        base + 4096 + g_off[3 % kVar], 0);
     };
     // Main-loop copies: every tile they name is either wholly inside the visible range, and its
     // base travels as the scalar offset, or below zero (steps past the wave's last tile), and then
@@ -331,7 +353,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
     auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
-        lds_copy_1k<sub * 1024>(d, lds_dst + half * 4096, g_off[(sub & 1) ? kOdd : 0], soff + half * 4096);
+        lds_copy_1k<sub * 1024>(d, lds_dst + half * 4096, g_off[sub % kVar], soff + half * 4096);
     };
     auto k_buf = [&](int par) { return ws_addr + G::kKOff + par * G::kTileB; };
     auto v_buf = [&](int par) { return ws_addr + G::kVOff + par * G::kTileB; };
@@ -370,12 +392,6 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         });
     }
     if (n_mine > 0) copy_checked(kdesc, k_buf(0), tile_of(0));
-    // The arguments that did not arrive in registers are fetched now, beside the first loads: left
-    // alone, the compiler fetches each where it is first used, behind the first products.
-    {
-        const void *p0 = a.out, *p1 = a.part_o, *p2 = a.part_ml;
-        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(a.c));
-    }
     FA_STAMP(9);
     // O = 0: a matrix instruction with a zero addend writes the accumulation registers without
     // touching memory.
@@ -392,6 +408,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             for (int db = 0; db < G::kDBlk; ++db) mfma_o_zero_n(o[cb][db], zero, zero);
         }
     }
+    FA_STAMP(11);
     if (n_mine > 0) {
         // V buffer 0 receives the diagonal tile, whose rows at or past kv_end are not fetched:
         // clear it first, so that no stale bit pattern meets a zero weight (0 * NaN is not 0).
@@ -402,8 +419,17 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         for (int i = 0; i < G::kCopies; ++i)
             *reinterpret_cast<u32x4*>(ws + G::kVOff + i * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        FA_STAMP(12);
         copy_checked(vdesc, v_buf(0), tile_of(0));
+        FA_STAMP(13);
         copy_checked(kdesc, k_buf(1), tile_of(1));
+    }
+    // The arguments that did not arrive in registers are fetched here, behind the prologue's loads
+    // and beside their trip to memory: left alone, the compiler fetches each where it is first
+    // used, one wait behind the other after the first products.
+    {
+        const void *p0 = a.out, *p1 = a.part_o, *p2 = a.part_ml;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(a.c));
     }
     FA_STAMP(10);
     // ---- query block -> LDS (fp16) ----
@@ -548,8 +574,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         auto read_v = [&](auto gc, int par_off) {
             constexpr int g = decltype(gc)::value;
             constexpr int db = g % G::kDBlk, kh = g / G::kDBlk;
-            const h4 v0 = lds_read_tr(vp[db] + par_off + kh * 16 * G::kRowB);
-            const h4 v1 = lds_read_tr(vp[db] + par_off + (kh * 16 + 8) * G::kRowB);
+            const h4 v0 = lds_read_tr(vp[0][db] + par_off + kh * 16 * G::kRowB);
+            const h4 v1 = lds_read_tr(vp[1][db] + par_off + kh * 16 * G::kRowB);
             return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
         };
         static_for<0, kAhead>([&](auto gc) { carry[kAhead - 1 - decltype(gc)::value] = read_v(IntC<kAhead - 1 - decltype(gc)::value>{}, 0); }); // for step 1: V(0)
@@ -721,8 +747,8 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
 #pragma unroll
             for (int j = 0; j < 2 * G::kDBlk; ++j) {
                 const int db = j % G::kDBlk, kh = j / G::kDBlk;
-                const h4 v0 = lds_read_tr(vp[db] + v_par + kh * 16 * G::kRowB);
-                const h4 v1 = lds_read_tr(vp[db] + v_par + (kh * 16 + 8) * G::kRowB);
+                const h4 v0 = lds_read_tr(vp[0][db] + v_par + kh * 16 * G::kRowB);
+                const h4 v1 = lds_read_tr(vp[1][db] + v_par + kh * 16 * G::kRowB);
                 va[j] = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
             }
 #pragma unroll

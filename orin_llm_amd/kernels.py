@@ -71,6 +71,12 @@ def lib():
         L.orin_fa_decode_ind_timed.restype = _int
         L.orin_fa_bench_hbm_read.argtypes = [_vp, ctypes.c_size_t, _int]
         L.orin_fa_bench_hbm_read.restype = _int
+        L.orin_fa_bench_handoff.argtypes = [_vp, _int, _vp, _vp]
+        L.orin_fa_bench_handoff.restype = _int
+        L.orin_fa_bench_handoff_scratch_bytes.argtypes = []
+        L.orin_fa_bench_handoff_scratch_bytes.restype = ctypes.c_size_t
+        L.orin_fa_bench_handoff_stream_bytes.argtypes = []
+        L.orin_fa_bench_handoff_stream_bytes.restype = ctypes.c_size_t
         L.orin_fa_bench_tiny_launch.argtypes = []
         L.orin_fa_bench_tiny_launch.restype = _int
         L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
@@ -254,3 +260,15 @@ def bench_tiny_launch():
     rc = lib().orin_fa_bench_tiny_launch()
     if rc != 0:
         raise OrinFaError("bench_tiny_launch", rc)
+
+
+def bench_handoff(src, fused, scratch, out):
+    """Measurement aid: a stand-in for a split-KV decode step, partial results merged by a second
+    kernel (fused=False) or inside the launch (fused=True)."""
+    rc = lib().orin_fa_bench_handoff(_ptr(src), 1 if fused else 0, _ptr(scratch), _ptr(out))
+    if rc != 0:
+        raise OrinFaError("bench_handoff", rc)
+
+
+def bench_handoff_sizes():
+    return int(lib().orin_fa_bench_handoff_stream_bytes()), int(lib().orin_fa_bench_handoff_scratch_bytes())
