@@ -22,6 +22,11 @@ __global__ __launch_bounds__(512) void hbm_read_kernel(const u32x4* __restrict__
     if (acc == 0x9E3779B9u) *sink = acc;
 }
 
+// The smallest launch there is: one wave that reads one word.
+__global__ void tiny_kernel(const unsigned* src, unsigned* sink) {
+    if (src[threadIdx.x & 1] == 0x9E3779B9u) *sink = 1;
+}
+
 // ---- what a split-KV decode step costs around its stream, two ways ----
 // A stand-in for the decode split kernel: 256 workgroups x 512 threads, each streams 128 KB and
 // leaves a partial result of kPart floats (values that depend on the workgroup only, so that the
@@ -56,9 +61,11 @@ __global__ __launch_bounds__(512) void handoff_split_kernel(const u32x4* __restr
     unsigned acc = 0;
 #pragma unroll
     for (int k = 0; k < 16; ++k) acc ^= r[k].x ^ r[k].y ^ r[k].z ^ r[k].w;
-    const float bump = acc == 0x9E3779B9u ? 1.0f : 0.0f; // never: ties the partial to the stream
+    // (every thread's loads are kept alive by a store that never happens: tied only to the partial, which
+    // 196 of the 512 threads write, the others' loads would be dropped)
+    if (acc == 0x9E3779B9u) ctr[4096] = acc;
     const int t = threadIdx.x;
-    const f4 mine = f4{(float)(blockIdx.x + 1) + bump, (float)(t & 7), 1.0f, (float)(blockIdx.x & 3)};
+    const f4 mine = f4{(float)(blockIdx.x + 1), (float)(t & 7), 1.0f, (float)(blockIdx.x & 3)};
     if constexpr (!FUSED) {
         if (t < kPart4) *reinterpret_cast<f4*>(part1 + ((size_t)blockIdx.x * kPart4 + t) * 4) = mine;
         return;
@@ -119,11 +126,6 @@ __global__ __launch_bounds__(256) void handoff_combine_kernel(const float* part1
     if (lane == 0) *reinterpret_cast<f4*>(out + e * 4) = sum;
 }
 
-// The smallest launch there is: one wave that reads one word.
-__global__ void tiny_kernel(const unsigned* src, unsigned* sink) {
-    if (src[threadIdx.x & 1] == 0x9E3779B9u) *sink = 1;
-}
-
 } // namespace
 
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream) {
@@ -157,11 +159,13 @@ hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out,
         if (e != hipSuccess) return e;
         allowed = true;
     }
-    if (fused) {
+    if (fused == 1) {
         hipLaunchKernelGGL(handoff_split_kernel<true>, dim3(kMockWgs), dim3(512), lds, stream, p, part1, part2, out, ctr);
     } else {
         hipLaunchKernelGGL(handoff_split_kernel<false>, dim3(kMockWgs), dim3(512), lds, stream, p, part1, part2, out, ctr);
-        hipLaunchKernelGGL(handoff_combine_kernel, dim3(kPart4 / 4), dim3(256), 0, stream, part1, out);
+        // (fused = 2: the first kernel alone; 3: followed by a one-wave kernel instead of the combine -- to price the parts)
+        if (fused == 0) hipLaunchKernelGGL(handoff_combine_kernel, dim3(kPart4 / 4), dim3(256), 0, stream, part1, out);
+        else if (fused == 3) hipLaunchKernelGGL(tiny_kernel, dim3(1), dim3(64), 0, stream, ctr, ctr + 2048);
     }
     return hipGetLastError();
 }

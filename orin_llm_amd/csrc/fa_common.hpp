@@ -35,7 +35,7 @@ struct FaArgs {
     const uint16_t* vc;
     float* out;
     float* part_o;    // decode: [split][n_head][D]
-    float* part_ml;   // decode: [split][n_head][2] = (reference maximum in log2 units, row sum)
+    float* part_ml;   // decode: [n_head][split][2] = (reference maximum in log2 units, row sum)
     const int* d_pos; // decode only
     const float* k_new; // decode with store: the current token's K and V rows, fp32 [n_kv][head_dim];
     const float* v_new; // null for plain decode (the cache pointers are then never written through)

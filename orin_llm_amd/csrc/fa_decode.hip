@@ -179,9 +179,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         // without reading the position itself (one more trip to memory on its short critical path);
         // the partial outputs are left as they are and get weight zero.
         if (threadIdx.x < 16 && hg * 16 + (int)threadIdx.x < r) {
-            const size_t pi = (size_t)id * a.n_head + kvh * r + hg * 16 + threadIdx.x;
-            a.part_ml[pi * 2 + 0] = -INFINITY;
-            a.part_ml[pi * 2 + 1] = 0.0f;
+            const size_t mi = (size_t)(kvh * r + hg * 16 + threadIdx.x) * n_splits + id; // [head][split]
+            a.part_ml[mi * 2 + 0] = -INFINITY;
+            a.part_ml[mi * 2 + 1] = 0.0f;
         }
         return;
     }
@@ -468,8 +468,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
             const size_t pi = (size_t)id * a.n_head + head;
             *reinterpret_cast<f4*>(a.part_o + pi * D + d4) = acc;
             if (d4 == 0) {
-                a.part_ml[pi * 2 + 0] = m_all;
-                a.part_ml[pi * 2 + 1] = l_all;
+                const size_t mi = (size_t)head * n_splits + id; // [head][split]: a head's pairs are one run of memory for the combine kernel
+                a.part_ml[mi * 2 + 0] = m_all;
+                a.part_ml[mi * 2 + 1] = l_all;
             }
         } else {
             const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
@@ -479,75 +480,103 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     FA_STAMP(7);
 }
 
-// Log-sum-exp merge of the decode splits.  One workgroup per (query head, 32-wide slice of
-// head_dim); 8 lane-groups of 32 take the splits round-robin.  A thread loads the (m, l) pair
-// and its element of the partial output for each of its splits -- every load issued before
-// anything is waited on, and nothing else is read (not even the position: splits that were
-// inactive for it have said so in their (m, l)) -- merges them on its own, relative to the
-// largest m it has seen, and the 8 groups' results meet in LDS behind the kernel's only
-// barrier.  No cross-lane step: the (m, l) pairs are read redundantly by the 32 threads of a
-// group (one address, one broadcast), which costs less than reductions across lanes would on a
-// kernel that is little more than one trip to memory.  Partial outputs of inactive splits hold
-// stale data and are never multiplied.
-// PER: splits per thread (n_splits <= 8 * PER; the launcher picks the smallest that fits).
-template <int D, int PER>
-__global__ __launch_bounds__(256) void fa_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                                 float* __restrict__ out, const int n_splits, const int n_head) {
-    constexpr int kSlices = D / 32;
-    constexpr int kGroups = 8;
-    constexpr int kPer = PER;
-    static_assert(kGroups * PER <= kMaxSplits, "more slots than splits can be");
-    __shared__ float sh_acc[kGroups][32];
-    __shared__ float sh_m[kGroups], sh_l[kGroups];
-    const int head = blockIdx.x / kSlices;
-    const int dl = threadIdx.x & 31;
-    const int d = (blockIdx.x % kSlices) * 32 + dl;
-    const int sg = threadIdx.x >> 5;
+// Log-sum-exp merge of the decode splits.  One workgroup of 8 waves per (query head, 64-wide
+// slice of head_dim); wave w takes the partial outputs of splits w, w + 8, ...; lane = element
+// of the slice.  The kernel is little more than a trip to memory, so everything is shaped to
+// make that one trip and little else:
+//   * a head's (m, l) pairs are one run of memory ([head][split]): every wave fetches all of them
+//     with one coalesced load per 64 splits (lane = split) and finds the overall maximum and the
+//     overall row sum itself, with lane-swap reductions, while its partial outputs are still on
+//     their way -- so no wave waits for another's statistics, and the weights of a wave's own
+//     splits are lane reads;
+//   * a wave's split indices are uniform, so the address arithmetic of the partial outputs
+//     stays in the scalar unit and every load is one coalesced 256 bytes (per-thread 64-bit
+//     address arithmetic for every load cost more than the trip);
+//   * every load is issued before anything is waited on, and nothing else is read (not even the
+//     position: splits that were inactive for it have said so in their (m, l)).
+// The 8 waves' weighted sums meet in LDS behind the kernel's only barrier.  Partial outputs of
+// inactive splits hold stale data and are never multiplied.
+// PER: splits per wave (n_splits <= 8 * PER; the launcher picks the smallest that fits).
+__device__ __forceinline__ float dpp_xor_step(float v, int which) {
+    // lane i <-> the lane whose index differs within its row of 16: 1, 2 (quad permutes), 7 - i within 8, 15 - i within 16
+    const int x = __float_as_int(v);
+    int y;
+    if (which == 0) y = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);       // quad_perm [1,0,3,2]
+    else if (which == 1) y = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    else if (which == 2) y = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false); // row_half_mirror
+    else y = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false);                 // row_mirror
+    return __int_as_float(y);
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v = fmaxf(v, dpp_xor_step(v, i));
+    return xor_max(v); // across the four rows of 16
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v += dpp_xor_step(v, i);
+    return xor_sum(v);
+}
 
-    float2 ml[kPer];
-    float x[kPer];
-    const float* po = part_o + (size_t)head * D + d;
-    const float* pm = part_ml + (size_t)head * 2;
-    const size_t stride = (size_t)n_head * D, stride_ml = (size_t)n_head * 2;
+template <int D, int PER>
+__global__ __launch_bounds__(512) void fa_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                                 float* __restrict__ out, const int n_splits, const int n_head) {
+    constexpr int kSlices = D / 64;
+    constexpr int kGroups = 8;
+    constexpr int kRounds = (kGroups * PER + 63) / 64; // (m, l) pairs per lane
+    static_assert(kGroups * PER <= kMaxSplits, "more slots than splits can be");
+    __shared__ float sh_acc[kGroups][64];
+    const int head = blockIdx.x / kSlices;
+    const int lane = threadIdx.x & 63;
+    const int d = (blockIdx.x % kSlices) * 64 + lane;
+    const int sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // (slots past n_splits read split 0 again and are voided below: a load under a branch
+    // would make the compiler wait for the loads before it where the branch ends)
+    float2 ml[kRounds];
+    const float* const pm = part_ml + (size_t)head * n_splits * 2;
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        // (slots past n_splits read split 0 again and are voided below: a load under a branch
-        // would make the compiler wait for the loads before it where the branch ends)
-        const int s = sg + j * kGroups, sc = s < n_splits ? s : 0;
-        ml[j] = *reinterpret_cast<const float2*>(pm + sc * stride_ml);
-        x[j] = po[sc * stride];
+    for (int rd = 0; rd < kRounds; ++rd) {
+        const int s = lane + 64 * rd;
+        ml[rd] = *reinterpret_cast<const float2*>(pm + (s < n_splits ? s : 0) * 2);
     }
+    float x[PER];
+    const int stride = n_head * D; // (a split's partial outputs; the whole array is below 2^31 bytes)
+    const float* const po = part_o + head * D + d;
 #pragma unroll
-    for (int j = 0; j < kPer; ++j)
-        if (sg + j * kGroups >= n_splits) ml[j] = float2{-INFINITY, 0.0f};
-    float m_loc = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) m_loc = fmaxf(m_loc, ml[j].x);
-    float l_loc = 0.0f, acc = 0.0f;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        const float w = ml[j].x > -INFINITY ? fast_exp2(ml[j].x - m_loc) : 0.0f;
-        l_loc = __builtin_fmaf(ml[j].y, w, l_loc);
-        if (w > 0.0f) acc = __builtin_fmaf(x[j], w, acc); // (what a weightless split left behind may be anything)
+    for (int j = 0; j < PER; ++j) {
+        const int s = sg + j * kGroups;
+        x[j] = po[(s < n_splits ? s : 0) * stride];
     }
-    sh_acc[sg][dl] = acc;
-    if (dl == 0) {
-        sh_m[sg] = m_loc;
-        sh_l[sg] = l_loc;
+    // ---- the head's statistics, in every wave, while the partial outputs travel ----
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int rd = 0; rd < kRounds; ++rd) {
+        if (lane + 64 * rd >= n_splits) ml[rd] = float2{-INFINITY, 0.0f};
+        m_all = fmaxf(m_all, ml[rd].x);
     }
+    m_all = wave_max(m_all);
+    float w[kRounds], l_all = 0.0f;
+#pragma unroll
+    for (int rd = 0; rd < kRounds; ++rd) {
+        w[rd] = ml[rd].x > -INFINITY ? fast_exp2(ml[rd].x - m_all) : 0.0f; // (no split active at all: every weight 0)
+        l_all = __builtin_fmaf(ml[rd].y, w[rd], l_all);
+    }
+    l_all = wave_sum(l_all);
+    // ---- this wave's splits: split sg + 8j sits in lane (8j mod 64) + sg of round 8j / 64 ----
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const float wj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w[(j * kGroups) / 64]), ((j * kGroups) % 64) + sg));
+        if (wj > 0.0f) acc = __builtin_fmaf(x[j], wj, acc); // (what a weightless split left behind may be anything)
+    }
+    sh_acc[sg][lane] = acc;
     __syncthreads();
     if (sg == 0) {
-        float m_all = -INFINITY;
+        float tot = 0.0f;
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) m_all = fmaxf(m_all, sh_m[g]);
-        float tot = 0.0f, l_all = 0.0f;
-#pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-            const float w = sh_m[g] > -INFINITY ? fast_exp2(sh_m[g] - m_all) : 0.0f;
-            l_all = __builtin_fmaf(sh_l[g], w, l_all);
-            tot = __builtin_fmaf(sh_acc[g][dl], w, tot);
-        }
-        out[(size_t)head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
+        for (int g = 0; g < kGroups; ++g) tot += sh_acc[g][lane];
+        out[head * D + d] = l_all > 0.0f ? tot / l_all : 0.0f;
     }
 }
 
@@ -564,12 +593,12 @@ hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
     if (e != hipSuccess || a.n_splits == 1) return e;
-    const dim3 cgrid(a.n_head * (D / 32));
+    const dim3 cgrid(a.n_head * (D / 64));
 #define ORIN_FA_COMBINE_ARGS a.part_o, a.part_ml, a.out, a.n_splits, a.n_head
-    if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
-    else if (a.n_splits <= 64) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 8>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
-    else if (a.n_splits <= 128) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 16>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
-    else hipLaunchKernelGGL((fa_decode_combine_kernel<D, 32>), cgrid, dim3(256), 0, stream, ORIN_FA_COMBINE_ARGS);
+    if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(512), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else if (a.n_splits <= 64) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 8>), cgrid, dim3(512), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else if (a.n_splits <= 128) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 16>), cgrid, dim3(512), 0, stream, ORIN_FA_COMBINE_ARGS);
+    else hipLaunchKernelGGL((fa_decode_combine_kernel<D, 32>), cgrid, dim3(512), 0, stream, ORIN_FA_COMBINE_ARGS);
 #undef ORIN_FA_COMBINE_ARGS
     return hipGetLastError();
 }

@@ -265,7 +265,7 @@ def bench_tiny_launch():
 def bench_handoff(src, fused, scratch, out):
     """Measurement aid: a stand-in for a split-KV decode step, partial results merged by a second
     kernel (fused=False) or inside the launch (fused=True)."""
-    rc = lib().orin_fa_bench_handoff(_ptr(src), 1 if fused else 0, _ptr(scratch), _ptr(out))
+    rc = lib().orin_fa_bench_handoff(_ptr(src), int(fused), _ptr(scratch), _ptr(out))
     if rc != 0:
         raise OrinFaError("bench_handoff", rc)
 
