@@ -68,9 +68,15 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // query can be requested at once instead of behind a trip to memory for their addresses.
     // (no __restrict__ on these: loads the compiler knows to be invariant are free to sink past
     // the statements below that hold them in place)
+    // Plain decode needs nothing but these 14 words: no trip to the launch's argument block at
+    // all, which is slower than the trip for the position (the caches hold that).  So: the grid
+    // is (KV head, head group, split) and says what n_kv and n_hgroups would; n_splits and r share
+    // a word (splits_r = n_splits | r << 16); the scale carries the sign that goes into Q
+    // (c_signed = |scale| log2(e) with the sign of scale; c2 below is its magnitude); dst is where this kernel writes: the
+    // partial outputs (followed by the (m, l) pairs) when there are splits, else `out` itself.
     const int* d_pos, const float* q, const uint16_t* kc, const uint16_t* vc,
-    const int n_ctx, const int n_splits, const int r, const float qsign, const int n_kv, const int n_hgroups,
-    const FaArgs a) {
+    const int n_ctx, const unsigned splits_r, const float c_signed, float* dst, const int n_head,
+    const FaArgs a) { // (a: what the store and rotate variants need besides)
     using G = DGeom<D>;
     constexpr int kWaves = kDecodeWaves;
     constexpr int kThreads = kWaves * 64;
@@ -82,12 +88,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     const int col = lane & 15; // MFMA column (query head of the group) / row (KV row or head_dim index) of the lane
     const int grp = lane >> 4; // lane-group: 8-wide k slice of an operand, 4-row slice of an accumulator
 
-    // Workgroup id -> (KV head, head group, split).  The KV head varies fastest.
-    int id = blockIdx.x;
-    const int kvh = id % n_kv;
-    id /= n_kv;
-    const int hg = id % n_hgroups;
-    id /= n_hgroups; // = split
+    const int n_splits = splits_r & 0xffffu, r = splits_r >> 16;
+    const float c2 = __builtin_fabsf(c_signed), qsign = c_signed < 0.0f ? -1.0f : 1.0f;
+    // Workgroup -> (KV head, head group, split); the KV head varies fastest in dispatch order.
+    const int kvh = blockIdx.x, hg = blockIdx.y, id = blockIdx.z;
+    float* const part_o = dst;
+    float* const part_ml = dst + (size_t)n_splits * n_head * D; // [n_head][split][2]
 
     unsigned char* const vs = smem + wave * G::kWaveB;
     const __amdgpu_buffer_rsrc_t krs = make_rsrc(kc + (size_t)kvh * n_ctx * D, (unsigned)n_ctx * D * 2);
@@ -112,13 +118,18 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     const int pos = *d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
     const int hl = hg * 16 + col;
     const bool valid = hl < r;
-    const float* qp = q + (size_t)(valid ? kvh * r + hl : 0) * D;
+    // Columns past the group's heads are padding: their loads carry an offset past the descriptor's
+    // end, which the hardware answers with zeros without going to memory.  (Every wave of every
+    // workgroup reads its group's heads: fetched for all 16 columns that was as many bytes through
+    // the L2 as the K rows.)
+    const __amdgpu_buffer_rsrc_t qrs = make_rsrc(q, 0x7ffffff0u);
+    const int q_off = valid ? ((kvh * r + hl) * D + grp * 8) * 4 : 0x7ffffff8;
     const float qmul = valid ? qsign : 0.0f;
     float4 qx[2 * G::kSteps];
 #pragma unroll
     for (int kk = 0; kk < G::kSteps; ++kk) {
-        qx[2 * kk] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8);
-        qx[2 * kk + 1] = *reinterpret_cast<const float4*>(qp + kk * 32 + grp * 8 + 4);
+        qx[2 * kk] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, kk * 128, 0));
+        qx[2 * kk + 1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, kk * 128 + 16, 0));
     }
     constexpr bool STORE = MODE != 0, ROPE = MODE == 2;
     // (rotate + store) lane i < n_rot/2 of every wave fetches what pair i's angle needs: its
@@ -144,12 +155,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // 128 KB of cache rows for nothing -- at a short position in a long cache, all of them but a
     // few, tens of megabytes per launch that the active ones then queue behind.
     asm volatile("" ::: "memory");
-    // The arguments that did not arrive in registers are fetched here, in the trip to memory that
-    // brings the position: left alone, the compiler fetches each where it is first used -- the
-    // scale behind the first tile's arrival, the partials' addresses behind the last product.
-    {
-        const void *p0 = a.part_o, *p1 = a.part_ml, *p2 = a.out;
-        asm volatile("" ::"s"(p0), "s"(p1), "s"(p2), "s"(a.c), "s"(a.n_head), "s"(pos));
+    // (store and rotate variants) The arguments that did not arrive in registers are fetched
+    // here, in the trip to memory that brings the position: left alone, the compiler fetches
+    // each where it is first used, behind the first tile's arrival.  (Fetched behind the tile
+    // requests instead, they queue behind the chip's 33 MB of tile traffic: 0.5 us per layer.)
+    if constexpr (MODE != 0) {
+        const void *p0 = a.k_new, *p1 = a.v_new;
+        asm volatile("" ::"s"(p0), "s"(p1), "s"(a.n_rot), "s"(a.neox), "s"(pos));
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -180,8 +192,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         // the partial outputs are left as they are and get weight zero.
         if (threadIdx.x < 16 && hg * 16 + (int)threadIdx.x < r) {
             const size_t mi = (size_t)(kvh * r + hg * 16 + threadIdx.x) * n_splits + id; // [head][split]
-            a.part_ml[mi * 2 + 0] = -INFINITY;
-            a.part_ml[mi * 2 + 1] = 0.0f;
+            part_ml[mi * 2 + 0] = -INFINITY;
+            part_ml[mi * 2 + 1] = 0.0f;
         }
         return;
     }
@@ -382,20 +394,20 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         mx = fmaxf(fmaxf(mx, v[5]), v[6]);
         mx = xor_max(fmaxf(mx, v[7]));
         // move the reference only when this tile's maximum is far above it (or it is unset)
-        const bool move = (mx - m_ref) * a.c > kLazy || (m_ref == -INFINITY && mx > -INFINITY);
+        const bool move = (mx - m_ref) * c2 > kLazy || (m_ref == -INFINITY && mx > -INFINITY);
         if (__builtin_amdgcn_ballot_w64(move) != 0) {
-            const float alpha = move ? fast_exp2((m_ref - mx) * a.c) : 1.0f; // unset reference -> 0
+            const float alpha = move ? fast_exp2((m_ref - mx) * c2) : 1.0f; // unset reference -> 0
             if (move) m_ref = mx;
             l_run *= alpha;
 #pragma unroll
             for (int db = 0; db < G::kDBlk; ++db) o[db] *= alpha;
         }
-        // exponent = s*c - m_ref*c + shift; a column that has seen no visible row keeps weight 0
-        const float nb = (m_ref == -INFINITY) ? kPShift : kPShift - m_ref * a.c;
+        // exponent = s*c2 - m_ref*c2 + shift; a column that has seen no visible row keeps weight 0
+        const float nb = (m_ref == -INFINITY) ? kPShift : kPShift - m_ref * c2;
         h8 ph, pl;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float pe = fast_exp2(__builtin_fmaf(v[e], a.c, nb));
+            const float pe = fast_exp2(__builtin_fmaf(v[e], c2, nb));
             l_run += pe;
             ph[e] = (_Float16)pe;
             pl[e] = (_Float16)(pe - (float)ph[e]);
@@ -432,7 +444,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     float* const obuf = reinterpret_cast<float*>(smem + wave * G::kWaveB);
     const float l_tot = xor_sum(l_run);
     if (grp == 0) {
-        ml[(wave * 16 + col) * 2 + 0] = (m_ref == -INFINITY) ? -INFINITY : m_ref * a.c; // log2 units
+        ml[(wave * 16 + col) * 2 + 0] = (m_ref == -INFINITY) ? -INFINITY : m_ref * c2; // log2 units
         ml[(wave * 16 + col) * 2 + 1] = l_tot;
     }
 #pragma unroll
@@ -465,16 +477,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         }
         const int head = kvh * r + h_local;
         if (n_splits > 1) {
-            const size_t pi = (size_t)id * a.n_head + head;
-            *reinterpret_cast<f4*>(a.part_o + pi * D + d4) = acc;
+            const size_t pi = (size_t)id * n_head + head;
+            *reinterpret_cast<f4*>(part_o + pi * D + d4) = acc;
             if (d4 == 0) {
                 const size_t mi = (size_t)head * n_splits + id; // [head][split]: a head's pairs are one run of memory for the combine kernel
-                a.part_ml[mi * 2 + 0] = m_all;
-                a.part_ml[mi * 2 + 1] = l_all;
+                part_ml[mi * 2 + 0] = m_all;
+                part_ml[mi * 2 + 1] = l_all;
             }
         } else {
             const float inv = l_all > 0.0f ? 1.0f / l_all : 0.0f;
-            *reinterpret_cast<f4*>(a.out + (size_t)head * D + d4) = acc * inv;
+            *reinterpret_cast<f4*>(dst + (size_t)head * D + d4) = acc * inv; // (no splits: dst is the output)
         }
     }
     FA_STAMP(7);
@@ -582,10 +594,12 @@ __global__ __launch_bounds__(512) void fa_decode_combine_kernel(const float* __r
 
 template <int D>
 hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
-    const int grid = a.n_kv * a.n_hgroups * a.n_splits;
+    if (a.n_splits > 0xffff || a.r > 0xffff || a.n_hgroups > 0xffff) return hipErrorInvalidValue;
     constexpr int lds = DGeom<D>::kLdsB;
-    const dim3 g(grid), b(kDecodeWaves * 64);
-#define ORIN_FA_SPLIT_ARGS a.d_pos, a.q, a.kc, a.vc, a.n_ctx, a.n_splits, a.r, a.qsign, a.n_kv, a.n_hgroups, a
+    const dim3 g(a.n_kv, a.n_hgroups, a.n_splits), b(kDecodeWaves * 64);
+    const unsigned splits_r = (unsigned)a.n_splits | (unsigned)a.r << 16;
+    float* const dst = a.n_splits > 1 ? a.part_o : a.out;
+#define ORIN_FA_SPLIT_ARGS a.d_pos, a.q, a.kc, a.vc, a.n_ctx, splits_r, a.c * a.qsign, dst, a.n_head, a
     if (a.k_new && a.n_rot > 0) hipLaunchKernelGGL((fa_decode_split_kernel<D, 2>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
     else if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, 1>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
     else hipLaunchKernelGGL((fa_decode_split_kernel<D, 0>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
