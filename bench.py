@@ -6,12 +6,12 @@
 Prints ONE JSON line.  A "step" is one pass of the attention operator over a whole layer
 stack of synthetic inputs already resident in HBM (independent seeds and buffers per layer):
 
-  qwen1.5b-prefill512   (default; BASELINE configs[1]) 28 layers x two 512-token causal chunks,
+  qwen1.5b-prefill512   (default; the configuration the headline metric is quoted on) 28 layers x two 512-token causal chunks,
                         at cache depth 0 and 3584, 12 Q heads / 2 KV heads, d=128, K with 4
                         outlier channels x8.  value = causal-exact TFLOP/s (step launched eagerly and as
                         one HIP graph; the faster counts, both are reported).
   llama8b-prefill512-d4096, qwen7b-prefill512-d32256, qwen1.5b-decode-32k, llama8b-decode-8k,
-  qwen7b-decode-32k     the other BASELINE shapes; the north-star cases are also run after the
+  qwen7b-decode-32k     the other benchmark shapes; the target cases are also run after the
                         default workload and reported under "also".
 
 FLOPs per prefill launch (causal-exact): 4*d*H*(B*P + B*(B+1)/2).  Bytes per decode launch:

@@ -277,7 +277,7 @@ def test_decode_graph_capture_replay(fa):
             check(outs[l].cpu().numpy(), want, f"graph replay pos {pos} layer {l}", floor=FLOOR_DECODE)
 
 
-# ---------------------------------------------------------------- BASELINE configs at full size (row-sampled oracle)
+# ---------------------------------------------------------------- the benchmark configurations at full size (row-sampled oracle)
 
 def _sample_rows(rng, batch, H, r, extra_tokens=()):
     toks = {0, 1, 7, 8, 15, 16, 31, 32, 255, 256, batch - 2, batch - 1, *extra_tokens}
