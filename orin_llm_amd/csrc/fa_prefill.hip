@@ -79,7 +79,15 @@ struct PGeom {
     }
     static constexpr int kKOff = 0;                   // wave slice: K buffers 0/1, then V buffers 0/1
     static constexpr int kVOff = 2 * kTileB;
-    static constexpr int kOStride = D + 4;
+    // Merge buffer: a column's partial output is one unpadded row of D floats whose 16-byte pieces
+    // are permuted, piece p of column c sitting at p ^ o_swz(c).  LDS serves a 16-byte access 16
+    // lanes at a time, and those 16 lanes must fall on 16 different piece columns of the 64 banks:
+    // the writers are 16 neighbouring columns at one piece (so the 4-bit pattern must differ over
+    // any 16 neighbouring columns), the readers are 4 neighbouring columns x 4 neighbouring pieces
+    // or 2 x 8 (so the columns' low bits must land in the pattern's high bits): reverse the bits.
+    // (Padded rows of D + 4 floats served the writers and left the readers four to a bank.)
+    static constexpr int kOStride = D;
+    __device__ static int o_swz(int c) { return ((c & 1) << 3) | ((c & 2) << 1) | ((c & 4) >> 1) | ((c & 8) >> 3); }
     static constexpr int kMergeB = kCols * kOStride * 4;
     static constexpr int kWaveB = (4 * kTileB > kMergeB) ? 4 * kTileB : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
@@ -470,6 +478,37 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
     };
     constexpr int kC = G::kCopies;
 
+    // ---- the wave's hand-over to the merge of the four waves through LDS ----
+    // (m, l) per wave and column, m = the reference in log2 units (the common shift cancels);
+    // a wave that saw no visible row of a column has l = 0 and is given m = -inf (weight 0).
+    float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
+    auto write_ml = [&]() {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            const float l_tot = pair_sum(lsum[cb][0] + lsum[cb][1]);
+            if (hh == 0) {
+                ml[(wave * G::kCols + cb * 32 + c32) * 2 + 0] = l_tot > 0.0f ? -nb[cb] : -INFINITY;
+                ml[(wave * G::kCols + cb * 32 + c32) * 2 + 1] = l_tot;
+            }
+        }
+    };
+    // O^T -> [column][head_dim] fp32: accumulator registers 4q..4q+3 of lane (c32, hh) are
+    // head_dim indices db*32 + 8q + 4*hh + 0..3 of column cb*32 + c32, i.e. the 16-byte piece
+    // db*8 + 2*q + hh of the column's row, of which only the low four bits are permuted.
+    // Accumulator a = cb * kDBlk + db; half h of it is its pieces q = 2h and 2h + 1.
+    constexpr int kAccs = NCB * G::kDBlk;
+    const int o_e = hh ^ G::o_swz(c32); // (column cb*32 + c32 has the low bits of c32)
+    auto write_o_half = [&](auto ac, auto hc, auto pinc) {
+        constexpr int acc = decltype(ac)::value, half = decltype(hc)::value;
+        constexpr int cb = acc / G::kDBlk, db = acc % G::kDBlk;
+        if constexpr (decltype(pinc)::value) pin_a(o[cb][db]); // (its reads stay behind this point of the instruction stream)
+        float* const row = reinterpret_cast<float*>(ws) + (cb * 32 + c32) * G::kOStride + (db >> 1) * 64;
+#pragma unroll
+        for (int qd = 2 * half; qd < 2 * half + 2; ++qd)
+            *reinterpret_cast<f4*>(row + ((((db & 1) * 8 + 2 * qd) ^ o_e) << 2)) =
+                f4{o[cb][db][4 * qd], o[cb][db][4 * qd + 1], o[cb][db][4 * qd + 2], o[cb][db][4 * qd + 3]};
+    };
+
     if (n_mine > 0) {
         const int R = n_mine - 1; // steps after step 0
         // Prologue form of A: S[spar] = K[kpar] Q^T with a zero addend, operands read up front.
@@ -492,54 +531,93 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         wait_copies(IntC<2 * kC>{});        // K0 landed (V0 K1 may be in flight)
         stage_a0(IntC<0>{}, IntC<0>{});     // S(0)
         __builtin_amdgcn_s_waitcnt(0xC07F); // its LDS reads have returned: K buffer 0 is free
+        wait_copies(IntC<0>{});             // K1 and V0 landed
+        // S(1), the scan of S(0) for each column's maximum and the copies of K(2) run as one
+        // stream: a matrix instruction, a share of the scan, a copy.  (Sixteen copies issued in
+        // one burst hold the wave for as long as the load unit takes to accept them, half a
+        // microsecond with four waves at it; one at a time between other work they cost nothing.
+        // When the wave has no tile 1 the products are of whatever K buffer 1 holds, and nobody
+        // reads them.)
+        const int ksoff0 = tile_soff(tile_of(2)), vsoff0 = tile_soff(tile_of(1));
+        float v0s[NCB][16];
+        float mxp[NCB][4];
         {
-            const int ksoff = tile_soff(tile_of(2));
-            static_for<0, kC>([&](auto ic) { copy_one(ic, kdesc, k_buf(0), ksoff); });
-            copy_checked(vdesc, v_buf(1), tile_of(1));
-        }
-        wait_copies(IntC<2 * kC>{});        // K1 and V0 landed (K2 V1 may be in flight)
-        if (R > 0) stage_a0(IntC<1>{}, IntC<1>{}); // S(1)
-        settle();
-        FA_STAMP(2);
-        // Reference maximum of each column: over its visible scores of tile 0 and, when there is
-        // one, tile 1 (every row of which is visible to every column).  A column with no visible
-        // row in this wave keeps weight zero whatever the reference.
-        {
+            h8 ka[G::kSteps];
+#pragma unroll
+            for (int ks = 0; ks < G::kSteps; ++ks) ka[ks] = *reinterpret_cast<const h8*>(kp[ks] + G::kTileB);
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            settle(); // S(0) is out of the matrix pipe
             const int row0 = tile_of(0) * kTile + 4 * hh;
             const bool masked = tile_of(0) * kTile + kTile > full_end;
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 pin_v(s[0][cb]); // (the reads below stay behind the settled pipe)
-                if (R > 0) pin_v(s[1][cb]);
-                float v[16];
-                float mxp[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}; // four chains instead of one long one
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    v[r] = s[0][cb][r];
-                    if (masked && row0 + 8 * (r / 4) + (r % 4) >= limit[cb]) v[r] = -INFINITY;
-                    mxp[r % 4] = fmaxf(mxp[r % 4], v[r]);
-                }
-                if (R > 0) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) mxp[r % 4] = fmaxf(mxp[r % 4], s[1][cb][r]);
-                }
-                const float mx = pair_max(fmaxf(fmaxf(mxp[0], mxp[1]), fmaxf(mxp[2], mxp[3])));
-                nb[cb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
-                float sump[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int kh = 0; kh < 2; ++kh) {
-                    h8 ph;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        ph[j] = (_Float16)fast_exp2(__builtin_fmaf(v[kh * 8 + j], a.c, nb[cb]));
-                        sump[j % 4] += (float)ph[j];
-                    }
-                    pw[0][cb][kh] = __builtin_bit_cast(u32x4, ph);
-                }
-                const float sum = (sump[0] + sump[1]) + (sump[2] + sump[3]);
-                lsum[cb][0] = sum;
-                lsum[cb][1] = 0.0f;
+                mxp[cb][0] = mxp[cb][1] = mxp[cb][2] = mxp[cb][3] = -INFINITY; // four chains instead of one long one
             }
+            constexpr int kSlots = G::kSteps * NCB;     // one matrix instruction each
+            constexpr int kScan = 16 * NCB / kSlots;    // scores scanned per slot
+            static_assert(kScan * kSlots == 16 * NCB && kC % (kSlots / NCB) == 0, "shares");
+            static_for<0, kSlots>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                constexpr int ks = i / NCB, m = i % NCB;
+                if constexpr (ks == 0) mfma_s_zero_n(s[1][m], ka[ks], q[m][ks]);
+                else mfma_s_n(s[1][m], ka[ks], q[m][ks]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < kScan; ++u) {
+                    constexpr int cb = (i * kScan) / 16;
+                    const int r = (i * kScan) % 16 + u;
+                    float x = s[0][cb][r];
+                    if (masked && row0 + 8 * (r / 4) + (r % 4) >= limit[cb]) x = -INFINITY;
+                    v0s[cb][r] = x;
+                    mxp[cb][r % 4] = fmaxf(mxp[cb][r % 4], x);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (m == NCB - 1) {
+                    constexpr int per = kC / G::kSteps; // copies per k-step
+                    static_for<0, per>([&](auto jc) { copy_one(IntC<ks * per + decltype(jc)::value>{}, kdesc, k_buf(0), ksoff0); });
+                }
+            });
+        }
+        settle();
+        FA_STAMP(2);
+        // Reference maximum of each column: over its visible scores of tile 0 and, when there is
+        // one, tile 1 (every row of which is visible to every column).  A column with no visible
+        // row in this wave keeps weight zero whatever the reference.  The copies of V(1) go out
+        // between the pieces of this.
+        {
+            constexpr int kPieces = 2 * NCB;
+            static_assert(kC % kPieces == 0, "copies per piece");
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                if (R > 0) {
+                    pin_v(s[1][cb]);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mxp[cb][r % 4] = fmaxf(mxp[cb][r % 4], s[1][cb][r]);
+                }
+                const float mx = pair_max(fmaxf(fmaxf(mxp[cb][0], mxp[cb][1]), fmaxf(mxp[cb][2], mxp[cb][3])));
+                nb[cb] = kPShift - (mx == -INFINITY ? 0.0f : mx) * a.c;
+            }
+            static_for<0, kPieces>([&](auto pc) {
+                constexpr int piece = decltype(pc)::value, cb = piece / 2, kh = piece % 2;
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, kC / kPieces>([&](auto jc) {
+                    copy_one(IntC<piece * (kC / kPieces) + decltype(jc)::value>{}, vdesc, v_buf(1), vsoff0);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                float sump[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                h8 ph;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    ph[j] = (_Float16)fast_exp2(__builtin_fmaf(v0s[cb][kh * 8 + j], a.c, nb[cb]));
+                    sump[j % 4] += (float)ph[j];
+                }
+                pw[0][cb][kh] = __builtin_bit_cast(u32x4, ph);
+                const float sum = (sump[0] + sump[1]) + (sump[2] + sump[3]);
+                if constexpr (kh == 0) lsum[cb][0] = sum;
+                else lsum[cb][0] += sum;
+                lsum[cb][1] = 0.0f;
+            });
         }
         settle(); // (the vector writes of P are well clear of the next matrix instruction)
         FA_STAMP(3);
@@ -727,12 +805,13 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         }
         if (t == R) body(IntC<0>{}, t);
         FA_STAMP(4);
-        // ---- drain: C(R) ----
+        // ---- drain: C(R), and the accumulators on their way to the merge ----
         // V(R) has landed once the two tiles of copies issued after it are all that is outstanding
         // (those, for steps past the last, land in buffers nobody reads; their latency hides
         // behind the matrix instructions below).
         wait_copies(IntC<2 * kC>{});
         settle(); // P(R) was converted just above
+        write_ml();
         {   // O += V(R)^T P(R); both live in the buffers of parity R & 1
             const bool odd = (R & 1) != 0;
             const int v_par = odd ? G::kTileB : 0;
@@ -756,41 +835,43 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
                 pl[cb][0] = __builtin_bit_cast(h8, pw[0][cb][0]);
                 pl[cb][1] = __builtin_bit_cast(h8, pw[0][cb][1]);
             }
-#pragma unroll
-            for (int j = 0; j < 2 * G::kDBlk; ++j)
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) mfma_o_n(o[cb][j % G::kDBlk], va[j], pl[cb][j / G::kDBlk]);
+            // The accumulators are finished two at a time (their two products each alternating,
+            // so that no product follows straight on the one it adds to), and a finished pair
+            // goes to the merge buffer between the products of the next pair: one 32-byte share
+            // per matrix instruction, read two or more matrix instructions after the last one
+            // that wrote it.  Only the last pair's way to LDS is not covered.
+            static_for<0, kAccs / 2>([&](auto pc) {
+                constexpr int p = decltype(pc)::value;
+                if constexpr (p == 1) // the merge buffer takes the tile buffers' place: every read of those has
+                    __builtin_amdgcn_s_waitcnt(0x0070); // returned and every copy into them has landed
+                static_for<0, 4>([&](auto sc) {
+                    constexpr int sl = decltype(sc)::value, acc = 2 * p + sl % 2, kh = sl / 2;
+                    constexpr int cb = acc / G::kDBlk, db = acc % G::kDBlk;
+                    mfma_o_n(o[cb][db], va[kh * G::kDBlk + db], pl[cb][kh]);
+                    if constexpr (p > 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        write_o_half(IntC<2 * (p - 1) + sl / 2>{}, IntC<sl % 2>{}, IntC<1>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                });
+            });
+            if constexpr (kAccs == 2) __builtin_amdgcn_s_waitcnt(0x0070);
         }
-        __builtin_amdgcn_s_waitcnt(0x0070); // every read of the tile buffers has returned and every copy into them has landed: the merge reuses them
+        settle(); // O is out of the matrix pipe
+        static_for<kAccs - 2, kAccs>([&](auto ac) {
+            write_o_half(ac, IntC<0>{}, IntC<1>{});
+            write_o_half(ac, IntC<1>{}, IntC<1>{});
+        });
+    } else {
+        // no tile for this wave: its share of the merge is zero, with weight zero
+        settle(); // (the matrix instructions that cleared O are long done; said once more for the reads below)
+        write_ml();
+        static_for<0, kAccs>([&](auto ac) { // (behind settle(): LDS writes do not move across it)
+            write_o_half(ac, IntC<0>{}, IntC<0>{});
+            write_o_half(ac, IntC<1>{}, IntC<0>{});
+        });
     }
-    settle(); // O is out of the matrix pipe
-    wave_lds_sync();
     FA_STAMP(5);
-
-    // ---- merge the four waves through LDS ----
-    // (m, l) per wave and column, m = the reference in log2 units (the common shift cancels);
-    // a wave that saw no visible row of a column has l = 0 and is given m = -inf (weight 0).
-    float* const ml = reinterpret_cast<float*>(smem + G::kMlOff);
-#pragma unroll
-    for (int cb = 0; cb < NCB; ++cb) {
-        const float l_tot = pair_sum(lsum[cb][0] + lsum[cb][1]);
-        if (hh == 0) {
-            ml[(wave * G::kCols + cb * 32 + c32) * 2 + 0] = l_tot > 0.0f ? -nb[cb] : -INFINITY;
-            ml[(wave * G::kCols + cb * 32 + c32) * 2 + 1] = l_tot;
-        }
-    }
-    // O^T -> [column][head_dim] fp32: accumulator registers 4q..4q+3 of lane (c32, hh) are
-    // head_dim indices db*32 + 8q + 4*hh + 0..3 of column cb*32 + c32.
-#pragma unroll
-    for (int cb = 0; cb < NCB; ++cb)
-#pragma unroll
-        for (int db = 0; db < G::kDBlk; ++db) {
-            pin_a(o[cb][db]); // (read behind the settled pipe)
-            float* const dst = reinterpret_cast<float*>(ws) + (cb * 32 + c32) * G::kOStride + db * 32 + 4 * hh;
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd)
-                *reinterpret_cast<f4*>(dst + 8 * qd) = f4{o[cb][db][4 * qd], o[cb][db][4 * qd + 1], o[cb][db][4 * qd + 2], o[cb][db][4 * qd + 3]};
-        }
     FA_STAMP(6);
     __syncthreads();
     FA_STAMP(7);
@@ -811,13 +892,14 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             lw[w] = ml[(w * G::kCols + cm) * 2 + 1];
         }
         constexpr int kHalfJ = D / (8 * kParts); // 16-byte pieces per thread and half
+        const int o_sw = G::o_swz(cm);           // where the writers put this column's pieces
         f4 x[kHalfJ][kWaves];
         auto load_half = [&](int j0) {
 #pragma unroll
             for (int j = 0; j < kHalfJ; ++j)
 #pragma unroll
                 for (int w = 0; w < kWaves; ++w)
-                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((j0 + j) * kParts + part) * 4) * 4);
+                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((((j0 + j) * kParts + part) ^ o_sw) << 2)) * 4);
         };
         load_half(0);
         __builtin_amdgcn_sched_barrier(0);
