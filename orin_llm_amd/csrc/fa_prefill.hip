@@ -79,15 +79,24 @@ struct PGeom {
     }
     static constexpr int kKOff = 0;                   // wave slice: K buffers 0/1, then V buffers 0/1
     static constexpr int kVOff = 2 * kTileB;
-    // Merge buffer: a column's partial output is one unpadded row of D floats whose 16-byte pieces
-    // are permuted, piece p of column c sitting at p ^ o_swz(c).  LDS serves a 16-byte access 16
-    // lanes at a time, and those 16 lanes must fall on 16 different piece columns of the 64 banks:
-    // the writers are 16 neighbouring columns at one piece (so the 4-bit pattern must differ over
-    // any 16 neighbouring columns), the readers are 4 neighbouring columns x 4 neighbouring pieces
-    // or 2 x 8 (so the columns' low bits must land in the pattern's high bits): reverse the bits.
-    // (Padded rows of D + 4 floats served the writers and left the readers four to a bank.)
-    static constexpr int kOStride = D;
-    __device__ static int o_swz(int c) { return ((c & 1) << 3) | ((c & 2) << 1) | ((c & 4) >> 1) | ((c & 8) >> 3); }
+    // Merge buffer of a wave: the 16-byte pieces of its partial outputs, one 1 KB block per store
+    // instruction of the hand-over.  Piece P = db*8 + 2*q + hh of column cb*32 + c32 (accumulator
+    // registers 4q..4q+3 of block db in lane (c32, hh)) is chunk o_chunk(c32, hh, q) of block
+    // (cb * kDBlk + db) * 4 + q.  A store instruction thus fills its own block with one chunk per
+    // lane, in lane order up to an exchange of whole groups of lanes -- the form LDS takes at its
+    // full write rate (53 counter ticks per instruction and wave with four waves storing, measured;
+    // column-major rows, padded or permuted, take 53-64).  The exchange is there for the readers:
+    // sixteen neighbouring threads of the merge, (4 columns) x (pieces hh, q & 1) or (2 columns) x
+    // (hh, q), then fall on sixteen different chunk columns of the banks (19-22 ticks per load;
+    // 48 with padded column-major rows, where they sat four to a bank).
+    __device__ static int o_chunk(int c32, int hh, int q) {
+        return (hh << 5) + (c32 ^ (hh << 3) ^ (NCB == 2 ? (q & 1) << 2 : q << 1));
+    }
+    __device__ static int o_byte(int col, int piece) { // where piece `piece` of column `col` sits in a wave's merge buffer
+        const int hh = piece & 1, q = (piece & 7) >> 1, db = piece >> 3;
+        return (((col >> 5) * kDBlk + db) * 4 + q) * 1024 + o_chunk(col & 31, hh, q) * 16;
+    }
+    static constexpr int kOStride = D; // floats of merge buffer per column
     static constexpr int kMergeB = kCols * kOStride * 4;
     static constexpr int kWaveB = (4 * kTileB > kMergeB) ? 4 * kTileB : kMergeB;
     static constexpr int kMlOff = kPrefillWaves * kWaveB;
@@ -492,20 +501,20 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             }
         }
     };
-    // O^T -> [column][head_dim] fp32: accumulator registers 4q..4q+3 of lane (c32, hh) are
-    // head_dim indices db*32 + 8q + 4*hh + 0..3 of column cb*32 + c32, i.e. the 16-byte piece
-    // db*8 + 2*q + hh of the column's row, of which only the low four bits are permuted.
-    // Accumulator a = cb * kDBlk + db; half h of it is its pieces q = 2h and 2h + 1.
+    // O^T -> merge buffer (layout: PGeom::o_byte).  Accumulator a = cb * kDBlk + db; half h of it is
+    // its pieces q = 2h and 2h + 1.  The block is an immediate offset; the chunk takes one of the
+    // two (NCB = 2) or four per-lane values below.
     constexpr int kAccs = NCB * G::kDBlk;
-    const int o_e = hh ^ G::o_swz(c32); // (column cb*32 + c32 has the low bits of c32)
+    unsigned char* o_lane[4];
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) o_lane[qd] = ws + G::o_chunk(c32, hh, qd) * 16;
     auto write_o_half = [&](auto ac, auto hc, auto pinc) {
         constexpr int acc = decltype(ac)::value, half = decltype(hc)::value;
         constexpr int cb = acc / G::kDBlk, db = acc % G::kDBlk;
         if constexpr (decltype(pinc)::value) pin_a(o[cb][db]); // (its reads stay behind this point of the instruction stream)
-        float* const row = reinterpret_cast<float*>(ws) + (cb * 32 + c32) * G::kOStride + (db >> 1) * 64;
 #pragma unroll
         for (int qd = 2 * half; qd < 2 * half + 2; ++qd)
-            *reinterpret_cast<f4*>(row + ((((db & 1) * 8 + 2 * qd) ^ o_e) << 2)) =
+            *reinterpret_cast<f4*>(o_lane[qd] + ((cb * G::kDBlk + db) * 4 + qd) * 1024) =
                 f4{o[cb][db][4 * qd], o[cb][db][4 * qd + 1], o[cb][db][4 * qd + 2], o[cb][db][4 * qd + 3]};
     };
 
@@ -892,14 +901,13 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             lw[w] = ml[(w * G::kCols + cm) * 2 + 1];
         }
         constexpr int kHalfJ = D / (8 * kParts); // 16-byte pieces per thread and half
-        const int o_sw = G::o_swz(cm);           // where the writers put this column's pieces
         f4 x[kHalfJ][kWaves];
         auto load_half = [&](int j0) {
 #pragma unroll
             for (int j = 0; j < kHalfJ; ++j)
 #pragma unroll
                 for (int w = 0; w < kWaves; ++w)
-                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + ((size_t)cm * G::kOStride + ((((j0 + j) * kParts + part) ^ o_sw) << 2)) * 4);
+                    x[j][w] = *reinterpret_cast<const f4*>(smem + w * G::kWaveB + G::o_byte(cm, (j0 + j) * kParts + part));
         };
         load_half(0);
         __builtin_amdgcn_sched_barrier(0);
