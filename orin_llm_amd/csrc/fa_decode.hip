@@ -46,7 +46,9 @@ struct DGeom {
     static constexpr int kMergeB = 16 * kOStride * 4;
     static constexpr int kWaveB = (kTileBV > kMergeB) ? kTileBV : kMergeB;
     static constexpr int kMlOff = kDecodeWaves * kWaveB;       // (m, l) per wave per column follow the wave slices
-    static constexpr int kLdsB = kMlOff + kDecodeWaves * 16 * 2 * 4;
+    static constexpr int kQOff = kMlOff + kDecodeWaves * 16 * 2 * 4; // the group's query heads, fp32 [16][kQStride]
+    static constexpr int kQStride = D + 4;                     // floats per head (4 of padding: the operand reads of 16 heads miss each other's banks)
+    static constexpr int kLdsB = kQOff + 16 * kQStride * 4;
 };
 
 // MODE 1 (store): the current token's K and V rows arrive as fp32 beside the cache (FaArgs::k_new,
@@ -122,15 +124,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // end, which the hardware answers with zeros without going to memory.  (Every wave of every
     // workgroup reads its group's heads: fetched for all 16 columns that was as many bytes through
     // the L2 as the K rows.)
+    // The workgroup fetches its group's heads once: wave w asks for one 16-byte piece per lane --
+    // piece (w & 1) of k-step (w >> 1) -- and the pieces meet in LDS further down.  (Every wave
+    // fetching all of them itself put 2048 waves x 8 loads on the same few dozen cache lines: 0.4 us
+    // per launch went into the queue for those lines, ahead of the tile loads.)
     const __amdgpu_buffer_rsrc_t qrs = make_rsrc(q, 0x7ffffff0u);
     const int q_off = valid ? ((kvh * r + hl) * D + grp * 8) * 4 : 0x7ffffff8;
     const float qmul = valid ? qsign : 0.0f;
-    float4 qx[2 * G::kSteps];
-#pragma unroll
-    for (int kk = 0; kk < G::kSteps; ++kk) {
-        qx[2 * kk] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, kk * 128, 0));
-        qx[2 * kk + 1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, kk * 128 + 16, 0));
-    }
+    static_assert(kWaves % (2 * G::kSteps) == 0, "a piece per wave (the same piece twice at head_dim 64)");
+    const int q_piece = __builtin_amdgcn_readfirstlane(wave) & (2 * G::kSteps - 1);
+    const float4 q_share = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, (q_piece >> 1) * 128 + (q_piece & 1) * 16, 0));
     constexpr bool STORE = MODE != 0, ROPE = MODE == 2;
     // (rotate + store) lane i < n_rot/2 of every wave fetches what pair i's angle needs: its
     // cosine and sine when the caller supplies them, else its frequency factor if there is one.
@@ -180,7 +183,15 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     const int tile_first = wave < wu ? id * wu + wave : n_tiles; // (n_tiles: none)
     const int tile_step = wu * n_splits;
     int tile = tile_first;
+    float* const qs = reinterpret_cast<float*>(smem + G::kQOff);
     if (id * wu < n_tiles) {
+        // The query pieces meet in LDS: each wave parks the piece it fetched, then a barrier that
+        // waits for LDS only.  Ahead of the tile requests, where the eight waves are still in
+        // step (the position and the pieces arrive together); behind them the waves are microseconds
+        // apart -- the load unit takes a CU's 128 KB of requests as fast as memory answers them --
+        // and a barrier there holds every wave's products until the last has all its requests out.
+        *reinterpret_cast<float4*>(qs + col * G::kQStride + (q_piece >> 1) * 32 + grp * 8 + (q_piece & 1) * 4) = q_share;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         fetch_k(tile);
         fetch_v(tile);
         asm volatile("" ::: "memory"); // (as above: ahead of the conversions that follow, not behind them)
@@ -199,10 +210,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     }
 
     FA_STAMP(1);
+    // (the query pieces met ahead of the tile requests; the operands are picked up while the first tile is on its way)
     float qf[G::kSteps][8]; // this lane's 8 elements of every k-step: head_dim indices kk*32 + grp*8 + 0..7
 #pragma unroll
     for (int kk = 0; kk < G::kSteps; ++kk) {
-        const float4 x0 = qx[2 * kk], x1 = qx[2 * kk + 1];
+        const float4 x0 = *reinterpret_cast<const float4*>(qs + col * G::kQStride + kk * 32 + grp * 8);
+        const float4 x1 = *reinterpret_cast<const float4*>(qs + col * G::kQStride + kk * 32 + grp * 8 + 4);
         qf[kk][0] = x0.x; qf[kk][1] = x0.y; qf[kk][2] = x0.z; qf[kk][3] = x0.w;
         qf[kk][4] = x1.x; qf[kk][5] = x1.y; qf[kk][6] = x1.z; qf[kk][7] = x1.w;
     }
