@@ -126,8 +126,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     // the L2 as the K rows.)
     // The workgroup fetches its group's heads once: wave w asks for one 16-byte piece per lane --
     // piece (w & 1) of k-step (w >> 1) -- and the pieces meet in LDS further down.  (Every wave
-    // fetching all of them itself put 2048 waves x 8 loads on the same few dozen cache lines: 0.4 us
-    // per launch went into the queue for those lines, ahead of the tile loads.)
+    // fetching all of them itself was seven more load instructions a wave whose lanes each count
+    // as a look-up of their own in the vector cache, a quarter again of the kernel's look-ups, all
+    // of them in the queue ahead of the tile requests: 0.4 us per launch.)
     const __amdgpu_buffer_rsrc_t qrs = make_rsrc(q, 0x7ffffff0u);
     const int q_off = valid ? ((kvh * r + hl) * D + grp * 8) * 4 : 0x7ffffff8;
     const float qmul = valid ? qsign : 0.0f;
