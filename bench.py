@@ -75,6 +75,13 @@ WORKLOADS = {
     # partials), its partials merged by a second kernel, as the library does, or inside the launch by a two-level
     # last-arriver reduction over write-through stores and relaxed atomics -- what fusing the combine would cost
     "decode-handoff-mock": (None, "handoff", 0, 32 << 20),
+    # not timed: where a kernel's microseconds go, from the timeline build of the library (the attention kernels'
+    # stage marks store the wall clock there; medians over the waves of one launch, cold inputs)
+    "llama8b-prefill512-d4096-timeline": ("llama8b", "timeline", 8192, ("prefill", 4096, 512)),
+    "qwen1.5b-prefill512-d3584-timeline": ("qwen1.5b", "timeline", 4096, ("prefill", 3584, 512)),
+    "qwen1.5b-prefill512-d0-timeline": ("qwen1.5b", "timeline", 4096, ("prefill", 0, 512)),
+    "qwen1.5b-decode-32k-timeline": ("qwen1.5b", "timeline", 32768, ("decode", 32768, 1)),
+    "qwen7b-decode-32k-timeline": ("qwen7b", "timeline", 32768, ("decode", 32767, 1)),
 }
 # HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
 # WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy: recorded
@@ -93,7 +100,8 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 # Run after the default workload and reported under "also"; the cases the targets are stated on come last, and
 # "targets" at the very end of the line repeats their figures in a few hundred characters.
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
-        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k", "decode-handoff-mock",
+        "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
+        "llama8b-prefill512-d4096-timeline", "qwen1.5b-decode-32k-timeline", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -761,6 +769,84 @@ def run_read(torch, kernels, name, steps, warmup, with_cpu):
                 parity=None)
 
 
+# Stage marks of the kernels (slot, what has happened by then), in the order a wave passes them.
+PREFILL_STAGES = [(0, "entry"), (9, "queries and first K tile requested"), (10, "first V tile and second K tile requested"),
+                  (1, "queries in registers"), (2, "first two score tiles"), (3, "first weights"), (4, "main loop done"),
+                  (5, "last products done, accumulators in LDS"), (7, "barrier passed"), (8, "output stored")]
+DECODE_STAGES = [(0, "entry"), (1, "position known, query pieces met, tile requests issued"), (2, "query converted"),
+                 (3, "K arrived, scores of the last tile done"), (4, "V arrived, last products done"), (5, "partials in LDS"),
+                 (6, "barrier passed"), (7, "partial written")]
+
+
+def run_timeline(torch, kernels, name, steps, warmup, with_cpu):
+    """Not a timed workload: launches the kernel from the timeline build over a few cold layers and reports, for the
+    last launch, when the waves pass each stage mark (microseconds after the first wave's entry: median, earliest,
+    latest).  The stamps cost a little time themselves; durations come from the ordinary library's workloads."""
+    import ctypes
+
+    shape, _, n_ctx, (what, a, batch) = WORKLOADS[name]
+    sh = SHAPES[shape]
+    H, G, d = sh["H"], sh["G"], sh["d"]
+    L = kernels.stamps_lib()
+    rc = L.orin_fa_init(0)
+    assert rc == 0, rc
+    L.orin_fa_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    scale = 1.0 / float(np.sqrt(d))
+    n_layers = 10  # > 256 MB of K/V at every shape: nothing is left in a cache from the launch before
+    n_filled = a + batch if what == "prefill" else a
+    layers = [make_layer(torch, 900 + i, H, G, d, n_ctx, min(n_filled, n_ctx), batch, sh["outliers"]) for i in range(n_layers)]
+    outs = [torch.empty((batch, H, d), dtype=torch.float32, device="cuda") for _ in range(n_layers)]
+    dpos = torch.tensor([a - 1], dtype=torch.int32, device="cuda")
+    waves = 4 if what == "prefill" else 8
+    stages = PREFILL_STAGES if what == "prefill" else DECODE_STAGES
+
+    def launch(i):
+        q, k, v = layers[i]
+        if what == "prefill":
+            rc = L.orin_fa_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(), outs[i].data_ptr(), H, G, d, n_ctx, a, batch, scale)
+        else:
+            rc = L.orin_fa_decode_ind(q.data_ptr(), k.data_ptr(), v.data_ptr(), outs[i].data_ptr(), H, G, d, n_ctx,
+                                      dpos.data_ptr(), scale)
+        assert rc == 0, rc
+
+    rows = []
+    host = np.zeros(1024 * waves * 16, np.int64)
+    for rep in range(1 + max(1, min(steps, 5))):
+        for i in range(n_layers - rep % 3):  # (the last launch of a pass is a different layer from pass to pass)
+            launch(i)
+        torch.cuda.synchronize()
+        rc = L.orin_fa_bench_stamps(0 if what == "prefill" else 1, host.ctypes.data, host.size)
+        assert rc == 0, rc
+        # (the library hands the table over and clears it, so a mark that a wave did not pass reads zero: workgroups
+        # beyond the launch's grid, decode workgroups the position leaves without a tile, prefill waves without one)
+        t = host.reshape(1024, waves, 16)[:, :, [slot for slot, _ in stages]].astype(np.float64) * 0.01  # 100 MHz -> us
+        passed = t > 0
+        passed &= passed[:, :, -1:]       # waves that went all the way
+        t0 = t[:, :, 0][passed[:, :, 0]].min()
+        if rep > 0:                       # (the first pass only clears what earlier launches left)
+            rows.append([(float(np.median(t[:, :, j][passed[:, :, j]] - t0)), float((t[:, :, j][passed[:, :, j]] - t0).min()),
+                          float((t[:, :, j][passed[:, :, j]] - t0).max())) for j in range(len(stages))])
+    med = np.median(np.array(rows), axis=0)
+    timeline = {label: dict(median=round(float(m[0]), 2), earliest=round(float(m[1]), 2), latest=round(float(m[2]), 2))
+                for (_, label), m in zip(stages, med)}
+    span = float(med[-1][2])
+    if what == "prefill":
+        work, peak, unit, bound = prefill_flops(H, d, a, batch), PEAK_FLOPS, "TFLOP/s", "mfma"
+        kern = "fa_prefill_kernel (timeline build)"
+    else:
+        work, peak, unit, bound = decode_bytes(H, G, d, a), PEAK_BYTES, "GB/s", "hbm"
+        kern = "fa_decode_split_kernel (timeline build; the combine kernel follows it)"
+    scale_u = 1e12 if what == "prefill" else 1e9
+    del layers, outs
+    torch.cuda.empty_cache()
+    return dict(value=work / (span * 1e-6) / scale_u, unit=unit, ms_per_step=span * 1e-3,
+                config=dict(workload=name, shape=f"H{H} G{G} d{d}", n_ctx=n_ctx, what=what, depth_or_length=a, batch=batch),
+                roofline=dict(bound=bound, achieved=work / (span * 1e-6) / scale_u, peak=peak / scale_u, unit=unit,
+                              frac=work / (span * 1e-6) / peak, traffic=None, kernel=kern, launch_us=span,
+                              note="launch_us: first wave's entry to last wave's last mark in the timeline build, stamps included"),
+                parity=None, timeline_us=timeline)
+
+
 def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
     """One step = 28 launches of the stand-in over rotating cold buffers; value = the two-launch form's rate."""
     nbytes, scratch_bytes = kernels.bench_handoff_sizes()
@@ -809,7 +895,7 @@ def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
@@ -857,6 +943,7 @@ def main():
                              roofline=r["roofline"], parity=r["parity"],
                              **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {}),
                              **({"into_the_cache": r["into_the_cache"]} if "into_the_cache" in r else {}),
+                             **({"timeline_us": r["timeline_us"]} if "timeline_us" in r else {}),
                              **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})))
         line["also"] = also
         # The figures the targets are stated on, once more and briefly, as the last thing on the line.

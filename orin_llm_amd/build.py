@@ -5,6 +5,10 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "liborin_fa.so")
+# The timeline build: the same sources, the two attention kernels compiled with -DORIN_FA_STAMPS so that their
+# stage marks store the wall clock.  A measurement aid for bench.py's timeline workloads; never the library that is timed.
+STAMPS_LIB = os.path.join(HERE, "liborin_fa_stamps.so")
+STAMPED = ("fa_prefill.hip", "fa_decode.hip")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
            for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
@@ -48,9 +52,13 @@ def build(verbose=False):
     os.makedirs(OBJ_DIR, exist_ok=True)
     objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in SOURCES]
     cmds = [[HIPCC] + FLAGS + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
+    stamped = {s: os.path.join(OBJ_DIR, os.path.basename(s) + ".stamps.o") for s in SOURCES if os.path.basename(s) in STAMPED}
+    cmds += [[HIPCC] + FLAGS + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
     with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
         lines = list(pool.map(_run, cmds))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]))
+    lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [stamped.get(s, o) for s, o in zip(SOURCES, objs)]
+                      + ["-o", STAMPS_LIB]))
     if verbose:
         print("\n".join(lines))
     return LIB

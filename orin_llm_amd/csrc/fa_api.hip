@@ -380,6 +380,12 @@ int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out)
 size_t orin_fa_bench_handoff_scratch_bytes(void) { return kHandoffScratchBytes; }
 size_t orin_fa_bench_handoff_stream_bytes(void) { return kHandoffStreamBytes; }
 
+int orin_fa_bench_stamps(int which, long long* host, size_t n) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!host || n == 0 || (which != 0 && which != 1)) return ORIN_FA_E_INVALID;
+    return hip_code(which == 0 ? prefill_stamps(host, n) : decode_stamps(host, n));
+}
+
 int orin_fa_bench_tiny_launch(void) {
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
     if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;

@@ -88,6 +88,28 @@ hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* 
 // Measurement aids (bench_aids.hip).
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream);
 hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream);
+
+// ---- timeline build (-DORIN_FA_STAMPS, liborin_fa_stamps.so; a measurement aid) ----
+// The attention kernels carry FA_STAMP(i) marks at the ends of their stages.  In the ordinary
+// library they are nothing.  In the timeline build lane 0 of every wave stores the 100 MHz
+// wall clock there, into [workgroup][wave][kStampSlots] of a table that the bench reads back:
+// medians over the waves of one launch say where a kernel's microseconds go.  The stores cost
+// a little time themselves, so this library is never the one that is timed.
+constexpr int kStampWgs = 1024, kStampSlots = 16;
+#ifdef ORIN_FA_STAMPS
+#define ORIN_FA_STAMP_STORE(table, waves, i)                                                                   \
+    do {                                                                                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                                     \
+        const unsigned fa_wg_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);                \
+        if ((threadIdx.x & 63) == 0 && fa_wg_ < (unsigned)orin_fa::kStampWgs)                                  \
+            table[(fa_wg_ * (waves) + (threadIdx.x >> 6)) * orin_fa::kStampSlots + (i)] = wall_clock64();        \
+        __builtin_amdgcn_sched_barrier(0);                                                                     \
+    } while (0)
+#endif
+// Copies a kernel's table to the host (which: 0 prefill, 4 waves a workgroup; 1 decode split, 8 waves);
+// hipErrorNotSupported in the ordinary library.
+hipError_t prefill_stamps(long long* host, size_t n);
+hipError_t decode_stamps(long long* host, size_t n);
 constexpr size_t kHandoffScratchBytes = 1u << 20; // partials of both levels and the arrival counters
 constexpr size_t kHandoffStreamBytes = (size_t)256 * 512 * 16 * 16; // 32 MiB read per launch
 hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out, hipStream_t stream);

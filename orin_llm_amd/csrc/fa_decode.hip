@@ -26,8 +26,13 @@
 //     written per split; the combine kernel merges the splits that were active.
 #include "fa_common.hpp"
 
-// Cycle-counter stamps for profiling builds (defined by a prefix header there); nothing otherwise.
-#ifndef FA_STAMP
+// Stage marks: wall-clock stamps in the timeline build, nothing otherwise (fa_common.hpp).
+#ifdef ORIN_FA_STAMPS
+namespace orin_fa {
+__device__ long long g_decode_stamps[kStampWgs * kDecodeWaves * kStampSlots];
+}
+#define FA_STAMP(i) ORIN_FA_STAMP_STORE(orin_fa::g_decode_stamps, orin_fa::kDecodeWaves, i)
+#else
 #define FA_STAMP(i)
 #endif
 
@@ -656,6 +661,20 @@ hipError_t decode_allow_lds() {
     if ((e = allow_lds<64, 0>()) != hipSuccess) return e;
     if ((e = allow_lds<64, 1>()) != hipSuccess) return e;
     return allow_lds<64, 2>();
+}
+
+hipError_t decode_stamps(long long* host, size_t n) {
+#ifdef ORIN_FA_STAMPS
+    if (n > (size_t)kStampWgs * kDecodeWaves * kStampSlots) return hipErrorInvalidValue;
+    hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(g_decode_stamps), n * sizeof(long long)); // (synchronises with the device)
+    void* dev = nullptr;
+    if (e == hipSuccess) e = hipGetSymbolAddress(&dev, HIP_SYMBOL(g_decode_stamps));
+    if (e == hipSuccess) e = hipMemset(dev, 0, sizeof(g_decode_stamps)); // the next launch starts from an empty table
+    return e;
+#else
+    (void)host; (void)n;
+    return hipErrorNotSupported;
+#endif
 }
 
 } // namespace orin_fa

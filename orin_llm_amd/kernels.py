@@ -14,7 +14,10 @@ _vp = ctypes.c_void_p
 _int = ctypes.c_int
 _flt = ctypes.c_float
 
+STAMPS_LIB_PATH = os.path.join(_HERE, "liborin_fa_stamps.so")
+
 _lib = None
+_stamps_lib = None
 
 
 class OrinFaError(RuntimeError):
@@ -268,6 +271,31 @@ def bench_handoff(src, fused, scratch, out):
     rc = lib().orin_fa_bench_handoff(_ptr(src), int(fused), _ptr(scratch), _ptr(out))
     if rc != 0:
         raise OrinFaError("bench_handoff", rc)
+
+
+def stamps_lib():
+    """The timeline build of the library (stage marks of the attention kernels store the wall clock), as a
+    second, independent ctypes handle with its own state: init, set_stream, the two attention entry points
+    and orin_fa_bench_stamps.  A measurement aid of bench.py."""
+    global _stamps_lib
+    if _stamps_lib is None:
+        if not os.path.exists(STAMPS_LIB_PATH):
+            raise ImportError(f"{STAMPS_LIB_PATH} is missing: build it with __graft_entry__.build()")
+        L = ctypes.CDLL(STAMPS_LIB_PATH)
+        L.orin_fa_init.argtypes = [_int]
+        L.orin_fa_init.restype = _int
+        L.orin_fa_set_stream.argtypes = [_vp]
+        L.orin_fa_set_stream.restype = None
+        L.orin_fa_prefill.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _flt]
+        L.orin_fa_prefill.restype = _int
+        L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
+        L.orin_fa_decode_ind.restype = _int
+        L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
+        L.orin_fa_decode_splits.restype = _int
+        L.orin_fa_bench_stamps.argtypes = [_int, _vp, ctypes.c_size_t]
+        L.orin_fa_bench_stamps.restype = _int
+        _stamps_lib = L
+    return _stamps_lib
 
 
 def bench_handoff_sizes():

@@ -42,12 +42,22 @@ def test_header_declares_the_expected_entry_points():
 def test_measurement_aids_sit_in_their_own_header():
     assert _declared_c_functions(BENCH_HDR) == sorted([
         "orin_fa_decode_ind_timed", "orin_fa_bench_hbm_read", "orin_fa_bench_tiny_launch", "orin_fa_bench_handoff",
-        "orin_fa_bench_handoff_scratch_bytes", "orin_fa_bench_handoff_stream_bytes"])
+        "orin_fa_bench_handoff_scratch_bytes", "orin_fa_bench_handoff_stream_bytes", "orin_fa_bench_stamps"])
 
 
 def test_library_exports_every_declared_symbol(lib):
     for name in _declared_c_functions() + _declared_c_functions(BENCH_HDR):
         assert hasattr(lib, name), f"{name} declared in a header but not exported"
+
+
+def test_timeline_build_exports_the_same_symbols():
+    """liborin_fa_stamps.so is the same library with the attention kernels' stage marks switched on."""
+    path = os.path.join(os.path.dirname(LIB), "liborin_fa_stamps.so")
+    if not os.path.exists(path):
+        pytest.fail("liborin_fa_stamps.so is not built: run `python orin_llm_amd/build.py`")
+    stamps = ctypes.CDLL(path)
+    for name in _declared_c_functions() + _declared_c_functions(BENCH_HDR):
+        assert hasattr(stamps, name), f"{name} missing from the timeline build"
 
 
 def test_calls_that_need_no_device(lib):
