@@ -80,6 +80,11 @@ WORKLOADS = {
     "llama8b-prefill512-d4096-timeline": ("llama8b", "timeline", 8192, ("prefill", 4096, 512)),
     "qwen1.5b-prefill512-d3584-timeline": ("qwen1.5b", "timeline", 4096, ("prefill", 3584, 512)),
     "qwen1.5b-prefill512-d0-timeline": ("qwen1.5b", "timeline", 4096, ("prefill", 0, 512)),
+    # not part of the path: the decode split kernel with parts taken out (cut-off builds of the library, results
+    # wrong by design), timed like the decode workloads: what the combine launch, the products and the merge,
+    # the trip for the position, the query and the operand-order K loads each cost on top of a plain read
+    "qwen1.5b-decode-32k-cutoffs": ("qwen1.5b", "cutoffs", 32768, 32768),
+    "llama8b-decode-8k-cutoffs": ("llama8b", "cutoffs", 8192, 8192),   # (shapes where a wave has one tile: the cut-off kernel leaves after its first)
     "qwen1.5b-decode-32k-timeline": ("qwen1.5b", "timeline", 32768, ("decode", 32768, 1)),
     "qwen7b-decode-32k-timeline": ("qwen7b", "timeline", 32768, ("decode", 32767, 1)),
 }
@@ -101,7 +106,7 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 # "targets" at the very end of the line repeats their figures in a few hundred characters.
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
-        "llama8b-prefill512-d4096-timeline", "qwen1.5b-decode-32k-timeline", "decode-handoff-mock",
+        "llama8b-prefill512-d4096-timeline", "qwen1.5b-decode-32k-timeline", "qwen1.5b-decode-32k-cutoffs", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -847,6 +852,64 @@ def run_timeline(torch, kernels, name, steps, warmup, with_cpu):
                 parity=None, timeline_us=timeline)
 
 
+CUTOFFS = [(None, "whole layer (split + combine kernels)"), (1, "split kernel alone"),
+           (3, "... leaving once its first tile has arrived (no products, no merge, no partial)"),
+           (7, "... with a constant position"), (15, "... and no query loads"), (31, "... and K fetched whole lines at a time")]
+
+
+def run_cutoffs(torch, kernels, name, steps, warmup, with_cpu):
+    """Not the operator: the decode layer stack timed with the ordinary library and with each cut-off build (the split
+    kernel with parts taken out; their results are wrong by design), microseconds per layer, launches back to back."""
+    import ctypes
+
+    shape, _, n_ctx, L = WORKLOADS[name]
+    sh = SHAPES[shape]
+    H, G, d, n_layers = sh["H"], sh["G"], sh["d"], sh["layers"]
+    scale = 1.0 / float(np.sqrt(d))
+    layers = [make_layer(torch, 700 + i, H, G, d, n_ctx, L, 1, sh["outliers"]) for i in range(n_layers)]
+    out = torch.empty((H, d), dtype=torch.float32, device="cuda")
+    dpos = torch.tensor([L - 1], dtype=torch.int32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    us = {}
+    for flags, label in CUTOFFS:
+        if flags is None:
+            lib = kernels.lib()
+        else:
+            lib = kernels.probe_lib(flags)
+            rc = lib.orin_fa_init(0)
+            assert rc == 0, rc
+            lib.orin_fa_set_stream(stream)
+
+        def stack():
+            for q, k, v in layers:
+                rc = lib.orin_fa_decode_ind(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), H, G, d, n_ctx, dpos.data_ptr(), scale)
+                assert rc == 0, rc
+
+        for _ in range(max(1, warmup)):
+            stack()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(max(3, min(steps, 8))):
+            e0.record()
+            stack()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e3 / n_layers)
+        us[label] = round(best, 2)
+    by = decode_bytes(H, G, d, L)
+    whole = us[CUTOFFS[0][1]]
+    del layers
+    torch.cuda.empty_cache()
+    return dict(value=by / (whole * 1e-6) / 1e9, unit="GB/s", ms_per_step=whole * n_layers * 1e-3,
+                config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=n_layers, n_ctx=n_ctx, L=L, launch="eager"),
+                roofline=dict(bound="hbm", achieved=by / (whole * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=by / (whole * 1e-6) / PEAK_BYTES, traffic=None,
+                              kernel="fa_decode_split_kernel<128, 0>, whole and with parts taken out", launch_us=whole,
+                              bytes_per_launch=by),
+                parity=None, cutoffs_us_per_layer=us)
+
+
 def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
     """One step = 28 launches of the stand-in over rotating cold buffers; value = the two-launch form's rate."""
     nbytes, scratch_bytes = kernels.bench_handoff_sizes()
@@ -895,7 +958,7 @@ def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "kv_store": run_kv_store,
+    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 
@@ -944,6 +1007,7 @@ def main():
                              **({"graph": r["graph"], "eager": r["eager"]} if "graph" in r else {}),
                              **({"into_the_cache": r["into_the_cache"]} if "into_the_cache" in r else {}),
                              **({"timeline_us": r["timeline_us"]} if "timeline_us" in r else {}),
+                             **({"cutoffs_us_per_layer": r["cutoffs_us_per_layer"]} if "cutoffs_us_per_layer" in r else {}),
                              **({"cpu_baseline": r["cpu_baseline"]} if "cpu_baseline" in r else {})))
         line["also"] = also
         # The figures the targets are stated on, once more and briefly, as the last thing on the line.

@@ -44,6 +44,10 @@ size_t orin_fa_bench_handoff_stream_bytes(void);
  * a launch as such, when timed back to back.  Asynchronous. */
 int orin_fa_bench_tiny_launch(void);
 
+/* (The cut-off builds liborin_fa_probe_<flags>.so export the product ABI too, with the decode split kernel's
+ * parts taken out as orin_llm_amd/csrc/fa_decode.hip describes under ORIN_FA_DECODE_PROBE: their results are
+ * wrong by design and only bench.py's cut-off workloads load them.) */
+
 /* Timeline build only (liborin_fa_stamps.so: the same sources compiled with -DORIN_FA_STAMPS, in which
  * lane 0 of every wave of the prefill kernel and of the decode split kernel stores the 100 MHz wall
  * clock at the end of each stage).  Copies the table of the kernel's last launch to host memory:

@@ -9,6 +9,10 @@ LIB = os.path.join(HERE, "liborin_fa.so")
 # stage marks store the wall clock.  A measurement aid for bench.py's timeline workloads; never the library that is timed.
 STAMPS_LIB = os.path.join(HERE, "liborin_fa_stamps.so")
 STAMPED = ("fa_prefill.hip", "fa_decode.hip")
+# The cut-off builds: the decode split kernel with parts taken out (-DORIN_FA_DECODE_PROBE=flags, see fa_decode.hip;
+# results wrong by design), one library per flag set, for bench.py's cut-off workload.  Measurement aids.
+PROBE_FLAGS = (1, 3, 7, 15, 31)
+PROBE_LIB = os.path.join(HERE, "liborin_fa_probe_{}.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
            for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
@@ -54,11 +58,17 @@ def build(verbose=False):
     cmds = [[HIPCC] + FLAGS + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
     stamped = {s: os.path.join(OBJ_DIR, os.path.basename(s) + ".stamps.o") for s in SOURCES if os.path.basename(s) in STAMPED}
     cmds += [[HIPCC] + FLAGS + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
-    with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
+    dec = next(s for s in SOURCES if os.path.basename(s) == "fa_decode.hip")
+    probes = {f: os.path.join(OBJ_DIR, f"fa_decode.hip.probe{f}.o") for f in PROBE_FLAGS}
+    cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_DECODE_PROBE={f}", "-c", dec, "-o", o] for f, o in probes.items()]
+    with ThreadPoolExecutor(max_workers=8) as pool:
         lines = list(pool.map(_run, cmds))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [stamped.get(s, o) for s, o in zip(SOURCES, objs)]
                       + ["-o", STAMPS_LIB]))
+    for f, o in probes.items():
+        lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [o if s == dec else x for s, x in zip(SOURCES, objs)]
+                          + ["-o", PROBE_LIB.format(f)]))
     if verbose:
         print("\n".join(lines))
     return LIB

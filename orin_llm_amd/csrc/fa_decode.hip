@@ -36,8 +36,21 @@ __device__ long long g_decode_stamps[kStampWgs * kDecodeWaves * kStampSlots];
 #define FA_STAMP(i)
 #endif
 
+// Cut-off builds (-DORIN_FA_DECODE_PROBE=flags, liborin_fa_probe_<flags>.so; measurement aids whose RESULTS ARE
+// WRONG by design): the split kernel with parts taken out, so that bench.py's cut-off workload can say
+// what each part costs.  1: no combine launch.  2: the kernel leaves once its first tile has arrived
+// (no products, no merge, no partial).  4: the position is n_ctx - 1, not read from memory.
+// 8: no query loads.  16: K fetched whole lines at a time like V (its contents then in the wrong
+// lanes).  0 in the library proper, where none of this exists.
+#ifndef ORIN_FA_DECODE_PROBE
+#define ORIN_FA_DECODE_PROBE 0
+#endif
+
 namespace orin_fa {
 namespace {
+constexpr int kProbe = ORIN_FA_DECODE_PROBE;
+constexpr bool kProbeNoCombine = (kProbe & 1) != 0, kProbeCutOff = (kProbe & 2) != 0, kProbeConstPos = (kProbe & 4) != 0,
+               kProbeNoQuery = (kProbe & 8) != 0, kProbeKWholeLines = (kProbe & 16) != 0;
 
 template <int D>
 struct DGeom {
@@ -113,7 +126,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int kk = 0; kk < G::kSteps; ++kk)
-                kreg[t * G::kSteps + kk] = buf_load16<true>(krs, soff + (t * 16 + col) * D * 2 + (kk * 4 + grp) * 16);
+                kreg[t * G::kSteps + kk] = buf_load16<true>(krs, kProbeKWholeLines ? soff + ((t * G::kSteps + kk) * 64 + lane) * 16
+                                                                                    : soff + (t * 16 + col) * D * 2 + (kk * 4 + grp) * 16);
     };
     auto fetch_v = [&](int tile) {
         const int soff = tile * kTile * D * 2;
@@ -122,7 +136,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     };
     // ---- query heads: requested before the first tile, so that they arrive before it (a wave's
     // loads complete in order) and the score product can start while V is still on its way ----
-    const int pos = *d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
+    const int pos = kProbeConstPos ? n_ctx - 1 - (d_pos == nullptr) : *d_pos; // (read here, ahead of the statement below that may write memory: a scalar load)
     const int hl = hg * 16 + col;
     const bool valid = hl < r;
     // Columns past the group's heads are padding: their loads carry an offset past the descriptor's
@@ -139,7 +153,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     const float qmul = valid ? qsign : 0.0f;
     static_assert(kWaves % (2 * G::kSteps) == 0, "a piece per wave (the same piece twice at head_dim 64)");
     const int q_piece = __builtin_amdgcn_readfirstlane(wave) & (2 * G::kSteps - 1);
-    const float4 q_share = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, (q_piece >> 1) * 128 + (q_piece & 1) * 16, 0));
+    const float4 q_share = kProbeNoQuery ? float4{1.f, 2.f, (float)q_off, (float)lane}
+                                         : __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(qrs, q_off, (q_piece >> 1) * 128 + (q_piece & 1) * 16, 0));
     constexpr bool STORE = MODE != 0, ROPE = MODE == 2;
     // (rotate + store) lane i < n_rot/2 of every wave fetches what pair i's angle needs: its
     // cosine and sine when the caller supplies them, else its frequency factor if there is one.
@@ -216,6 +231,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     }
 
     FA_STAMP(1);
+    if constexpr (kProbeCutOff) { // (cut-off build: wait for the tile, keep every load alive, leave)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned acc = __float_as_uint(q_share.x) ^ __float_as_uint(q_share.w);
+#pragma unroll
+        for (int i = 0; i < 2 * G::kSteps; ++i) acc ^= kreg[i].x ^ kreg[i].y ^ kreg[i].z ^ kreg[i].w;
+#pragma unroll
+        for (int i = 0; i < G::kLoads; ++i) acc ^= vreg[i].x ^ vreg[i].y ^ vreg[i].z ^ vreg[i].w;
+        if (acc == 0x9E3779B9u) part_ml[0] = 1.0f;
+        if (acc != 0x9E3779BAu) return;
+    }
     // (the query pieces met ahead of the tile requests; the operands are picked up while the first tile is on its way)
     float qf[G::kSteps][8]; // this lane's 8 elements of every k-step: head_dim indices kk*32 + grp*8 + 0..7
 #pragma unroll
@@ -625,7 +650,7 @@ hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
 #undef ORIN_FA_SPLIT_ARGS
     hipError_t e = hipGetLastError();
     if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
-    if (e != hipSuccess || a.n_splits == 1) return e;
+    if (e != hipSuccess || a.n_splits == 1 || kProbeNoCombine) return e;
     const dim3 cgrid(a.n_head * (D / 64));
 #define ORIN_FA_COMBINE_ARGS a.part_o, a.part_ml, a.out, a.n_splits, a.n_head
     if (a.n_splits <= 32) hipLaunchKernelGGL((fa_decode_combine_kernel<D, 4>), cgrid, dim3(512), 0, stream, ORIN_FA_COMBINE_ARGS);

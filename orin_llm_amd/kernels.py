@@ -273,6 +273,22 @@ def bench_handoff(src, fused, scratch, out):
         raise OrinFaError("bench_handoff", rc)
 
 
+def probe_lib(flags):
+    """A cut-off build of the library (liborin_fa_probe_<flags>.so: the decode split kernel with parts taken
+    out, results wrong by design; see fa_decode.hip) as an independent ctypes handle.  A measurement aid of bench.py."""
+    path = os.path.join(_HERE, f"liborin_fa_probe_{int(flags)}.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with __graft_entry__.build()")
+    L = ctypes.CDLL(path)
+    L.orin_fa_init.argtypes = [_int]
+    L.orin_fa_init.restype = _int
+    L.orin_fa_set_stream.argtypes = [_vp]
+    L.orin_fa_set_stream.restype = None
+    L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
+    L.orin_fa_decode_ind.restype = _int
+    return L
+
+
 def stamps_lib():
     """The timeline build of the library (stage marks of the attention kernels store the wall clock), as a
     second, independent ctypes handle with its own state: init, set_stream, the two attention entry points

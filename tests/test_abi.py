@@ -60,6 +60,15 @@ def test_timeline_build_exports_the_same_symbols():
         assert hasattr(stamps, name), f"{name} missing from the timeline build"
 
 
+def test_cut_off_builds_are_there():
+    """The decode kernel's cut-off builds (measurement aids, results wrong by design) load and export the decode call."""
+    for flags in (1, 3, 7, 15, 31):
+        path = os.path.join(os.path.dirname(LIB), f"liborin_fa_probe_{flags}.so")
+        if not os.path.exists(path):
+            pytest.fail(f"{path} is not built: run `python orin_llm_amd/build.py`")
+        assert hasattr(ctypes.CDLL(path), "orin_fa_decode_ind")
+
+
 def test_calls_that_need_no_device(lib):
     lib.orin_fa_workspace_bytes.restype = ctypes.c_size_t
     assert lib.orin_fa_workspace_bytes() >= 256 * 32 * (128 + 2) * 4  # 256 splits of a 32-head model
