@@ -83,6 +83,8 @@ WORKLOADS = {
     # not part of the path: the decode split kernel with parts taken out (cut-off builds of the library, results
     # wrong by design), timed like the decode workloads: what the combine launch, the products and the merge,
     # the trip for the position, the query and the operand-order K loads each cost on top of a plain read
+    "llama8b-prefill512-d4096-cutoffs": ("llama8b", "cutoffs", 8192, (4096, 512)),   # ... and of the prefill kernel
+    "qwen1.5b-prefill512-d3584-cutoffs": ("qwen1.5b", "cutoffs", 4096, (3584, 512)),
     "qwen1.5b-decode-32k-cutoffs": ("qwen1.5b", "cutoffs", 32768, 32768),
     "llama8b-decode-8k-cutoffs": ("llama8b", "cutoffs", 8192, 8192),   # (shapes where a wave has one tile: the cut-off kernel leaves after its first)
     "qwen1.5b-decode-32k-timeline": ("qwen1.5b", "timeline", 32768, ("decode", 32768, 1)),
@@ -106,7 +108,8 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 # "targets" at the very end of the line repeats their figures in a few hundred characters.
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
-        "llama8b-prefill512-d4096-timeline", "qwen1.5b-decode-32k-timeline", "qwen1.5b-decode-32k-cutoffs", "decode-handoff-mock",
+        "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
+        "qwen1.5b-decode-32k-cutoffs", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -857,11 +860,69 @@ CUTOFFS = [(None, "whole layer (split + combine kernels)"), (1, "split kernel al
            (7, "... with a constant position"), (15, "... and no query loads"), (31, "... and K fetched whole lines at a time")]
 
 
+PREFILL_CUTOFFS = [(None, "whole kernel"), (16, "leaving once the accumulators are handed over (no barrier, merge, store)"),
+                   (8, "leaving behind the main loop (no last products either)"),
+                   (1, "whole, main loop without its vector work"), (2, "whole, main loop without its LDS operand reads"),
+                   (4, "whole, main loop without its copies"), (7, "whole, main loop of matrix instructions only")]
+
+
+def run_prefill_cutoffs(torch, kernels, name, steps, warmup):
+    """The prefill layer stack timed with the ordinary library and with each cut-off build of the prefill kernel."""
+    import ctypes
+
+    shape, _, n_ctx, (P, B) = WORKLOADS[name]
+    sh = SHAPES[shape]
+    H, G, d, n_layers = sh["H"], sh["G"], sh["d"], sh["layers"]
+    scale = 1.0 / float(np.sqrt(d))
+    layers = [make_layer(torch, 800 + i, H, G, d, n_ctx, P + B, B, sh["outliers"]) for i in range(n_layers)]
+    outs = [torch.empty((B, H, d), dtype=torch.float32, device="cuda") for _ in range(n_layers)]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    us = {}
+    for flags, label in PREFILL_CUTOFFS:
+        if flags is None:
+            lib = kernels.lib()
+        else:
+            lib = kernels.probe_lib(flags, prefill=True)
+            rc = lib.orin_fa_init(0)
+            assert rc == 0, rc
+            lib.orin_fa_set_stream(stream)
+
+        def stack():
+            for (q, k, v), o in zip(layers, outs):
+                rc = lib.orin_fa_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), H, G, d, n_ctx, P, B, scale)
+                assert rc == 0, rc
+
+        for _ in range(max(1, warmup)):
+            stack()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(max(3, min(steps, 6))):
+            e0.record()
+            stack()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e3 / n_layers)
+        us[label] = round(best, 2)
+    f = prefill_flops(H, d, P, B)
+    whole = us[PREFILL_CUTOFFS[0][1]]
+    del layers, outs
+    torch.cuda.empty_cache()
+    return dict(value=f / (whole * 1e-6) / 1e12, unit="TFLOP/s", ms_per_step=whole * n_layers * 1e-3,
+                config=dict(workload=name, shape=f"H{H} G{G} d{d}", layers=n_layers, n_ctx=n_ctx, n_past=P, batch=B, launch="eager"),
+                roofline=dict(bound="mfma", achieved=f / (whole * 1e-6) / 1e12, peak=PEAK_FLOPS / 1e12, unit="TFLOP/s",
+                              frac=f / (whole * 1e-6) / PEAK_FLOPS, traffic=None,
+                              kernel="fa_prefill_kernel, whole and with parts taken out", launch_us=whole, flops_per_launch=f),
+                parity=None, cutoffs_us_per_layer=us)
+
+
 def run_cutoffs(torch, kernels, name, steps, warmup, with_cpu):
     """Not the operator: the decode layer stack timed with the ordinary library and with each cut-off build (the split
     kernel with parts taken out; their results are wrong by design), microseconds per layer, launches back to back."""
     import ctypes
 
+    if isinstance(WORKLOADS[name][3], tuple):
+        return run_prefill_cutoffs(torch, kernels, name, steps, warmup)
     shape, _, n_ctx, L = WORKLOADS[name]
     sh = SHAPES[shape]
     H, G, d, n_layers = sh["H"], sh["G"], sh["d"], sh["layers"]

@@ -13,6 +13,9 @@ STAMPED = ("fa_prefill.hip", "fa_decode.hip")
 # results wrong by design), one library per flag set, for bench.py's cut-off workload.  Measurement aids.
 PROBE_FLAGS = (1, 3, 7, 15, 31)
 PROBE_LIB = os.path.join(HERE, "liborin_fa_probe_{}.so")
+# ... and of the prefill kernel (-DORIN_FA_PREFILL_PROBE=flags, see fa_prefill.hip)
+PPROBE_FLAGS = (1, 2, 4, 7, 8, 16)
+PPROBE_LIB = os.path.join(HERE, "liborin_fa_pprobe_{}.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
            for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
@@ -61,6 +64,9 @@ def build(verbose=False):
     dec = next(s for s in SOURCES if os.path.basename(s) == "fa_decode.hip")
     probes = {f: os.path.join(OBJ_DIR, f"fa_decode.hip.probe{f}.o") for f in PROBE_FLAGS}
     cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_DECODE_PROBE={f}", "-c", dec, "-o", o] for f, o in probes.items()]
+    pre = next(s for s in SOURCES if os.path.basename(s) == "fa_prefill.hip")
+    pprobes = {f: os.path.join(OBJ_DIR, f"fa_prefill.hip.probe{f}.o") for f in PPROBE_FLAGS}
+    cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_PREFILL_PROBE={f}", "-c", pre, "-o", o] for f, o in pprobes.items()]
     with ThreadPoolExecutor(max_workers=8) as pool:
         lines = list(pool.map(_run, cmds))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]))
@@ -69,6 +75,9 @@ def build(verbose=False):
     for f, o in probes.items():
         lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [o if s == dec else x for s, x in zip(SOURCES, objs)]
                           + ["-o", PROBE_LIB.format(f)]))
+    for f, o in pprobes.items():
+        lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [o if s == pre else x for s, x in zip(SOURCES, objs)]
+                          + ["-o", PPROBE_LIB.format(f)]))
     if verbose:
         print("\n".join(lines))
     return LIB

@@ -51,8 +51,19 @@ __device__ long long g_prefill_stamps[kStampWgs * kPrefillWaves * kStampSlots];
 #define FA_STAMP(i)
 #endif
 
+// Cut-off builds (-DORIN_FA_PREFILL_PROBE=flags, liborin_fa_pprobe_<flags>.so; measurement aids whose RESULTS
+// ARE WRONG by design): the kernel with parts taken out, so that bench.py's cut-off workload can say what
+// each part costs.  In the main loop -- 1: no vector work (the softmax of the step), 2: no LDS operand
+// reads, 4: no copies of the next tiles (7: matrix instructions only).  8: the kernel leaves behind the
+// main loop (no last products, no merge, no store).  16: it leaves once the waves have handed their
+// accumulators over (no barrier, no merge, no store).  0 in the library proper, where none of this exists.
+#ifndef ORIN_FA_PREFILL_PROBE
+#define ORIN_FA_PREFILL_PROBE 0
+#endif
+
 namespace orin_fa {
 namespace {
+constexpr int kPProbe = ORIN_FA_PREFILL_PROBE;
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
@@ -686,7 +697,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             // in order, so the wait for the earlier group's operand covers the later group's too.
             auto read_group = [&](auto gc) {
                 constexpr int g = decltype(gc)::value;
-                if constexpr (g < kCG) gop[g] = read_v(gc, (TP ^ 1) * G::kTileB);
+                if constexpr ((kPProbe & 2) != 0) { // (cut-off build: whatever the registers hold)
+                    if constexpr (g < kGroups) gop[g] = carry[g % kAhead];
+                }
+                else if constexpr (g < kCG) gop[g] = read_v(gc, (TP ^ 1) * G::kTileB);
                 else if constexpr (g < kGroups) gop[g] = *reinterpret_cast<const h8*>(kp[g - kCG] + (TP ^ 1) * G::kTileB);
                 else carry[g - kGroups] = read_v(IntC<g - kGroups>{}, TP * G::kTileB);     // for C(t) of the next step
             };
@@ -750,10 +764,10 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
                 // (the compiler orders the vector instructions within a ticket, not across tickets:
                 // the scores they read were written two or more matrix instructions earlier)
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (i >= kSkip)
+                if constexpr (i >= kSkip && (kPProbe & 1) == 0)
                     static_for<((i - kSkip) * kItems) / (kTickets - kSkip), ((i + 1 - kSkip) * kItems) / (kTickets - kSkip)>(item);
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (m == NCB - 1) {
+                if constexpr (m == NCB - 1 && (kPProbe & 4) == 0) {
                     if constexpr (i < kHalf) copy_one(IntC<i / NCB>{}, kdesc, k_buf(TP), ksoff);
                     else copy_one(IntC<(i - kHalf) / NCB>{}, vdesc, v_buf(TP ^ 1), vsoff);
                 }
@@ -819,6 +833,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         }
         if (t == R) body(IntC<0>{}, t);
         FA_STAMP(4);
+        if constexpr ((kPProbe & 8) != 0) { if (n_past >= 0) return; } // (cut-off build)
         // ---- drain: C(R), and the accumulators on their way to the merge ----
         // V(R) has landed once the two tiles of copies issued after it are all that is outstanding
         // (those, for steps past the last, land in buffers nobody reads; their latency hides
@@ -886,6 +901,7 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
         });
     }
     FA_STAMP(5);
+    if constexpr ((kPProbe & 16) != 0) { if (n_past >= 0) return; } // (cut-off build)
     FA_STAMP(6);
     __syncthreads();
     FA_STAMP(7);
@@ -949,8 +965,18 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
             __builtin_amdgcn_sched_barrier(0);
             if (h == 0) load_half(kHalfJ);
             __builtin_amdgcn_sched_barrier(0);
+            // Output rows leave with streaming stores: they go on their way to memory as each workgroup
+            // finishes, instead of sitting in L2 until the kernel's end writes megabytes of them back at
+            // once (1.2 us per launch on a Llama-3-8B chunk; a KV split's partial results, which the
+            // combine kernel reads next, are better left to the caches: 1.5 us the other way on 16 splits).
+            if (kv_split_shift > 0) {
 #pragma unroll
-            for (int j = 0; j < kHalfJ; ++j) *reinterpret_cast<f4*>(dst + ((h * kHalfJ + j) * kParts + part) * 4) = acc[j];
+                for (int j = 0; j < kHalfJ; ++j) *reinterpret_cast<f4*>(dst + ((h * kHalfJ + j) * kParts + part) * 4) = acc[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < kHalfJ; ++j) // (spelled out: as a builtin the hint is lost when the compiler merges the two branches)
+                    asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(dst + ((h * kHalfJ + j) * kParts + part) * 4), "v"(acc[j]) : "memory");
+            }
         }
     }
     FA_STAMP(8);

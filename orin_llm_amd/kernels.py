@@ -273,10 +273,11 @@ def bench_handoff(src, fused, scratch, out):
         raise OrinFaError("bench_handoff", rc)
 
 
-def probe_lib(flags):
+def probe_lib(flags, prefill=False):
     """A cut-off build of the library (liborin_fa_probe_<flags>.so: the decode split kernel with parts taken
-    out, results wrong by design; see fa_decode.hip) as an independent ctypes handle.  A measurement aid of bench.py."""
-    path = os.path.join(_HERE, f"liborin_fa_probe_{int(flags)}.so")
+    out; liborin_fa_pprobe_<flags>.so: the prefill kernel; results wrong by design; see fa_decode.hip and
+    fa_prefill.hip) as an independent ctypes handle.  A measurement aid of bench.py."""
+    path = os.path.join(_HERE, f"liborin_fa_{'pprobe' if prefill else 'probe'}_{int(flags)}.so")
     if not os.path.exists(path):
         raise ImportError(f"{path} is missing: build it with __graft_entry__.build()")
     L = ctypes.CDLL(path)
@@ -286,6 +287,8 @@ def probe_lib(flags):
     L.orin_fa_set_stream.restype = None
     L.orin_fa_decode_ind.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt]
     L.orin_fa_decode_ind.restype = _int
+    L.orin_fa_prefill.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _flt]
+    L.orin_fa_prefill.restype = _int
     return L
 
 

@@ -67,6 +67,11 @@ def test_cut_off_builds_are_there():
         if not os.path.exists(path):
             pytest.fail(f"{path} is not built: run `python orin_llm_amd/build.py`")
         assert hasattr(ctypes.CDLL(path), "orin_fa_decode_ind")
+    for flags in (1, 2, 4, 7, 8, 16):
+        path = os.path.join(os.path.dirname(LIB), f"liborin_fa_pprobe_{flags}.so")
+        if not os.path.exists(path):
+            pytest.fail(f"{path} is not built: run `python orin_llm_amd/build.py`")
+        assert hasattr(ctypes.CDLL(path), "orin_fa_prefill")
 
 
 def test_calls_that_need_no_device(lib):
