@@ -51,7 +51,8 @@ __global__ __launch_bounds__(256) void kv_store_kernel(uint16_t* kc, uint16_t* v
         half8 h;
         h[0] = (_Float16)x0.x; h[1] = (_Float16)x0.y; h[2] = (_Float16)x0.z; h[3] = (_Float16)x0.w;
         h[4] = (_Float16)x1.x; h[5] = (_Float16)x1.y; h[6] = (_Float16)x1.z; h[7] = (_Float16)x1.w;
-        *reinterpret_cast<half8*>(dst) = h;
+        // (streaming store: the row is read next by another kernel, from other compute units)
+        __builtin_nontemporal_store(h, reinterpret_cast<half8*>(dst));
     } else {
         const _Float16 h = (_Float16)src[0];
         dst[0] = __builtin_bit_cast(uint16_t, h);
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(256) void kv_shift_kernel(uint16_t* kc, uint16_t* v
     for (; p + shift < n_ctx; p += shift) {
         if constexpr (PIECE == 16) {
             const piece_t x = *reinterpret_cast<const piece_t*>(base + (size_t)(p + shift) * row_bytes);
-            *reinterpret_cast<piece_t*>(base + (size_t)p * row_bytes) = x;
+            __builtin_nontemporal_store(x, reinterpret_cast<piece_t*>(base + (size_t)p * row_bytes));
         } else {
             const uint16_t x = *reinterpret_cast<const uint16_t*>(base + (size_t)(p + shift) * row_bytes);
             *reinterpret_cast<uint16_t*>(base + (size_t)p * row_bytes) = x;

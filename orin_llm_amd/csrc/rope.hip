@@ -24,6 +24,13 @@ namespace {
 
 constexpr int kHeadsPerThread = 8;
 
+// The rotated rows and the cache rows are read next by another kernel, on other compute units:
+// streaming stores send them on instead of leaving them dirty in this die's cache until the
+// kernel ends.
+__device__ __forceinline__ void store_stream(float* p, const float4& v) {
+    __builtin_nontemporal_store(f4{v.x, v.y, v.z, v.w}, reinterpret_cast<f4*>(p));
+}
+
 template <bool NEOX, bool IND>
 __global__ __launch_bounds__(256) void rope_kernel(float* x, int tokens, int heads, int head_dim, int n_rot,
                                                    float theta, int n_past, const int* d_pos,
@@ -132,8 +139,8 @@ __global__ __launch_bounds__(256) void rope4_kernel(float* x, int tokens, int he
                 rope_rotate(b[u].x, b[u].y, c[2], sn[2]);
                 rope_rotate(b[u].z, b[u].w, c[3], sn[3]);
             }
-            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o0) = a[u];
-            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o1) = b[u];
+            store_stream(row + (size_t)u * head_dim + o0, a[u]);
+            store_stream(row + (size_t)u * head_dim + o1, b[u]);
         }
 }
 
@@ -164,7 +171,7 @@ __global__ __launch_bounds__(256) void rope_store_kernel(float* q, float* k, con
         half8_t h;
         h[0] = (_Float16)x0.x; h[1] = (_Float16)x0.y; h[2] = (_Float16)x0.z; h[3] = (_Float16)x0.w;
         h[4] = (_Float16)x1.x; h[5] = (_Float16)x1.y; h[6] = (_Float16)x1.z; h[7] = (_Float16)x1.w;
-        *reinterpret_cast<half8_t*>(vc + ((size_t)head * n_ctx + pos) * head_dim + piece * 8) = h;
+        __builtin_nontemporal_store(h, reinterpret_cast<half8_t*>(vc + ((size_t)head * n_ctx + pos) * head_dim + piece * 8));
         return;
     }
     const bool is_k = blockIdx.x >= nbq;
@@ -212,15 +219,15 @@ __global__ __launch_bounds__(256) void rope_store_kernel(float* q, float* k, con
                 rope_rotate(b[u].x, b[u].y, c[2], sn[2]);
                 rope_rotate(b[u].z, b[u].w, c[3], sn[3]);
             }
-            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o0) = a[u];
-            *reinterpret_cast<float4*>(row + (size_t)u * head_dim + o1) = b[u];
+            store_stream(row + (size_t)u * head_dim + o0, a[u]);
+            store_stream(row + (size_t)u * head_dim + o1, b[u]);
             if (is_k) {
                 uint16_t* dst = kc + ((size_t)(h0 + u) * n_ctx + pos) * head_dim;
                 half4_t ha, hb;
                 ha[0] = (_Float16)a[u].x; ha[1] = (_Float16)a[u].y; ha[2] = (_Float16)a[u].z; ha[3] = (_Float16)a[u].w;
                 hb[0] = (_Float16)b[u].x; hb[1] = (_Float16)b[u].y; hb[2] = (_Float16)b[u].z; hb[3] = (_Float16)b[u].w;
-                *reinterpret_cast<half4_t*>(dst + o0) = ha;
-                *reinterpret_cast<half4_t*>(dst + o1) = hb;
+                __builtin_nontemporal_store(ha, reinterpret_cast<half4_t*>(dst + o0));
+                __builtin_nontemporal_store(hb, reinterpret_cast<half4_t*>(dst + o1));
             }
         }
 }
