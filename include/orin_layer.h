@@ -1,0 +1,119 @@
+/*
+ * orin_layer -- C ABI of the decode layer around the attention path on MI355X (gfx950): the
+ * operators the orin_llm engine's decode_layer calls between its attention calls (reference:
+ * src/model_gpu.cu:251-293, captured as a graph by :295-316), and one call that runs a whole
+ * layer in six launches.  Part of liborin_fa.so; conventions as in orin_fa.h (device pointers
+ * owned by the caller, asynchronous launches on the stream of orin_fa_set_stream, process-global
+ * state, 0 or a negative ORIN_FA_E_* code).  Nothing here allocates or synchronises: every entry
+ * point may run under stream capture.
+ *
+ * Weight matrices are GGUF tensors as the reference maps them (reference: src/common.h:47-77,
+ * src/quant.h:14-45): `type` is the ggml type number (0 F32, 1 F16, 8 Q8_0, 12 Q4_K, 13 Q5_K,
+ * 14 Q6_K), a matrix is n_out rows of n_in elements, rows packed back to back.
+ * Limits: n_in a multiple of 32 (256 for the K types), at most 24576; matrices of type F32, F16,
+ * Q4_K, Q5_K 16-byte aligned (2 bytes for Q8_0 and Q6_K, whose blocks are 34 and 210 bytes);
+ * activations and outputs 16-byte aligned.  ORIN_FA_E_INVALID otherwise.
+ *
+ * Arithmetic: the reference's GPU operators round the activation to int8 in blocks of 32 before a
+ * product (quantize_activation + dp4a).  These keep it in fp32 and decode the weights to the exact
+ * fp32 values of the reference's CPU backend (src/model_cpu.cpp:70-167), so results agree with that
+ * backend up to the order of the fp32 sum.
+ */
+#ifndef ORIN_LAYER_H
+#define ORIN_LAYER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ORIN_F32 = 0, ORIN_F16 = 1, ORIN_Q8_0 = 8, ORIN_Q4_K = 12, ORIN_Q5_K = 13, ORIN_Q6_K = 14 };
+
+/* Bytes of a row of n elements of the given type; 0 for an unknown type or a partial block
+ * (reference: tensor_nbytes, src/common.h:72-77). */
+size_t orin_row_bytes(int type, int n);
+
+/* Replaces llm::cuda::rms_norm and rms_norm_rows (reference: src/kernels.h:43-44,
+ * src/kernels.cu:1596-1617, 2029-2039): y = x / sqrt(mean(x^2) + eps) * w, per row of `cols` elements with
+ * one weight vector for all rows.  y may be x. */
+int orin_rms_norm(const float* x, const float* w, int n, float eps, float* y);
+int orin_rms_norm_rows(const float* x, const float* w, int rows, int cols, float eps, float* y);
+
+/* Replaces llm::cuda::quantize_activation (reference: src/kernels.h:15, src/kernels.cu:136-157, 1778-1784).
+ * The reference stores an int8 copy of x for the *_q8 products that follow; this stores an fp32
+ * copy (n_in <= 32768) in the library's own device memory, so that those products see x as it
+ * was at this call, as they do in the reference. */
+int orin_quantize_activation(const float* x, int n_in);
+
+/* Replace llm::cuda::gemv_q8 / gemv_q8_bias / gemv_q8_add (reference: src/kernels.h:21-27,
+ * src/kernels.cu:1786-1806, 1825-1836): y = W xs, y = W xs + bias, y += W xs, with xs the activation of the
+ * last orin_quantize_activation call (whose n_in must equal this n_in). */
+int orin_gemv_q8(int type, const void* W, float* y, int n_in, int n_out);
+int orin_gemv_q8_bias(int type, const void* W, const float* bias, float* y, int n_in, int n_out);
+int orin_gemv_q8_add(int type, const void* W, float* y, int n_in, int n_out);
+
+/* Replaces llm::cuda::gemv_fused_gate_up_swiglu (reference: src/kernels.h:33-34,
+ * src/kernels.cu:1944-1954): out[i] = silu(Wg[i] . xs) * (Wu[i] . xs), both matrices of `type`. */
+int orin_gemv_fused_gate_up_swiglu(int type, const void* Wg, const void* Wu, float* out, int n_in, int n_out);
+
+/* Replaces llm::cuda::gemv (reference: src/kernels.h:18, src/kernels.cu:1808-1823): y = W x with x
+ * given directly (the output matrix behind the last norm). */
+int orin_gemv(int type, const void* W, const float* x, float* y, int n_in, int n_out);
+
+/* Replaces llm::cuda::dequant_row (reference: src/kernels.h:38, src/kernels.cu:1572-1585, 2004-2014): one
+ * weight row of n elements to fp32 (the token's embedding), bit for bit what the reference's CPU
+ * backend decodes. */
+int orin_dequant_row(int type, const void* src, float* y, int n);
+
+/* Replaces llm::cuda::swiglu (reference: src/kernels.h:47, src/kernels.cu:1702-1707, 2041-2044):
+ * act[i] = silu(gate[i]) * up[i]. */
+int orin_swiglu(float* act, const float* gate, const float* up, int n);
+
+/* ---- forms with no counterpart in the reference: fewer launches per layer ---- */
+
+/* Up to three matrices of one type over the same activation in one launch (the q, k, v
+ * projections), the RMS norm folded in: y_m = W_m norm(x) + bias_m, with
+ * norm(x) = x / sqrt(mean(x^2) + eps) * norm_w computed by every workgroup for itself (norm_w NULL:
+ * no norm), bias_m NULL: none.  accumulate != 0: y_m += instead. */
+int orin_gemv_multi(int type, int n_mat, const void* const* W, const float* const* bias, float* const* y,
+                    const int* n_out, const float* x, const float* norm_w, float eps, int n_in, int accumulate);
+
+/* out[i] = silu(Wg[i] . norm(x)) * (Wu[i] . norm(x)): the layer's second norm and its gate/up pair in
+ * one launch. */
+int orin_gemv_norm_gate_up_swiglu(int type, const void* Wg, const void* Wu, const float* x, const float* norm_w,
+                                  float eps, float* out, int n_in, int n_out);
+
+/* One decode layer (reference: src/model_gpu.cu:251-293), six launches where the types allow:
+ *   [attn_norm + q, k, v projections (+ bias)]  [per-head q/k norms, if the model has them]
+ *   [rotary embedding + cache store + attention: orin_fa_decode_rope_store_ind, two launches]
+ *   [output projection, added to x]  [ffn_norm + gate/up + SwiGLU]  [down projection, added to x]
+ * Projections of different types take a launch each; a rotary layout the fused attention call does
+ * not take (NeoX pairing with n_rot < head_dim) goes through the separate rope and store calls.
+ * x is updated in place; q, k, v, attn, act (and up_tmp, needed only when ffn_gate and ffn_up
+ * differ in type) are scratch the caller provides; k and v leave un-rotated / as projected. */
+typedef struct orin_decode_layer_desc {
+    int n_embd, n_head, n_kv, head_dim, n_ff, n_ctx, n_rot, neox;
+    float rms_eps, rope_theta, scale;
+    int wq_type, wk_type, wv_type, wo_type, gate_type, up_type, down_type;
+    const void *wq, *wk, *wv, *wo, *ffn_gate, *ffn_up, *ffn_down;
+    const float *attn_norm, *ffn_norm;
+    const float *q_norm, *k_norm;   /* [head_dim] each, or NULL */
+    const float *bq, *bk, *bv;      /* or NULL */
+    const float* freq_factors;      /* [n_rot / 2], or NULL */
+    const float* rope_angles;       /* table of orin_fa_rope_angles_ind for this token, or NULL */
+    uint16_t *kc, *vc;              /* this layer's cache */
+    float* x;                       /* [n_embd] */
+    float *q, *k, *v;               /* [n_head * head_dim], [n_kv * head_dim] twice */
+    float* attn;                    /* [n_head * head_dim] */
+    float* act;                     /* [n_ff] */
+    float* up_tmp;                  /* [n_ff], or NULL */
+    const int* d_pos;
+} orin_decode_layer_desc;
+int orin_decode_layer(const orin_decode_layer_desc* layer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -191,3 +191,134 @@ def attention_f64(q, k, v, n_past, scale):
         p /= p.sum(axis=1, keepdims=True)
         out[:, h, :] = p @ v[g, :L, :]
     return out
+
+
+# ---- the decode layer around attention (layer_ref.h) ----
+
+F32, F16, Q8_0, Q4_K, Q5_K, Q6_K = 0, 1, 8, 12, 13, 14
+_vp = ctypes.c_void_p
+
+
+def _layer_lib():
+    l = lib()
+    if not getattr(l, "_layer_ready", False):
+        l.orc_row_bytes.argtypes = [_int, ctypes.c_int64]
+        l.orc_row_bytes.restype = ctypes.c_size_t
+        l.orc_dequantize_row.argtypes = [_int, _vp, _f32p, ctypes.c_int64]
+        l.orc_dequantize_row.restype = _int
+        l.orc_gemv.argtypes = [_int, _vp, _f32p, _f32p, _int, _int, _f32p]
+        l.orc_gemv.restype = _int
+        l.orc_rms_norm.argtypes = [_f32p, _f32p, _int, _flt, _f32p]
+        l.orc_rms_norm.restype = None
+        l.orc_swiglu.argtypes = [_f32p, _f32p, _f32p, _int]
+        l.orc_swiglu.restype = None
+        l._layer_ready = True
+    return l
+
+
+def row_bytes(wtype, n):
+    return int(_layer_lib().orc_row_bytes(wtype, n))
+
+
+def dequantize_row(wtype, raw, k):
+    """raw: the row's bytes (uint8 array); returns fp32 [k]."""
+    raw = _c(raw, np.uint8)
+    assert raw.size >= row_bytes(wtype, k) > 0
+    y = np.empty(k, np.float32)
+    assert _layer_lib().orc_dequantize_row(wtype, raw.ctypes.data, _p(y, _f32p), k) == 0
+    return y
+
+
+def gemv(wtype, raw, x, n_in, n_out):
+    """raw: n_out rows of n_in elements of type wtype (uint8 array); x fp32 [n_in]; returns fp32 [n_out]."""
+    raw, x = _c(raw, np.uint8), _c(x, np.float32)
+    assert raw.size >= row_bytes(wtype, n_in) * n_out > 0 and x.size == n_in
+    y = np.empty(n_out, np.float32)
+    row = np.empty(n_in, np.float32)
+    assert _layer_lib().orc_gemv(wtype, raw.ctypes.data, _p(x, _f32p), _p(y, _f32p), n_in, n_out, _p(row, _f32p)) == 0
+    return y
+
+
+def rms_norm(x, w, eps):
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    y = np.empty(x.size, np.float32)
+    _layer_lib().orc_rms_norm(_p(x, _f32p), _p(w, _f32p), x.size, np.float32(eps), _p(y, _f32p))
+    return y
+
+
+def swiglu(gate, up):
+    gate, up = _c(gate, np.float32), _c(up, np.float32)
+    act = np.empty(gate.size, np.float32)
+    _layer_lib().orc_swiglu(_p(act, _f32p), _p(gate, _f32p), _p(up, _f32p), gate.size)
+    return act
+
+
+class RefState:
+    """The caches of one sequence: fp32 as the reference's CPU backend keeps them
+    (src/model_cpu.cpp:217,226-231), or, with fp16_cache, rounded to fp16 on the way in as the
+    GPU backend's cache is (src/kernels.cu:1675-1677)."""
+
+    def __init__(self, model, n_ctx, fp16_cache=False):
+        hp = model["hp"]
+        shape = (hp["n_layer"], hp["n_kv"], n_ctx, hp["head_dim"])
+        self.n_ctx, self.fp16_cache = n_ctx, fp16_cache
+        self.kc = np.zeros(shape, np.float32)
+        self.vc = np.zeros(shape, np.float32)
+
+
+def decode_forward(model, state, token, n_past, trace=None):
+    """One token through the whole model, as src/model_cpu.cpp:241-312 walks it; returns the logits.
+
+    model: {"hp": {n_vocab, n_embd, n_layer, n_head, n_kv, head_dim, n_ff, n_rot, rms_eps,
+    rope_theta, neox, freq_factors}, "token_embd": T, "output": T, "output_norm": fp32 array,
+    "layers": [{"wq", "wk", "wv", "wo", "ffn_gate", "ffn_up", "ffn_down": T, "attn_norm", "ffn_norm":
+    fp32 arrays, optional "bq", "bk", "bv", "q_norm", "k_norm": fp32 arrays}]} with
+    T = (type, uint8 array of the tensor's bytes, n_in, n_out).
+    trace: optional dict that receives the intermediate vectors of every layer.
+    """
+    hp = model["hp"]
+    ne, nh, nkv, d, nff = hp["n_embd"], hp["n_head"], hp["n_kv"], hp["head_dim"], hp["n_ff"]
+    eps, n_ctx = hp["rms_eps"], state.n_ctx
+    scale = np.float32(1.0) / np.sqrt(np.float32(d))
+
+    def mv(t, x):
+        return gemv(t[0], t[1], x, t[2], t[3])
+
+    def rope(x, heads):
+        return rope_batch(x.reshape(heads, d), d, hp["n_rot"], hp["rope_theta"], n_past, heads,
+                          hp.get("freq_factors"), bool(hp["neox"])).reshape(-1)
+
+    et, eraw, e_in, _ = model["token_embd"]
+    rb = row_bytes(et, e_in)
+    x = dequantize_row(et, eraw[token * rb:(token + 1) * rb], ne)
+    for li, L in enumerate(model["layers"]):
+        xn = rms_norm(x, L["attn_norm"], eps)
+        q, k, v = mv(L["wq"], xn), mv(L["wk"], xn), mv(L["wv"], xn)
+        if L.get("bq") is not None:
+            q = q + L["bq"]
+        if L.get("bk") is not None:
+            k = k + L["bk"]
+        if L.get("bv") is not None:
+            v = v + L["bv"]
+        if L.get("q_norm") is not None:
+            q = np.concatenate([rms_norm(q[h * d:(h + 1) * d], L["q_norm"], eps) for h in range(nh)])
+        if L.get("k_norm") is not None:
+            k = np.concatenate([rms_norm(k[h * d:(h + 1) * d], L["k_norm"], eps) for h in range(nkv)])
+        q, k = rope(q, nh), rope(k, nkv)
+        if state.fp16_cache:
+            k_in, v_in = fp16_to_fp32(fp32_to_fp16(k)), fp16_to_fp32(fp32_to_fp16(v))
+        else:
+            k_in, v_in = k, v
+        state.kc[li, :, n_past, :] = k_in.reshape(nkv, d)
+        state.vc[li, :, n_past, :] = v_in.reshape(nkv, d)
+        attn = attention_token_f32(q.reshape(nh, d), state.kc[li], state.vc[li], nh, nkv, d, n_ctx, n_past + 1,
+                                   scale).reshape(-1)
+        x1 = x + mv(L["wo"], attn)
+        xn2 = rms_norm(x1, L["ffn_norm"], eps)
+        act = swiglu(mv(L["ffn_gate"], xn2), mv(L["ffn_up"], xn2))
+        x2 = x1 + mv(L["ffn_down"], act)
+        if trace is not None:
+            trace[li] = dict(x_in=x, xn=xn, q=q, k=k, v=v, attn=attn, x_mid=x1, xn2=xn2, act=act, x_out=x2)
+        x = x2
+    xn = rms_norm(x, model["output_norm"], eps)
+    return mv(model["output"], xn)

@@ -5,7 +5,7 @@
 // (reference: src/kernels.h:77-81, launchers at src/kernels.cu:1944-2000) and its KV-cache
 // mutators kv_store_batch / kv_store_ind / kv_shift (src/kernels.h:66-73, src/kernels.cu:2079-2093) and the
 // rotary embedding rope_{neox,normal}_{batch,ind} (src/kernels.h:55-62, src/kernels.cu:2059-2075).
-#include "fa_common.hpp"
+#include "layer_common.hpp"
 
 #include <stdio.h>
 
@@ -22,6 +22,9 @@ namespace {
 constexpr size_t kStaticScratchBytes = 2u << 20;
 constexpr int kMaxDevices = 16;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// The activation that orin_quantize_activation stages for the *_q8 products (include/orin_layer.h),
+// held the same way.
+static __device__ __align__(256) float stage[kStageFloats];
 
 struct State {
     bool ready = false;
@@ -34,6 +37,7 @@ struct State {
     size_t ws_bytes = 0;
     bool ws_is_own = false;
     void* static_ws[kMaxDevices] = {}; // device address of `scratch`, per device
+    float* stage[kMaxDevices] = {};    // device address of `stage`, per device
 };
 State g_state;
 
@@ -78,6 +82,12 @@ int check_common(const void* q, const void* kc, const void* vc, const void* out,
 }
 
 } // namespace
+
+bool lib_ready() { return g_state.ready; }
+int lib_cu_count() { return g_state.cu_count; }
+hipStream_t lib_stream() { return g_state.stream; }
+float* lib_stage() { return g_state.ready ? g_state.stage[g_state.device] : nullptr; }
+
 } // namespace orin_fa
 
 using namespace orin_fa;
@@ -132,6 +142,15 @@ int orin_fa_init(int device) {
             return hip_code(e);
         }
         g_state.static_ws[device] = ptr;
+    }
+    if (!g_state.stage[device]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(stage));
+        if (e != hipSuccess) {
+            fprintf(stderr, "[orin_fa] hipGetSymbolAddress(stage) failed on device %d: %s\n", device, hipGetErrorString(e));
+            return hip_code(e);
+        }
+        g_state.stage[device] = static_cast<float*>(ptr);
     }
     g_state.ready = true;
     return ORIN_FA_OK;

@@ -1,0 +1,51 @@
+// Shared pieces of the decode-layer operators around attention (gemv.hip, layer_ops.hip,
+// layer_api.hip): weight types, launch arguments, launchers.
+#pragma once
+
+#include "fa_common.hpp"
+
+namespace orin_fa {
+
+// Weight types, numbered as the reference numbers them (reference: src/common.h:47-54).
+enum : int { kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14 };
+
+constexpr int kMaxGemvIn = 24576;   // elements per weight row, at most (4 waves x 64 lanes x 3 slots x 32)
+constexpr int kStageFloats = 32768; // the staged activation of the *_q8 entry points
+
+struct GemvSeg {
+    const void* w;     // n_out rows
+    const float* bias; // or null
+    float* y;
+    int n_out;
+};
+
+struct GemvArgs {
+    GemvSeg seg[3];      // matrices of one type that share the activation
+    int n_seg;
+    const void* w_up;    // not null: seg[0].w is the gate matrix, this the up matrix, y = SiLU(gate x) * (up x)
+    const float* x;      // activation, n_in floats, 16-byte aligned
+    const float* norm_w; // not null: the activation is RMS-normalised with this weight first
+    float eps;
+    int n_in;
+    int accumulate;      // y += instead of y =
+    // filled in by the launcher
+    size_t row_bytes;
+    int rows_per_wg, team_waves;
+};
+
+size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
+int weight_align(int type);               // alignment the kernels need of a matrix's base address
+hipError_t gemv_launch(int type, GemvArgs args, int cu_count, hipStream_t stream);
+
+hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream);
+hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream);
+hipError_t swiglu_launch(float* act, const float* gate, const float* up, int n, hipStream_t stream);
+hipError_t dequant_row_launch(int type, const void* src, float* y, int n, hipStream_t stream);
+
+// Library state the operators share with the attention entry points (fa_api.hip).
+bool lib_ready();
+int lib_cu_count();
+hipStream_t lib_stream();
+float* lib_stage(); // device address of the staged activation on the current device, or null
+
+} // namespace orin_fa

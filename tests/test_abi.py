@@ -10,6 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "orin_llm_amd", "liborin_fa.so")
 HDR = os.path.join(ROOT, "include", "orin_fa.h")
 BENCH_HDR = os.path.join(ROOT, "include", "orin_fa_bench.h")
+LAYER_HDR = os.path.join(ROOT, "include", "orin_layer.h")
 SHIM_HDR = os.path.join(ROOT, "include", "orin_llm_amd", "kernels.h")
 REF_HDR = "/root/reference/src/kernels.h"
 
@@ -21,7 +22,7 @@ def _strip_comments(text):
 
 def _declared_c_functions(header=HDR):
     body = _strip_comments(open(header).read())
-    return sorted(set(re.findall(r"\b(orin_fa_[a-z_]+)\s*\(", body)))
+    return sorted(set(re.findall(r"\b(orin_[a-z0-9_]+)\s*\(", body)))
 
 
 @pytest.fixture(scope="module")
@@ -45,8 +46,15 @@ def test_measurement_aids_sit_in_their_own_header():
         "orin_fa_bench_handoff_scratch_bytes", "orin_fa_bench_handoff_stream_bytes", "orin_fa_bench_stamps"])
 
 
+def test_layer_header_declares_the_expected_entry_points():
+    assert _declared_c_functions(LAYER_HDR) == sorted([
+        "orin_row_bytes", "orin_rms_norm", "orin_rms_norm_rows", "orin_quantize_activation", "orin_gemv_q8",
+        "orin_gemv_q8_bias", "orin_gemv_q8_add", "orin_gemv_fused_gate_up_swiglu", "orin_gemv", "orin_dequant_row",
+        "orin_swiglu", "orin_gemv_multi", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"])
+
+
 def test_library_exports_every_declared_symbol(lib):
-    for name in _declared_c_functions() + _declared_c_functions(BENCH_HDR):
+    for name in _declared_c_functions() + _declared_c_functions(BENCH_HDR) + _declared_c_functions(LAYER_HDR):
         assert hasattr(lib, name), f"{name} declared in a header but not exported"
 
 
