@@ -34,9 +34,9 @@ PEAK_FLOPS = 2.5e15
 PEAK_BYTES = 8.0e12
 
 SHAPES = {
-    "qwen1.5b": dict(H=12, G=2, d=128, layers=28, outliers=4),
-    "llama8b": dict(H=32, G=8, d=128, layers=32, outliers=0),
-    "qwen7b": dict(H=28, G=4, d=128, layers=28, outliers=4),
+    "qwen1.5b": dict(H=12, G=2, d=128, layers=28, outliers=4, n_embd=1536, n_ff=8960, bias=True, neox=1, theta=1.0e6),
+    "llama8b": dict(H=32, G=8, d=128, layers=32, outliers=0, n_embd=4096, n_ff=14336, bias=False, neox=0, theta=5.0e5),
+    "qwen7b": dict(H=28, G=4, d=128, layers=28, outliers=4, n_embd=3584, n_ff=18944, bias=True, neox=1, theta=1.0e6),
 }
 
 WORKLOADS = {
@@ -75,6 +75,12 @@ WORKLOADS = {
     # partials), its partials merged by a second kernel, as the library does, or inside the launch by a two-level
     # last-arriver reduction over write-through stores and relaxed atomics -- what fusing the combine would cost
     "decode-handoff-mock": (None, "handoff", 0, 32 << 20),
+    # The whole decode layer around the path (norms, quantised projections, rotary embedding, cache store,
+    # attention, feed-forward block): one token through every layer of the model, replayed as one graph.
+    # Weights are random blocks in the mix of a Q4_K_M file (Q4_K; attn_v and ffn_down Q6_K).
+    "qwen1.5b-decode-layer-32k": ("qwen1.5b", "decode_layer", 32768, 32768),
+    "llama8b-decode-layer-8k": ("llama8b", "decode_layer", 8192, 8192),
+    "qwen7b-decode-layer-32k": ("qwen7b", "decode_layer", 32768, 32767),
     # not timed: where a kernel's microseconds go, from the timeline build of the library (the attention kernels'
     # stage marks store the wall clock there; medians over the waves of one launch, cold inputs)
     "llama8b-prefill512-d4096-timeline": ("llama8b", "timeline", 8192, ("prefill", 4096, 512)),
@@ -109,7 +115,7 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
         "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
-        "qwen1.5b-decode-32k-cutoffs", "decode-handoff-mock",
+        "qwen1.5b-decode-32k-cutoffs", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -1017,9 +1023,171 @@ def run_handoff(torch, kernels, name, steps, warmup, with_cpu):
                 parity=dict(both_forms_give_the_known_sum=same))
 
 
+def random_weight(torch, gen, wtype, n_in, n_out, std=0.03):
+    """Random blocks of a weight type with sane fp16 scales (every other byte random), on the device."""
+    per, nbytes = {0: (1, 4), 1: (1, 2), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210)}[wtype]
+    nb = n_in // per * n_out
+    if wtype in (0, 1):
+        w = torch.randn((n_out, n_in), generator=gen, device="cuda") * std
+        return (w if wtype == 0 else w.half()).contiguous().view(torch.uint8).reshape(-1)
+    raw = torch.randint(0, 256, (nb, nbytes), generator=gen, device="cuda", dtype=torch.uint8)
+    halves = raw.view(torch.float16)  # [nb][nbytes / 2]
+    u = torch.rand(nb, generator=gen, device="cuda") + 0.5
+    if wtype == 8:
+        halves[:, 0] = (std / 74.0 * u).half()
+    elif wtype == 12:
+        halves[:, 0] = (std / 166.0 * u).half()
+        halves[:, 1] = (std / 166.0 * 7.5 * u).half()
+    elif wtype == 13:
+        halves[:, 0] = (std / 340.0 * u).half()
+        halves[:, 1] = (std / 340.0 * 15.5 * u).half()
+    else:
+        halves[:, 104] = (std / 1369.0 * u).half()
+    return raw.reshape(-1)
+
+
+def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = one token through every layer of the model: orin_decode_layer per layer (six or seven
+    launches: norm + q/k/v projections, rotary embedding + cache store + attention, output projection,
+    norm + gate/up + SwiGLU, down projection), replayed as one HIP graph as the reference replays its decode
+    step (src/model_gpu.cu:295-344).  value = HBM bytes the layer must read (its weights once, its cache
+    once) per second."""
+    from oracle import ref
+    from orin_llm_amd import layer as ly
+
+    shape_name, _, n_ctx, L = WORKLOADS[name]
+    s = SHAPES[shape_name]
+    H, G, d, layers, ne, nff = s["H"], s["G"], s["d"], s["layers"], s["n_embd"], s["n_ff"]
+    Q4, Q6 = ly.Q4_K, ly.Q6_K
+    types = dict(wq=Q4, wk=Q4, wv=Q6, wo=Q4, ffn_gate=Q4, ffn_up=Q4, ffn_down=Q6)
+    dims = dict(wq=(ne, H * d), wk=(ne, G * d), wv=(ne, G * d), wo=(H * d, ne), ffn_gate=(ne, nff), ffn_up=(ne, nff),
+                ffn_down=(nff, ne))
+    hp = dict(n_embd=ne, n_head=H, n_kv=G, head_dim=d, n_ff=nff, n_rot=d, neox=s["neox"], rms_eps=1e-6, rope_theta=s["theta"],
+              freq_factors_dev=None)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4242)
+    weight_bytes = sum(ly.row_bytes(types[k], dims[k][0]) * dims[k][1] for k in types)
+    kv_bytes = 4.0 * G * L * d
+    bytes_layer = weight_bytes + kv_bytes
+    model = []
+    for l in range(layers):
+        Lw = {k: (types[k], random_weight(torch, gen, types[k], *dims[k])) for k in types}
+        Lw["attn_norm"] = 1.0 + 0.1 * torch.randn(ne, generator=gen, device="cuda")
+        Lw["ffn_norm"] = 1.0 + 0.1 * torch.randn(ne, generator=gen, device="cuda")
+        if s["bias"]:
+            Lw["bq"], Lw["bk"], Lw["bv"] = (0.1 * torch.randn(n, generator=gen, device="cuda") for n in (H * d, G * d, G * d))
+        k = torch.randn((G, n_ctx, d), generator=gen, device="cuda", dtype=torch.float32).half().view(torch.int16)
+        v = torch.randn((G, n_ctx, d), generator=gen, device="cuda", dtype=torch.float32).half().view(torch.int16)
+        model.append((Lw, k, v))
+    z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")  # noqa: E731
+    bufs = dict(x=z(ne), q=z(H * d), k=z(G * d), v=z(G * d), attn=z(H * d), act=z(nff), up_tmp=z(nff), xn=z(ne), xn2=z(ne))
+    x0 = torch.randn(ne, generator=gen, device="cuda")
+    dpos = torch.tensor([L - 1], dtype=torch.int32, device="cuda")
+    angles = torch.zeros((d // 2, 2), device="cuda")
+    descs = [ly.make_desc(hp, Lw, bufs, k, v, dpos, n_ctx, rope_angles=angles) for Lw, k, v in model]
+
+    def one_step():
+        bufs["x"].copy_(x0)
+        kernels.rope_angles_ind(angles, d, s["theta"], dpos)
+        for dsc in descs:
+            ly.decode_layer(dsc)
+
+    def one_step_calls():  # the reference's own sequence of operator calls (src/model_gpu.cu:251-293)
+        bufs["x"].copy_(x0)
+        for Lw, k, v in model:
+            ly.decode_layer_calls(hp, Lw, bufs, k, v, dpos, n_ctx)
+
+    wall, dev_ms, forms = time_eager_and_graph(torch, kernels, one_step, steps, warmup)
+    us_layer = dev_ms * 1e3 / (steps * layers)
+    _, dev_calls_ms, forms_calls = time_eager_and_graph(torch, kernels, one_step_calls, max(3, steps // 2), min(warmup, 2))
+    us_layer_calls = dev_calls_ms * 1e3 / (max(3, steps // 2) * layers)
+
+    # Each launch of layer 0 alone, by event pairs (eager, cold-ish: the other layers ran in between).
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    Lw, k0, v0 = model[0]
+    launches = {
+        "norm + q,k (one launch)": lambda: ly.gemv_multi(Q4, [Lw["wq"][1], Lw["wk"][1]], [Lw.get("bq"), Lw.get("bk")], [bufs["q"], bufs["k"]],
+                                                         [H * d, G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
+        "norm + v": lambda: ly.gemv_multi(Q6, [Lw["wv"][1]], [Lw.get("bv")], [bufs["v"]], [G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
+        "rope + store + attention (two launches)": lambda: kernels.flash_attention_decode_rope_store_ind(
+            bufs["q"], bufs["k"], bufs["v"], k0, v0, bufs["attn"], H, G, d, n_ctx, dpos, float(1.0 / np.sqrt(d)), d, s["theta"],
+            None, bool(s["neox"]), angles),
+        "output projection (+=)": lambda: ly.gemv_multi(Q4, [Lw["wo"][1]], None, [bufs["x"]], [ne], bufs["attn"], None, 0.0, H * d, True),
+        "norm + gate/up + SwiGLU": lambda: ly.gemv_norm_gate_up_swiglu(Q4, Lw["ffn_gate"][1], Lw["ffn_up"][1], bufs["x"], Lw["ffn_norm"], 1e-6,
+                                                                      bufs["act"], ne, nff),
+        "down projection (+=)": lambda: ly.gemv_multi(Q6, [Lw["ffn_down"][1]], None, [bufs["x"]], [ne], bufs["act"], None, 0.0, nff, True),
+    }
+    launch_bytes = {"norm + q,k (one launch)": ly.row_bytes(Q4, ne) * (H + G) * d, "norm + v": ly.row_bytes(Q6, ne) * G * d,
+                    "rope + store + attention (two launches)": kv_bytes, "output projection (+=)": ly.row_bytes(Q4, H * d) * ne,
+                    "norm + gate/up + SwiGLU": 2 * ly.row_bytes(Q4, ne) * nff, "down projection (+=)": ly.row_bytes(Q6, nff) * ne}
+    launch_us = {}
+    bufs["x"].copy_(x0)
+    for what, fn in launches.items():
+        ts = []
+        for rep in range(7):
+            for dsc in descs[1:4]:  # other layers' weights through the caches in between
+                ly.decode_layer(dsc)
+            ev[0].record()
+            fn()
+            ev[1].record()
+            torch.cuda.synchronize()
+            ts.append(ev[0].elapsed_time(ev[1]) * 1e3)
+        launch_us[what] = dict(us=round(float(np.median(ts)), 2), MB=round(launch_bytes[what] / 1e6, 2),
+                               GBps=round(launch_bytes[what] / (float(np.median(ts)) * 1e-6) / 1e9, 1))
+
+    # Parity: layer 0 from x0, against the oracle's operators in the reference's order (fp16 cache).
+    bufs["x"].copy_(x0)
+    kernels.rope_angles_ind(angles, d, s["theta"], dpos)
+    kc_before, vc_before = k0.clone(), v0.clone()
+    ly.decode_layer(descs[0])
+    torch.cuda.synchronize()
+    got = bufs["x"].cpu().numpy()
+    t0 = time.perf_counter()
+    host = {k: (v[0], v[1].cpu().numpy()) if isinstance(v, tuple) else v.cpu().numpy() for k, v in Lw.items()}
+    mv = lambda key, x: ref.gemv(host[key][0], host[key][1], x, dims[key][0], dims[key][1])  # noqa: E731
+    xh = x0.cpu().numpy()
+    t_cpu0 = time.perf_counter()
+    xn = ref.rms_norm(xh, host["attn_norm"], 1e-6)
+    qh, kh, vh = mv("wq", xn), mv("wk", xn), mv("wv", xn)
+    if s["bias"]:
+        qh, kh, vh = qh + host["bq"], kh + host["bk"], vh + host["bv"]
+    qh = ref.rope_batch(qh.reshape(H, d), d, d, s["theta"], L - 1, H, None, bool(s["neox"]))
+    kh = ref.rope_batch(kh.reshape(G, d), d, d, s["theta"], L - 1, G, None, bool(s["neox"]))
+    kc_h, vc_h = kc_before.cpu().numpy().view(np.uint16).copy(), vc_before.cpu().numpy().view(np.uint16).copy()
+    ref.kv_store_f16(kc_h, vc_h, kh.reshape(1, G, d), vh.reshape(1, G, d), G, d, n_ctx, L - 1, 1)
+    attn = ref.flash_attention_decode_ind(qh, kc_h, vc_h, H, G, d, n_ctx, L - 1, float(1.0 / np.sqrt(d))).reshape(-1)
+    x1 = xh + mv("wo", attn)
+    act = ref.swiglu(mv("ffn_gate", ref.rms_norm(x1, host["ffn_norm"], 1e-6)), mv("ffn_up", ref.rms_norm(x1, host["ffn_norm"], 1e-6)))
+    want = x1 + mv("ffn_down", act)
+    cpu_s = time.perf_counter() - t_cpu0
+    err = float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max())
+    # the token's cache rows: fp16 roundings of projections that differ in the last bits of their fp32 sums
+    row_k = ref.fp16_to_fp32(k0.cpu().numpy().view(np.uint16)[:, L - 1]) - ref.fp16_to_fp32(kc_h[:, L - 1])
+    row_v = ref.fp16_to_fp32(v0.cpu().numpy().view(np.uint16)[:, L - 1]) - ref.fp16_to_fp32(vc_h[:, L - 1])
+    cache_err = float(max(np.abs(row_k).max() / np.abs(ref.fp16_to_fp32(kc_h[:, L - 1])).max(),
+                          np.abs(row_v).max() / np.abs(ref.fp16_to_fp32(vc_h[:, L - 1])).max()))
+    main_key = "norm + gate/up + SwiGLU"
+    res = dict(value=bytes_layer * layers * steps / (dev_ms * 1e-3) / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3,
+               config=dict(workload=name, shape=f"H{H} G{G} d{d} n_embd {ne} n_ff {nff}", layers=layers, n_ctx=n_ctx, L=L,
+                           weights="Q4_K, attn_v and ffn_down Q6_K", weight_MB_per_layer=round(weight_bytes / 1e6, 2),
+                           cache_MB_per_layer=round(kv_bytes / 1e6, 2), launch="graph" if forms["graph"]["device_ms_per_step"] <= forms["eager"]["device_ms_per_step"] else "eager"),
+               roofline=dict(bound="hbm", achieved=launch_bytes[main_key] / (launch_us[main_key]["us"] * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9,
+                             unit="GB/s", frac=launch_bytes[main_key] / (launch_us[main_key]["us"] * 1e-6) / PEAK_BYTES, traffic=None,
+                             kernel="gemv_kernel<Q4_K, dual> (norm + gate/up + SwiGLU)", launch_us=launch_us[main_key]["us"],
+                             bytes_per_launch=launch_bytes[main_key], layer_us=us_layer, layer_frac=bytes_layer / (us_layer * 1e-6) / PEAK_BYTES,
+                             layer_us_reference_call_sequence=us_layer_calls, launches=launch_us),
+               parity=dict(err_row=err, err_floor1pct=err, cache_row_err=cache_err,
+                           rows="layer 0's output vector, max |got - want| / max |want|, vs the CPU oracle's operators in the reference's order"),
+               **forms)
+    if with_cpu:
+        res["cpu_baseline"] = dict(value=bytes_layer / cpu_s / 1e9, unit="GB/s", cores=1, kind="port",
+                                   sample=f"layer 0 of {layers}, every operator, {cpu_s:.1f} s")
+    return res
+
+
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
+    fn = {"decode_layer": run_decode_layer, "prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 

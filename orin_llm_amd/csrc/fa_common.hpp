@@ -144,6 +144,29 @@ __device__ __forceinline__ float xor_sum(float v) {
     return __uint_as_float(s.x) + __uint_as_float(s.y);
 }
 
+// Sums and maxima over the 64 lanes of a wave: inside rows of 16 by DPP moves, across the four rows by
+// the lane-swap instructions; every lane ends up with the result.
+__device__ __forceinline__ float dpp_xor_step(float v, int which) {
+    // lane i <-> the lane whose index differs within its row of 16: 1, 2 (quad permutes), 7 - i within 8, 15 - i within 16
+    const int x = __float_as_int(v);
+    int y;
+    if (which == 0) y = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);       // quad_perm [1,0,3,2]
+    else if (which == 1) y = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    else if (which == 2) y = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false); // row_half_mirror
+    else y = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false);                 // row_mirror
+    return __int_as_float(y);
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v = fmaxf(v, dpp_xor_step(v, i));
+    return xor_max(v); // across the four rows of 16
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v += dpp_xor_step(v, i);
+    return xor_sum(v);
+}
+
 // 16-byte load through a buffer descriptor: the hardware returns zeros for offsets at or
 // past the descriptor's byte count, so rows beyond the bound are never fetched and need no
 // branch.

@@ -553,27 +553,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
 // The 8 waves' weighted sums meet in LDS behind the kernel's only barrier.  Partial outputs of
 // inactive splits hold stale data and are never multiplied.
 // PER: splits per wave (n_splits <= 8 * PER; the launcher picks the smallest that fits).
-__device__ __forceinline__ float dpp_xor_step(float v, int which) {
-    // lane i <-> the lane whose index differs within its row of 16: 1, 2 (quad permutes), 7 - i within 8, 15 - i within 16
-    const int x = __float_as_int(v);
-    int y;
-    if (which == 0) y = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);       // quad_perm [1,0,3,2]
-    else if (which == 1) y = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
-    else if (which == 2) y = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false); // row_half_mirror
-    else y = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false);                 // row_mirror
-    return __int_as_float(y);
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v = fmaxf(v, dpp_xor_step(v, i));
-    return xor_max(v); // across the four rows of 16
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v += dpp_xor_step(v, i);
-    return xor_sum(v);
-}
-
 template <int D, int PER>
 __global__ __launch_bounds__(512) void fa_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                                  float* __restrict__ out, const int n_splits, const int n_head) {

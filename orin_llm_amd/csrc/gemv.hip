@@ -26,6 +26,8 @@
 //     type that share the activation (the q, k, v projections).
 #include "layer_common.hpp"
 
+#include <stdlib.h>
+
 namespace orin_fa {
 namespace {
 
@@ -40,12 +42,6 @@ struct __attribute__((packed, aligned(2))) Loose { // a vector at an address tha
 template <typename V>
 __device__ __forceinline__ V load_loose(const unsigned char* p) {
     return reinterpret_cast<const Loose<V>*>(p)->v;
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
 }
 
 // Per weight type: kRuns runs of kRunLen consecutive activations make up a slot's 32; run_start
@@ -263,30 +259,62 @@ struct Fmt<kF32> {
 constexpr int kGemvWaves = 4;
 
 // T: weight type.  SLOTS: slots per lane.  DUAL: two matrices (gate, up) and SiLU(gate) * up.
-// Grid: (row blocks, matrices).  Rows per iteration and team: RB.
+// Grid: (workgroups, matrices).  A workgroup walks row groups g = blockIdx.x, + gridDim.x, ...; a row
+// group is RB rows for each of the workgroup's teams.  The rows of group g + gridDim.x are requested
+// before those of group g are multiplied out, and the first group before the activation is even
+// loaded, so a workgroup always has two groups of weight bytes on their way.
 template <int T, int SLOTS, bool DUAL>
 __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const GemvArgs a) {
     using F = Fmt<T>;
-    constexpr int RB = SLOTS == 1 ? 4 : SLOTS == 2 ? 2 : 1;
-    __shared__ float sh_red[kGemvWaves][4];
+    constexpr int RB = SLOTS == 1 ? 2 : 1;
+    constexpr int M = DUAL ? 2 : 1;
+    __shared__ float sh_red[kGemvWaves][M * RB];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int kw = a.team_waves;                 // waves per row: 1, 2 or 4
     const int team = wave / kw, n_teams = kGemvWaves / kw;
     const int tt = (wave % kw) * 64 + lane, ts = kw * 64;
     const int n_slots = a.n_in >> 5;
     const GemvSeg seg = a.seg[blockIdx.y];
+    const size_t row_bytes = a.row_bytes;
+    const unsigned char* const w0 = static_cast<const unsigned char*>(seg.w);
+    const unsigned char* const w1 = static_cast<const unsigned char*>(DUAL ? a.w_up : seg.w);
+    const int last = seg.n_out - 1;
+    const int per_group = n_teams * RB;
+    const int n_groups = (seg.n_out + per_group - 1) / per_group;
+    if ((int)blockIdx.x >= n_groups) return; // (whole workgroup: a shorter matrix of a shared launch)
+
+    bool live[SLOTS];
+    int slot[SLOTS];
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) {
+        live[i] = i * ts + tt < n_slots;
+        slot[i] = live[i] ? i * ts + tt : 0; // (idle lanes repeat slot 0 and count for nothing)
+    }
+    typedef typename F::Raw Raw;
+    Raw raw_a[M][RB][SLOTS], raw_b[M][RB][SLOTS];
+    auto request = [&](Raw (&raw)[M][RB][SLOTS], int g) {
+        g = min(g, n_groups - 1); // (past the end: the last group once more, from the cache; never used)
+#pragma unroll
+        for (int b = 0; b < RB; ++b) {
+            const int row = min(g * per_group + team * RB + b, last);
+#pragma unroll
+            for (int i = 0; i < SLOTS; ++i) {
+                F::load(w0 + (size_t)row * row_bytes, slot[i], raw[0][b][i]);
+                if constexpr (DUAL) F::load(w1 + (size_t)row * row_bytes, slot[i], raw[1][b][i]);
+            }
+        }
+    };
+    request(raw_a, blockIdx.x);
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- this lane's activations, once ----
     float x[SLOTS][32], xs[SLOTS][F::kRuns];
-    bool live[SLOTS];
     float ss = 0.0f;
 #pragma unroll
     for (int i = 0; i < SLOTS; ++i) {
-        const int s = i * ts + tt;
-        live[i] = s < n_slots;
 #pragma unroll
         for (int r = 0; r < F::kRuns; ++r) {
-            const int e0 = live[i] ? F::run_start(s, r) : 0;
+            const int e0 = F::run_start(slot[i], r);
 #pragma unroll
             for (int j = 0; j < F::kRunLen; j += 4) {
                 const float4 v = *reinterpret_cast<const float4*>(a.x + e0 + j);
@@ -303,7 +331,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const GemvArgs a)
         }
     }
     if (a.norm_w) {
-        // x / sqrt(mean(x^2) + eps) * w (reference: src/kernels.cu rms_norm_k, CPU src/model_cpu.cpp:13-18)
+        // x / sqrt(mean(x^2) + eps) * w (reference: src/kernels.cu:1596-1604, CPU src/model_cpu.cpp:13-18)
         ss = wave_sum(ss);
         if (kw > 1) {
             if (lane == 0) sh_red[wave][0] = ss;
@@ -328,62 +356,45 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const GemvArgs a)
             xs[i][r] = t;
         }
 
-    const size_t row_bytes = a.row_bytes;
-    const unsigned char* const w0 = static_cast<const unsigned char*>(seg.w);
-    const unsigned char* const w1 = static_cast<const unsigned char*>(DUAL ? a.w_up : seg.w);
-    const int row_begin = blockIdx.x * a.rows_per_wg;
-    const int last = seg.n_out - 1;
-    if (row_begin > last) return; // (whole workgroup: a shorter matrix of a shared launch)
-    for (int r0 = row_begin + team * RB; r0 < row_begin + a.rows_per_wg; r0 += n_teams * RB) {
-        typename F::Raw raw[DUAL ? 2 : 1][RB][SLOTS];
+    auto finish = [&](const Raw (&raw)[M][RB][SLOTS], int g) {
+        float acc[M][RB];
 #pragma unroll
-        for (int b = 0; b < RB; ++b) {
-            const int row = min(r0 + b, last); // (rows past the end repeat the last one; nothing is written for them)
-#pragma unroll
-            for (int i = 0; i < SLOTS; ++i) {
-                const int s = live[i] ? i * ts + tt : 0;
-                F::load(w0 + (size_t)row * row_bytes, s, raw[0][b][i]);
-                if constexpr (DUAL) F::load(w1 + (size_t)row * row_bytes, s, raw[1][b][i]);
-            }
-        }
-        float acc[DUAL ? 2 : 1][RB];
-#pragma unroll
-        for (int m = 0; m < (DUAL ? 2 : 1); ++m)
+        for (int m = 0; m < M; ++m)
 #pragma unroll
             for (int b = 0; b < RB; ++b) {
                 float t = 0.0f;
 #pragma unroll
                 for (int i = 0; i < SLOTS; ++i) {
-                    const int s = live[i] ? i * ts + tt : 0;
-                    const float part = F::dot(raw[m][b][i], s, x[i], xs[i]);
+const float part = F::dot(raw[m][b][i], slot[i], x[i], xs[i]);
                     t += live[i] ? part : 0.0f;
                 }
                 acc[m][b] = wave_sum(t);
             }
-        if (kw > 1) { // the team's waves meet in LDS (every wave of the workgroup walks the same number of iterations)
+        if (kw > 1) { // the team's waves meet in LDS (every wave of the workgroup walks the same groups)
+            if (lane == 0)
 #pragma unroll
-            for (int m = 0; m < (DUAL ? 2 : 1); ++m) {
-                if (lane == 0)
+                for (int m = 0; m < M; ++m)
 #pragma unroll
-                    for (int b = 0; b < RB; ++b) sh_red[wave][b] = acc[m][b];
-                __syncthreads();
+                    for (int b = 0; b < RB; ++b) sh_red[wave][m * RB + b] = acc[m][b];
+            __syncthreads();
+#pragma unroll
+            for (int m = 0; m < M; ++m)
 #pragma unroll
                 for (int b = 0; b < RB; ++b) {
                     float t = 0.0f;
-                    for (int w = 0; w < kw; ++w) t += sh_red[team * kw + w][b];
+                    for (int w = 0; w < kw; ++w) t += sh_red[team * kw + w][m * RB + b];
                     acc[m][b] = t;
                 }
-                __syncthreads();
-            }
+            __syncthreads();
         }
         if (lane == 0 && wave % kw == 0) {
 #pragma unroll
             for (int b = 0; b < RB; ++b) {
-                const int row = r0 + b;
+                const int row = g * per_group + team * RB + b;
                 if (row > last) continue;
                 float v = acc[0][b];
                 if constexpr (DUAL) {
-                    // SiLU(gate) * up (reference: src/kernels.cu gemv_fused_gate_up_swiglu_k, CPU src/model_cpu.cpp:11,302)
+                    // SiLU(gate) * up (reference: src/kernels.cu:396-492, CPU src/model_cpu.cpp:11,302)
                     v = v / (1.0f + expf(-v)) * acc[1][b];
                 }
                 if (seg.bias) v += seg.bias[row];
@@ -391,6 +402,14 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const GemvArgs a)
                 seg.y[row] = v;
             }
         }
+    };
+    const int stride = gridDim.x;
+    for (int g = blockIdx.x; g < n_groups; g += 2 * stride) {
+        request(raw_b, g + stride);
+        finish(raw_a, g);
+        if (g + stride >= n_groups) break;
+        request(raw_a, g + 2 * stride);
+        finish(raw_b, g + stride);
     }
 }
 
@@ -405,7 +424,6 @@ hipError_t launch_slots(const GemvArgs& a, dim3 grid, hipStream_t stream) {
 
 template <int T>
 hipError_t launch_type(GemvArgs& a, int cu_count, hipStream_t stream) {
-    using F = Fmt<T>;
     const int n_slots = a.n_in / 32;
     // Fewest waves per row that keep a lane at three slots or fewer (96 activations in registers).
     int kw = 1;
@@ -413,16 +431,14 @@ hipError_t launch_type(GemvArgs& a, int cu_count, hipStream_t stream) {
     const int slots = (n_slots + kw * 64 - 1) / (kw * 64);
     if (slots > 3) return hipErrorInvalidValue;
     a.team_waves = kw;
-    const int rb = slots == 1 ? 4 : slots == 2 ? 2 : 1;
-    const int per_iter = (kGemvWaves / kw) * rb; // rows a workgroup finishes per iteration
+    const int per_group = (kGemvWaves / kw) * (slots == 1 ? 2 : 1);
     int max_out = 0;
     for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
-    // About eight workgroups per CU when the matrix has the rows for it, at most eight iterations each.
-    int iters = max_out / (per_iter * cu_count * 8);
-    iters = iters < 1 ? 1 : iters > 8 ? 8 : iters;
-    a.rows_per_wg = per_iter * iters;
-    const dim3 grid((max_out + a.rows_per_wg - 1) / a.rows_per_wg, a.n_seg);
-    (void)F::kAlign;
+    // At most kGemvWgsPerCu workgroups per CU, each walking its share of the row groups: the activation is
+    // fetched once per workgroup, so fewer, longer-lived workgroups keep that traffic below the weights'.
+    const int n_groups = (max_out + per_group - 1) / per_group;
+    const int wgs = min(n_groups, cu_count * a.wgs_per_cu);
+    const dim3 grid(wgs, a.n_seg);
     switch (slots) {
     case 1: return launch_slots<T, 1>(a, grid, stream);
     case 2: return launch_slots<T, 2>(a, grid, stream);
@@ -431,6 +447,16 @@ hipError_t launch_type(GemvArgs& a, int cu_count, hipStream_t stream) {
 }
 
 } // namespace
+
+// Workgroups per CU of a launch (ORIN_GEMV_WGS_PER_CU overrides, for tuning runs).
+int gemv_wgs_per_cu() {
+    static const int v = [] {
+        const char* e = getenv("ORIN_GEMV_WGS_PER_CU");
+        const int n = e ? atoi(e) : 0;
+        return n >= 1 && n <= 16 ? n : 2;
+    }();
+    return v;
+}
 
 size_t weight_row_bytes(int type, int n) {
     switch (type) {
@@ -449,6 +475,7 @@ int weight_align(int type) { return type == kQ6_K || type == kQ8_0 ? 2 : 16; }
 hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
     a.row_bytes = weight_row_bytes(type, a.n_in);
     if (a.row_bytes == 0 || a.n_in % 32 != 0 || a.n_seg < 1 || a.n_seg > 3) return hipErrorInvalidValue;
+    if (a.wgs_per_cu < 1) a.wgs_per_cu = gemv_wgs_per_cu();
     switch (type) {
     case kF32: return launch_type<kF32>(a, cu_count, stream);
     case kF16: return launch_type<kF16>(a, cu_count, stream);

@@ -30,7 +30,7 @@ struct GemvArgs {
     int accumulate;      // y += instead of y =
     // filled in by the launcher
     size_t row_bytes;
-    int rows_per_wg, team_waves;
+    int team_waves, wgs_per_cu;
 };
 
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks

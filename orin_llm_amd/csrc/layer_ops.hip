@@ -10,12 +10,6 @@
 namespace orin_fa {
 namespace {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-
 // y = x / sqrt(mean(x^2) + eps) * w over each row of cols elements (reference CPU statement:
 // src/model_cpu.cpp:13-18; w is shared by the rows).  One workgroup per row; y may be x: a thread
 // writes only elements it has read itself.
