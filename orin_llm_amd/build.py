@@ -18,7 +18,7 @@ PPROBE_FLAGS = (1, 2, 4, 7, 8, 16)
 PPROBE_LIB = os.path.join(HERE, "liborin_fa_pprobe_{}.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
-           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "gemv.hip", "layer_ops.hip",
+           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "gemv.hip", "gemv_mfma.hip", "layer_ops.hip",
                      "layer_api.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

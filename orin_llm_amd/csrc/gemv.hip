@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_kernel(const GemvArgs a)
                 float t = 0.0f;
 #pragma unroll
                 for (int i = 0; i < SLOTS; ++i) {
-const float part = F::dot(raw[m][b][i], slot[i], x[i], xs[i]);
+                    const float part = F::dot(raw[m][b][i], slot[i], x[i], xs[i]);
                     t += live[i] ? part : 0.0f;
                 }
                 acc[m][b] = wave_sum(t);
@@ -458,6 +458,25 @@ int gemv_wgs_per_cu() {
     return v;
 }
 
+// Workgroups per CU of the matrix-core kernel (0: one per 16-row tile; ORIN_GEMV_MFMA_WGS_PER_CU overrides).
+int gemv_mfma_wgs_per_cu() {
+    static const int v = [] {
+        const char* e = getenv("ORIN_GEMV_MFMA_WGS_PER_CU");
+        const int n = e ? atoi(e) : -1;
+        return n >= 0 && n <= 16 ? n : 2;
+    }();
+    return v;
+}
+
+// ORIN_GEMV_NO_MFMA=1 keeps every type on the vector-ALU kernel (for comparisons).
+bool gemv_use_mfma() {
+    static const bool v = [] {
+        const char* e = getenv("ORIN_GEMV_NO_MFMA");
+        return !(e && e[0] == '1');
+    }();
+    return v;
+}
+
 size_t weight_row_bytes(int type, int n) {
     switch (type) {
     case kF32: return (size_t)n * 4;
@@ -476,11 +495,14 @@ hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
     a.row_bytes = weight_row_bytes(type, a.n_in);
     if (a.row_bytes == 0 || a.n_in % 32 != 0 || a.n_seg < 1 || a.n_seg > 3) return hipErrorInvalidValue;
     if (a.wgs_per_cu < 1) a.wgs_per_cu = gemv_wgs_per_cu();
+    a.mfma_wgs_per_cu = gemv_mfma_wgs_per_cu();
     switch (type) {
     case kF32: return launch_type<kF32>(a, cu_count, stream);
     case kF16: return launch_type<kF16>(a, cu_count, stream);
     case kQ8_0: return launch_type<kQ8_0>(a, cu_count, stream);
-    case kQ4_K: return launch_type<kQ4_K>(a, cu_count, stream);
+    case kQ4_K:
+        if (gemv_use_mfma() && gemv_q4k_mfma_ok(a)) return gemv_q4k_mfma_launch(a, cu_count, stream);
+        return launch_type<kQ4_K>(a, cu_count, stream);
     case kQ5_K: return launch_type<kQ5_K>(a, cu_count, stream);
     case kQ6_K: return launch_type<kQ6_K>(a, cu_count, stream);
     default: return hipErrorInvalidValue;
