@@ -109,6 +109,7 @@ int orin_fa_init(int device) {
     g_state.cu_count = prop.multiProcessorCount;
     if ((e = prefill_allow_lds()) != hipSuccess) return hip_code(e);
     if ((e = decode_allow_lds()) != hipSuccess) return hip_code(e);
+    if ((e = gemv_mfma_allow_lds()) != hipSuccess) return hip_code(e);
     // The library's own workspace lives on the device it was last initialised for: a second init
     // on another device moves it there (the old block is released; graphs captured with it must
     // not be replayed any more, as after any change of workspace).

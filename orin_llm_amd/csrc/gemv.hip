@@ -496,13 +496,12 @@ hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
     if (a.row_bytes == 0 || a.n_in % 32 != 0 || a.n_seg < 1 || a.n_seg > 3) return hipErrorInvalidValue;
     if (a.wgs_per_cu < 1) a.wgs_per_cu = gemv_wgs_per_cu();
     a.mfma_wgs_per_cu = gemv_mfma_wgs_per_cu();
+    if (gemv_use_mfma() && gemv_mfma_ok(type, a)) return gemv_mfma_launch(type, a, cu_count, stream);
     switch (type) {
     case kF32: return launch_type<kF32>(a, cu_count, stream);
     case kF16: return launch_type<kF16>(a, cu_count, stream);
     case kQ8_0: return launch_type<kQ8_0>(a, cu_count, stream);
-    case kQ4_K:
-        if (gemv_use_mfma() && gemv_q4k_mfma_ok(a)) return gemv_q4k_mfma_launch(a, cu_count, stream);
-        return launch_type<kQ4_K>(a, cu_count, stream);
+    case kQ4_K: return launch_type<kQ4_K>(a, cu_count, stream);
     case kQ5_K: return launch_type<kQ5_K>(a, cu_count, stream);
     case kQ6_K: return launch_type<kQ6_K>(a, cu_count, stream);
     default: return hipErrorInvalidValue;

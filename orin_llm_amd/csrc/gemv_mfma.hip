@@ -1,44 +1,54 @@
-// Matrix-vector products over Q4_K weight rows on the matrix cores of gfx950 (MI355X).
+// Matrix-vector products over Q4_K and Q6_K weight rows on the matrix cores of gfx950 (MI355X).
 //
 // The vector-ALU kernel of gemv.hip spends about three instructions per weight (byte to float,
 // multiply-add, unpacking) and is bound by them at twice the time HBM needs for the bytes.  Here
-// the multiply-adds run as integer matrix instructions and the vector ALU only splits nibbles and
-// applies the blocks' scales:
+// the multiply-adds run as integer matrix instructions and the vector ALU only assembles the
+// weights' bytes and applies the blocks' scales:
 //
-//   * The activation is cut, per 32-element sub-block, into three signed 8-bit digits of a 24-bit
-//     integer, x = s (65536 d0 + 256 d1 + d2) with s = max|x| / (2^23 - 2^16): what the reference
-//     does with one digit (quantize_q8_1_k, reference: src/kernels.cu:136-157), carried to the
-//     precision of an fp32 mantissa.  Every workgroup builds the digits once, in LDS (together
-//     with the RMS norm, when that is folded in), with the sub-blocks' scales and sums beside them.
-//   * v_mfma_i32_16x16x64_i8 then multiplies 16 weight rows by 64 elements at a time: the weights'
-//     nibbles, widened to bytes, are the B operand exactly as a lane loaded them (lane (n, g) holds
-//     16 bytes of row n), and the A operand's rows are (sub-block, digit) pairs, each row zero
-//     outside its own sub-block.  One accumulator therefore holds, for a row of weights, the exact
-//     integer sums of four sub-blocks against the three digits, already separated: lane (n, g)
-//     receives the three sums of sub-block g.  They are recombined in fp32 and multiplied by the
-//     sub-block's scales, d * scale * sum - dmin * min * sum(x) (reference CPU statement:
-//     src/model_cpu.cpp:70-89).
+//   * The activation is cut, per sub-block of the weight format (32 elements for Q4_K, 16 for
+//     Q6_K), into three signed 8-bit digits of a 24-bit integer, x = s (65536 d0 + 256 d1 + d2)
+//     with s = max|x| / (2^23 - 2^16): what the reference does with one digit (quantize_q8_1_k,
+//     reference: src/kernels.cu:136-157), carried to the precision of an fp32 mantissa.  Every
+//     workgroup builds the digits once, in LDS (together with the RMS norm, when that is folded
+//     in), with the sub-blocks' scales and sums beside them.
+//   * v_mfma_i32_16x16x64_i8 then multiplies 16 weight rows by 64 elements at a time: the weights,
+//     widened to bytes, are the B operand (lane (n, g) holds 16 elements of row n), and the A
+//     operand's rows are (sub-block, digit) pairs, each row zero outside its own sub-block.  An
+//     accumulator therefore holds, for a row of weights, the exact integer sums of four sub-blocks
+//     against the three digits, already separated: lane (n, g) receives the three sums of
+//     sub-block g.  They are recombined in fp32 and multiplied by the sub-block's scales:
+//     d * scale * sum - dmin * min * sum(x) for Q4_K, d * scale * (sum - 32 sum(x)) for Q6_K
+//     (reference CPU statements: src/model_cpu.cpp:70-89, 115-142).
+//   * Loads are made with four neighbouring lanes on 64 consecutive bytes of a row (lane = 4 * row +
+//     piece: the vector cache then sees 16 runs per instruction; with the matrix instruction's own
+//     lane order, lane = row + 16 * piece, it sees 64 separate 16-byte requests and the kernel runs
+//     10 % slower) and moved to the matrix instruction's lanes by one lane permutation per register.
 //   * The four waves of a workgroup take every fourth 256-element block of the same 16 rows and meet
-//     in LDS at the end; blocks are requested one iteration ahead.
+//     in LDS at the end; blocks are requested one iteration ahead, across row tiles.
 #include "layer_common.hpp"
 
 namespace orin_fa {
 namespace {
 
-constexpr int kWaves = 4;
+constexpr int kMaxWaves = 8; // waves per workgroup: 4, or 8 where a matrix has few 16-row tiles and long rows
 constexpr float kDigitRange = 8388608.0f - 65536.0f; // largest |integer| the three signed digits hold
 
 struct XPair {
-    float scale, sum; // of one 32-element sub-block of the activation
+    float scale, sum; // of one sub-block of the activation
 };
 
-// LDS: digit planes [3][n_in] | XPair [n_in / 32] | 16 zero bytes | partial row sums [waves][M][16]
-__device__ __forceinline__ int lds_pairs_off(int n_in) { return 3 * n_in; }
-__device__ __forceinline__ int lds_zero_off(int n_in) { return 3 * n_in + (n_in >> 5) * 8; }
-__device__ __forceinline__ int lds_red_off(int n_in) { return lds_zero_off(n_in) + 16; }
+// LDS: digit planes [3][n_in] | XPair [n_in / G] | 16 zero bytes | partial row sums [kMaxWaves][2][16]
+template <int G>
+struct Lds {
+    static __host__ __device__ int pairs_off(int n_in) { return 3 * n_in; }
+    static __host__ __device__ int zero_off(int n_in) { return 3 * n_in + n_in / G * 8; }
+    static __host__ __device__ int red_off(int n_in) { return zero_off(n_in) + 16; }
+    static __host__ __device__ size_t bytes(int n_in) { return (size_t)red_off(n_in) + kMaxWaves * 2 * 16 * 4; }
+};
 
-// Digits of the (optionally normalised) activation into LDS.  Thread t takes elements 8 t .. 8 t + 7
-// of every 2048; the four threads of a sub-block meet by DPP moves inside their quad.
+// Digits of the (optionally normalised) activation into LDS, in groups of G elements.  Thread t takes
+// elements 8 t .. 8 t + 7 of every 2048; the G / 8 threads of a group meet by DPP moves inside their quad.
+template <int G, int kWaves>
 __device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red) {
     const int n_in = a.n_in, tid = threadIdx.x;
     float rinv = 1.0f;
@@ -51,11 +61,13 @@ __device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red)
         ss = wave_sum(ss);
         if ((tid & 63) == 0) red[tid >> 6] = ss;
         __syncthreads();
-        ss = red[0] + red[1] + red[2] + red[3];
+        ss = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) ss += red[w];
         __syncthreads();
         rinv = 1.0f / sqrtf(ss / (float)n_in + a.eps);
     }
-    XPair* pairs = reinterpret_cast<XPair*>(smem + lds_pairs_off(n_in));
+    XPair* pairs = reinterpret_cast<XPair*>(smem + Lds<G>::pairs_off(n_in));
     for (int e = tid * 8; e < n_in; e += kWaves * 64 * 8) {
         float x[8];
         *reinterpret_cast<float4*>(x) = *reinterpret_cast<const float4*>(a.x + e);
@@ -73,131 +85,230 @@ __device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red)
             mx = fmaxf(mx, fabsf(x[i]));
             sum += x[i];
         }
-        // the sub-block's four threads are one quad (n_in is a multiple of 32, so a quad is never split)
+        // a group's threads sit in one quad (n_in is a multiple of 32, so a quad is never split)
         mx = fmaxf(mx, dpp_xor_step(mx, 0));
-        mx = fmaxf(mx, dpp_xor_step(mx, 1));
         sum += dpp_xor_step(sum, 0);
-        sum += dpp_xor_step(sum, 1);
+        if constexpr (G == 32) {
+            mx = fmaxf(mx, dpp_xor_step(mx, 1));
+            sum += dpp_xor_step(sum, 1);
+        }
         const float scale = mx > 0.0f ? mx / kDigitRange : 1.0f;
         const float inv = 1.0f / scale;
-        unsigned d0[2] = {0, 0}, d1[2] = {0, 0}, d2[2] = {0, 0};
+        // X + 0x808080 carries 128 into each of the three byte positions, so its bytes are the signed
+        // digits plus 128 (byte k of X + 0x808080 is ((X >> 8 k) + 128) & 255 with the lower digits'
+        // carries already taken out); the exclusive-or takes the 128 off again, byte by byte.
+        unsigned z[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int X = (int)rintf(x[i] * inv);
-            const int lo = ((X + 128) & 255) - 128;
-            const int X1 = (X - lo) >> 8;
-            const int mid = ((X1 + 128) & 255) - 128;
-            const int hi = (X1 - mid) >> 8;
-            d0[i >> 2] |= (unsigned)(hi & 255) << (8 * (i & 3));
-            d1[i >> 2] |= (unsigned)(mid & 255) << (8 * (i & 3));
-            d2[i >> 2] |= (unsigned)(lo & 255) << (8 * (i & 3));
+        for (int i = 0; i < 8; ++i) z[i] = ((unsigned)((int)rintf(x[i] * inv)) + 0x808080u) ^ 0x808080u;
+        // byte k of four consecutive elements into one word of plane 2 - k (plane 0 holds the top digits)
+        u32x2 plane[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const unsigned pick = (unsigned)k | ((unsigned)(4 + k) << 8); // byte k of the second operand, then of the first
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                const unsigned t01 = __builtin_amdgcn_perm(z[4 * w + 1], z[4 * w + 0], pick);
+                const unsigned t23 = __builtin_amdgcn_perm(z[4 * w + 3], z[4 * w + 2], pick);
+                plane[2 - k][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+            }
         }
-        *reinterpret_cast<u32x2*>(smem + e) = u32x2{d0[0], d0[1]};
-        *reinterpret_cast<u32x2*>(smem + n_in + e) = u32x2{d1[0], d1[1]};
-        *reinterpret_cast<u32x2*>(smem + 2 * n_in + e) = u32x2{d2[0], d2[1]};
-        if ((tid & 3) == 0) pairs[e >> 5] = XPair{scale, sum};
+        *reinterpret_cast<u32x2*>(smem + e) = plane[0];
+        *reinterpret_cast<u32x2*>(smem + n_in + e) = plane[1];
+        *reinterpret_cast<u32x2*>(smem + 2 * n_in + e) = plane[2];
+        if ((tid & (G / 8 - 1)) == 0) pairs[e / G] = XPair{scale, sum};
     }
-    if (tid < 4) reinterpret_cast<unsigned*>(smem + lds_zero_off(n_in))[tid] = 0u;
+    if (tid < 4) reinterpret_cast<unsigned*>(smem + Lds<G>::zero_off(n_in))[tid] = 0u;
     __syncthreads();
 }
 
-struct Q4Raw {
-    u32x4 hdr, q1, q2; // a block's header and this lane's 16 bytes of each half of its nibbles
+__device__ __forceinline__ float half_of(unsigned bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
+__device__ __forceinline__ unsigned from_lane(int src_lane4, unsigned v) {
+    return (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)v);
+}
+__device__ __forceinline__ float digits_sum(const i32x4& acc) {
+    return ((float)acc[0] * 256.0f + (float)acc[1]) * 256.0f + (float)acc[2];
+}
+
+// What a lane needs to know of itself: as a loader (row ln of the tile, 16-byte piece lg), as a lane of
+// the matrix instruction (weight row / column n, element group g; the loader of its data is lane
+// 4 n + g, whose piece is g as well), and as a lane of the A operand (accumulator row am = 4 p + digit).
+struct LaneCtx {
+    int n, g, ln, lg, src_lane4, am;
+    const unsigned char* smem;
+    const XPair* pairs;
+    int n_in, zero_off;
 };
 
-// DUAL: two matrices (gate, up) and SiLU(gate) * up.  Grid: (workgroups, matrices); a workgroup walks the
-// 16-row tiles blockIdx.x, + gridDim.x, ...
-template <bool DUAL>
-__global__ __launch_bounds__(kWaves * 64) void gemv_q4k_mfma_kernel(const GemvArgs a) {
+template <int T>
+struct MF;
+
+// Q4_K (reference: src/quant.h:14-21): per 128-element half of a block, the lane's 16 bytes of nibbles
+// are 16 elements of sub-block 2 (g / 2) (low nibbles) and of 2 (g / 2) + 1 (high nibbles); the two
+// matrix instructions of a half add into one accumulator whose row group p is sub-block p of the half.
+template <>
+struct MF<kQ4_K> {
+    static constexpr int kGroup = 32, kBlockBytes = 144;
+    struct Raw {
+        u32x4 hdr, q1, q2; // a block's header and this lane's 16 bytes of each half of its nibbles
+    };
+    struct Addr {
+        int lo_base, hi_base, lo_step, hi_step; // LDS byte offsets of this lane's A operands; a lane whose row is zero reads the 16 zero bytes, stride 0
+    };
+    static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
+        r.hdr = *reinterpret_cast<const u32x4*>(blk);
+        r.q1 = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * lg);
+        r.q2 = *reinterpret_cast<const u32x4*>(blk + 80 + 16 * lg);
+    }
+    static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
+        const int ap = c.am >> 2, ad = c.am & 3, g = c.g;
+        const bool live = ad < 3 && (ap >> 1) == (g >> 1);
+        const int elem = 64 * (g >> 1) + 16 * (g & 1);
+        const bool lo = live && (ap & 1) == 0, hi = live && (ap & 1) == 1;
+        return Addr{lo ? ad * c.n_in + elem : c.zero_off, hi ? ad * c.n_in + elem + 32 : c.zero_off, lo ? 256 : 0, hi ? 256 : 0};
+    }
+    static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
+        // (the loading lane holds piece lg of its row, and lane (n, g) wants piece g of row n: the bytes of
+        // the packed pairs it needs are bytes lg of the loading lane's three words)
+        const unsigned mine = ((r.hdr.y >> (8 * c.lg)) & 0xffu) | (((r.hdr.z >> (8 * c.lg)) & 0xffu) << 8) |
+                              (((r.hdr.w >> (8 * c.lg)) & 0xffu) << 16);
+        const unsigned dd = from_lane(c.src_lane4, r.hdr.x), bb = from_lane(c.src_lane4, mine);
+        const float d = half_of(dd & 0xffffu), dmin = half_of(dd >> 16);
+        const unsigned b0 = bb & 0xffu, b1 = (bb >> 8) & 0xffu, b2 = (bb >> 16) & 0xffu;
+        // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
+        const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
+        const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
+        float out = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + ad.lo_base + b * ad.lo_step + (ad.lo_step ? 128 * h : 0));
+            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + ad.hi_base + b * ad.hi_step + (ad.hi_step ? 128 * h : 0));
+            const XPair xp = c.pairs[8 * b + 4 * h + c.g];
+            const u32x4 qs = h ? r.q2 : r.q1;
+            i32x4 lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const unsigned q = from_lane(c.src_lane4, qs[i]);
+                lo[i] = (int)(q & 0x0f0f0f0fu);
+                hi[i] = (int)((q >> 4) & 0x0f0f0f0fu);
+            }
+            i32x4 acc = {0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, lo, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, hi, acc, 0, 0, 0);
+            out += (d * sc[h]) * (digits_sum(acc) * xp.scale) - (dmin * mn[h]) * xp.sum;
+        }
+        return out;
+    }
+};
+
+// Q6_K (reference: src/quant.h:34-40; blocks of 210 bytes, 2-byte aligned): per 128-element half, piece g
+// of the half's 64 low-nibble bytes holds sub-block g (elements 16 g .. 16 g + 15 of the half) in its low
+// nibbles and sub-block 4 + g in its high nibbles; their high bit pairs sit in high byte 16 (g & 1) + i at
+// bits 2 (g / 2) and 4 + 2 (g / 2).  One matrix instruction and one accumulator per nibble; the element
+// group g of the instruction is sub-block g (or 4 + g), so the A operand's row group p is live in group p.
+template <>
+struct MF<kQ6_K> {
+    static constexpr int kGroup = 16, kBlockBytes = 210;
+    struct Raw {
+        u32x4 ql[2], qh[2], sc;
+        unsigned d;
+    };
+    struct Addr {
+        int base, step;
+    };
+    template <typename V>
+    struct __attribute__((packed, aligned(2))) Loose {
+        V v;
+    };
+    static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            r.ql[h] = reinterpret_cast<const Loose<u32x4>*>(blk + 64 * h + 16 * lg)->v;
+            r.qh[h] = reinterpret_cast<const Loose<u32x4>*>(blk + 128 + 32 * h + 16 * (lg & 1))->v;
+        }
+        r.sc = reinterpret_cast<const Loose<u32x4>*>(blk + 192)->v;
+        r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
+    }
+    static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
+        const int ap = c.am >> 2, ad = c.am & 3;
+        const bool live = ad < 3 && ap == c.g;
+        return Addr{live ? ad * c.n_in + 16 * c.g : c.zero_off, live ? 1 : 0};
+    }
+    static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
+        // scales 8 h + g and 8 h + 4 + g of both halves: byte lg of each of the loading lane's four words
+        const unsigned mine = ((r.sc.x >> (8 * c.lg)) & 0xffu) | (((r.sc.y >> (8 * c.lg)) & 0xffu) << 8) |
+                              (((r.sc.z >> (8 * c.lg)) & 0xffu) << 16) | (((r.sc.w >> (8 * c.lg)) & 0xffu) << 24);
+        const unsigned ss = from_lane(c.src_lane4, mine);
+        const float d = half_of(from_lane(c.src_lane4, r.d));
+        const int s1 = 2 * (c.g >> 1);
+        float out = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int off = ad.step ? 256 * b + 128 * h : 0;
+            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + ad.base + off);
+            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + ad.base + off + (ad.step ? 64 : 0));
+            const XPair xlo = c.pairs[16 * b + 8 * h + c.g], xhi = c.pairs[16 * b + 8 * h + 4 + c.g];
+            i32x4 lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const unsigned l = from_lane(c.src_lane4, r.ql[h][i]), u = from_lane(c.src_lane4, r.qh[h][i]) >> s1;
+                lo[i] = (int)((l & 0x0f0f0f0fu) | ((u & 0x03030303u) << 4));
+                hi[i] = (int)(((l >> 4) & 0x0f0f0f0fu) | (((u >> 4) & 0x03030303u) << 4));
+            }
+            const i32x4 zero = {0, 0, 0, 0};
+            const i32x4 acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, lo, zero, 0, 0, 0);
+            const i32x4 acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, hi, zero, 0, 0, 0);
+            const float sc_lo = (float)((int)(ss << (24 - 16 * h)) >> 24), sc_hi = (float)((int)(ss << (16 - 16 * h)) >> 24);
+            out += (d * sc_lo) * (digits_sum(acc_lo) * xlo.scale - 32.0f * xlo.sum) +
+                   (d * sc_hi) * (digits_sum(acc_hi) * xhi.scale - 32.0f * xhi.sum);
+        }
+        return out;
+    }
+};
+
+// T: weight type.  DUAL: two matrices (gate, up) and SiLU(gate) * up.  Grid: (workgroups, matrices); a
+// workgroup walks the 16-row tiles blockIdx.x, + gridDim.x, ...
+template <int T, bool DUAL, int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a) {
+    using F = MF<T>;
+    using L = Lds<F::kGroup>;
+    typedef typename F::Raw Raw;
     constexpr int M = DUAL ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int n_in = a.n_in, nb = n_in >> 8;
-    float* const red = reinterpret_cast<float*>(smem + lds_red_off(n_in));
+    float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
     const GemvSeg seg = a.seg[blockIdx.y];
     const int n_tiles = (seg.n_out + 15) >> 4;
     if ((int)blockIdx.x >= n_tiles) return; // (whole workgroup: a shorter matrix of a shared launch)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n = lane & 15, g = lane >> 4;
+    LaneCtx c;
+    c.n = lane & 15; c.g = lane >> 4; c.ln = lane >> 2; c.lg = lane & 3;
+    c.src_lane4 = 4 * (4 * c.n + c.g);
+    c.am = lane & 15;
+    c.smem = smem;
+    c.pairs = reinterpret_cast<const XPair*>(smem + L::pairs_off(n_in));
+    c.n_in = n_in;
+    c.zero_off = L::zero_off(n_in);
     const unsigned char* const wbase[2] = {static_cast<const unsigned char*>(seg.w),
                                            static_cast<const unsigned char*>(DUAL ? a.w_up : seg.w)};
     // (rows past the end repeat the last one; nothing is written for them.  Blocks past a row's end: the
     // last block once more, never used.)
-    // Loads are made with four neighbouring lanes on 64 consecutive bytes of a row (lane = 4 * row + piece:
-    // the vector cache then sees 16 runs per instruction; with the matrix instruction's own lane order,
-    // lane = row + 16 * piece, it sees 64 separate 16-byte requests and the kernel runs 10 % slower) and
-    // moved to the matrix instruction's lanes by one lane permutation per register afterwards.
-    const int ln = lane >> 2, lg = lane & 3;
-    const int src_lane4 = 4 * (4 * n + g); // (byte address of the lane that loaded what lane (n, g) multiplies)
-    auto request = [&](Q4Raw (&r)[M], int tile, int b) {
-        const int row = min(tile * 16 + ln, seg.n_out - 1);
+    auto request = [&](Raw (&r)[M], int tile, int b) {
+        const int row = min(tile * 16 + c.ln, seg.n_out - 1);
         b = min(b, nb - 1);
 #pragma unroll
-        for (int m = 0; m < M; ++m) {
-            const unsigned char* blk = wbase[m] + (size_t)row * a.row_bytes + (size_t)b * 144;
-            r[m].hdr = *reinterpret_cast<const u32x4*>(blk);
-            r[m].q1 = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * lg);
-            r[m].q2 = *reinterpret_cast<const u32x4*>(blk + 80 + 16 * lg);
-        }
+        for (int m = 0; m < M; ++m) F::load(wbase[m] + (size_t)row * a.row_bytes + (size_t)b * F::kBlockBytes, c.lg, r[m]);
     };
-    Q4Raw raw_a[M], raw_b[M];
+    Raw raw_a[M], raw_b[M];
     request(raw_a, blockIdx.x, wave);
     __builtin_amdgcn_sched_barrier(0);
 
-    stage_digits(a, smem, red);
+    stage_digits<F::kGroup, kWaves>(a, smem, red);
 
-    // As a lane of the A operand: row m = 4 p + digit of an accumulator covers sub-block p of the four
-    // that a 128-element half of a block holds; this lane's 16 elements belong to sub-block
-    // 2 (g / 2) (their low nibbles) and 2 (g / 2) + 1 (their high nibbles).
-    const int am = lane & 15, ap = am >> 2, ad = am & 3;
-    const bool a_live = ad < 3 && (ap >> 1) == (g >> 1);
-    const int zero_off = lds_zero_off(n_in);
-    // (byte offsets into LDS; lanes whose row is zero here read the 16 zero bytes, with stride 0)
-    const int a_elem = 64 * (g >> 1) + 16 * (g & 1);
-    const int a_lo_base = a_live && (ap & 1) == 0 ? ad * n_in + a_elem : zero_off;
-    const int a_hi_base = a_live && (ap & 1) == 1 ? ad * n_in + a_elem + 32 : zero_off;
-    const int a_lo_step = a_live && (ap & 1) == 0 ? 256 : 0, a_hi_step = a_live && (ap & 1) == 1 ? 256 : 0;
-    const XPair* const pairs = reinterpret_cast<const XPair*>(smem + lds_pairs_off(n_in));
-
+    const typename F::Addr addr = F::addr(c);
     float rowacc[M];
-    auto finish = [&](const Q4Raw (&r)[M], int b) {
-        i32x4 alo[2], ahi[2];
+    auto finish = [&](const Raw (&r)[M], int b) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            alo[h] = *reinterpret_cast<const i32x4*>(smem + a_lo_base + b * a_lo_step + (a_lo_step ? 128 * h : 0));
-            ahi[h] = *reinterpret_cast<const i32x4*>(smem + a_hi_base + b * a_hi_step + (a_hi_step ? 128 * h : 0));
-        }
-        const XPair xp[2] = {pairs[8 * b + g], pairs[8 * b + 4 + g]};
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-            // (the loading lane holds piece lg of row ln, and lane (n, g) wants piece g of row n: the bytes
-            // of the packed pairs it needs are bytes lg of the loading lane's three words)
-            const unsigned mine = ((r[m].hdr.y >> (8 * lg)) & 0xffu) | (((r[m].hdr.z >> (8 * lg)) & 0xffu) << 8) |
-                                  (((r[m].hdr.w >> (8 * lg)) & 0xffu) << 16);
-            const unsigned dd = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)r[m].hdr.x);
-            const unsigned bb = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)mine);
-            const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(dd & 0xffffu));
-            const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(dd >> 16));
-            const unsigned b0 = bb & 0xffu, b1 = (bb >> 8) & 0xffu, b2 = (bb >> 16) & 0xffu;
-            // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
-            const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
-            const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const u32x4 qs = h ? r[m].q2 : r[m].q1;
-                i32x4 lo, hi;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const unsigned q = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)qs[i]);
-                    lo[i] = (int)(q & 0x0f0f0f0fu);
-                    hi[i] = (int)((q >> 4) & 0x0f0f0f0fu);
-                }
-                i32x4 acc = {0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo[h], lo, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi[h], hi, acc, 0, 0, 0);
-                const float t = ((float)acc[0] * 256.0f + (float)acc[1]) * 256.0f + (float)acc[2];
-                rowacc[m] += (d * sc[h]) * (t * xp[h].scale) - (dmin * mn[h]) * xp[h].sum;
-            }
-        }
+        for (int m = 0; m < M; ++m) rowacc[m] += F::block(r[m], c, addr, b);
     };
     // Row tiles blockIdx.x, + gridDim.x, ...: the digits are staged once per workgroup.  The first block of
     // the next tile is requested while the last of this one is multiplied out.
@@ -225,7 +336,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4k_mfma_kernel(const GemvAr
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const float t = xor_sum(rowacc[m]);
-            if (g == 0) red[(wave * M + m) * 16 + n] = t;
+            if (c.g == 0) red[(wave * M + m) * 16 + c.n] = t;
         }
         __syncthreads();
         if (threadIdx.x < 16 && row0 + (int)threadIdx.x < seg.n_out) {
@@ -247,24 +358,60 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_q4k_mfma_kernel(const GemvAr
     }
 }
 
-} // namespace
+constexpr size_t kMfmaLdsMax = 96u * 1024u;
 
-bool gemv_q4k_mfma_ok(const GemvArgs& a) {
-    const size_t lds = 3u * a.n_in + (a.n_in / 32) * 8u + 16u + kWaves * 2 * 16 * 4u;
-    return a.n_in % 256 == 0 && lds <= 64u * 1024u;
-}
+template <int T>
+size_t lds_bytes(int n_in) { return Lds<MF<T>::kGroup>::bytes(n_in); }
 
-hipError_t gemv_q4k_mfma_launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
+template <int T>
+hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     int max_out = 0;
     for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
     const int cap = a.mfma_wgs_per_cu > 0 ? cu_count * a.mfma_wgs_per_cu : (max_out + 15) / 16;
     const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
-    const size_t lds = 3u * a.n_in + (a.n_in / 32) * 8u + 16u + kWaves * 2 * 16 * 4u;
-    if (a.w_up)
-        hipLaunchKernelGGL((gemv_q4k_mfma_kernel<true>), grid, dim3(kWaves * 64), lds, stream, a);
-    else
-        hipLaunchKernelGGL((gemv_q4k_mfma_kernel<false>), grid, dim3(kWaves * 64), lds, stream, a);
+    // Eight waves a workgroup where the tiles would not give every SIMD a second wave and a row has the
+    // blocks to share out (a down projection: few rows, long ones).
+    const bool wide = (int)(grid.x * grid.y) <= cu_count && a.n_in / 256 >= 16;
+    const size_t lds = lds_bytes<T>(a.n_in);
+    if (a.w_up) {
+        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 8>), grid, dim3(512), lds, stream, a);
+        else hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 4>), grid, dim3(256), lds, stream, a);
+    } else {
+        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 8>), grid, dim3(512), lds, stream, a);
+        else hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 4>), grid, dim3(256), lds, stream, a);
+    }
     return hipGetLastError();
+}
+
+template <int T, bool DUAL>
+hipError_t allow() {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel<T, DUAL, 4>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel<T, DUAL, 8>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+}
+
+} // namespace
+
+bool gemv_mfma_ok(int type, const GemvArgs& a) {
+    if (a.n_in % 256 != 0) return false;
+    if (type == kQ4_K) return lds_bytes<kQ4_K>(a.n_in) <= kMfmaLdsMax;
+    if (type == kQ6_K) return lds_bytes<kQ6_K>(a.n_in) <= kMfmaLdsMax;
+    return false;
+}
+
+hipError_t gemv_mfma_launch(int type, const GemvArgs& a, int cu_count, hipStream_t stream) {
+    return type == kQ4_K ? launch<kQ4_K>(a, cu_count, stream) : launch<kQ6_K>(a, cu_count, stream);
+}
+
+// More than 64 KB of LDS per workgroup (rows longer than about 16k elements) needs to be allowed once.
+hipError_t gemv_mfma_allow_lds() {
+    hipError_t e;
+    if ((e = allow<kQ4_K, false>()) != hipSuccess) return e;
+    if ((e = allow<kQ4_K, true>()) != hipSuccess) return e;
+    if ((e = allow<kQ6_K, false>()) != hipSuccess) return e;
+    return allow<kQ6_K, true>();
 }
 
 } // namespace orin_fa

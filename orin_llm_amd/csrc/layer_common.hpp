@@ -36,9 +36,11 @@ struct GemvArgs {
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
 int weight_align(int type);               // alignment the kernels need of a matrix's base address
 hipError_t gemv_launch(int type, GemvArgs args, int cu_count, hipStream_t stream);
-// Q4_K on the matrix cores (gemv_mfma.hip): whether the shape fits, and the launch.
-bool gemv_q4k_mfma_ok(const GemvArgs& args);
-hipError_t gemv_q4k_mfma_launch(const GemvArgs& args, int cu_count, hipStream_t stream);
+// Q4_K and Q6_K on the matrix cores (gemv_mfma.hip): whether type and shape fit, the launch, and the once-only
+// permission for large LDS blocks.
+bool gemv_mfma_ok(int type, const GemvArgs& args);
+hipError_t gemv_mfma_launch(int type, const GemvArgs& args, int cu_count, hipStream_t stream);
+hipError_t gemv_mfma_allow_lds();
 
 hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream);
 hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream);
