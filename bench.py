@@ -1047,8 +1047,8 @@ def random_weight(torch, gen, wtype, n_in, n_out, std=0.03):
 
 
 def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
-    """One step = one token through every layer of the model: orin_decode_layer per layer (six or seven
-    launches: norm + q/k/v projections, rotary embedding + cache store + attention, output projection,
+    """One step = one token through every layer of the model: orin_decode_layer per layer (six launches:
+    norm + q/k/v projections, rotary embedding + cache store + attention, output projection,
     norm + gate/up + SwiGLU, down projection), replayed as one HIP graph as the reference replays its decode
     step (src/model_gpu.cu:295-344).  value = HBM bytes the layer must read (its weights once, its cache
     once) per second."""
@@ -1106,9 +1106,9 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
     Lw, k0, v0 = model[0]
     launches = {
-        "norm + q,k (one launch)": lambda: ly.gemv_multi(Q4, [Lw["wq"][1], Lw["wk"][1]], [Lw.get("bq"), Lw.get("bk")], [bufs["q"], bufs["k"]],
-                                                         [H * d, G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
-        "norm + v": lambda: ly.gemv_multi(Q6, [Lw["wv"][1]], [Lw.get("bv")], [bufs["v"]], [G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
+        "norm + q,k,v (one launch)": lambda: ly.gemv_multi_types([Q4, Q4, Q6], [Lw["wq"][1], Lw["wk"][1], Lw["wv"][1]],
+                                                                  [Lw.get("bq"), Lw.get("bk"), Lw.get("bv")], [bufs["q"], bufs["k"], bufs["v"]],
+                                                                  [H * d, G * d, G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
         "rope + store + attention (two launches)": lambda: kernels.flash_attention_decode_rope_store_ind(
             bufs["q"], bufs["k"], bufs["v"], k0, v0, bufs["attn"], H, G, d, n_ctx, dpos, float(1.0 / np.sqrt(d)), d, s["theta"],
             None, bool(s["neox"]), angles),
@@ -1117,7 +1117,7 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
                                                                       bufs["act"], ne, nff),
         "down projection (+=)": lambda: ly.gemv_multi(Q6, [Lw["ffn_down"][1]], None, [bufs["x"]], [ne], bufs["act"], None, 0.0, nff, True),
     }
-    launch_bytes = {"norm + q,k (one launch)": ly.row_bytes(Q4, ne) * (H + G) * d, "norm + v": ly.row_bytes(Q6, ne) * G * d,
+    launch_bytes = {"norm + q,k,v (one launch)": ly.row_bytes(Q4, ne) * (H + G) * d + ly.row_bytes(Q6, ne) * G * d,
                     "rope + store + attention (two launches)": kv_bytes, "output projection (+=)": ly.row_bytes(Q4, H * d) * ne,
                     "norm + gate/up + SwiGLU": 2 * ly.row_bytes(Q4, ne) * nff, "down projection (+=)": ly.row_bytes(Q6, nff) * ne}
     launch_us = {}

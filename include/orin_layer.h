@@ -80,6 +80,11 @@ int orin_swiglu(float* act, const float* gate, const float* up, int n);
 int orin_gemv_multi(int type, int n_mat, const void* const* W, const float* const* bias, float* const* y,
                     const int* n_out, const float* x, const float* norm_w, float eps, int n_in, int accumulate);
 
+/* The same with a type per matrix (a file that keeps attn_v in Q6_K beside Q4_K projections): one launch
+ * where every type is Q4_K or Q6_K, one launch per matrix otherwise. */
+int orin_gemv_multi_types(const int* types, int n_mat, const void* const* W, const float* const* bias, float* const* y,
+                          const int* n_out, const float* x, const float* norm_w, float eps, int n_in);
+
 /* out[i] = silu(Wg[i] . norm(x)) * (Wu[i] . norm(x)): the layer's second norm and its gate/up pair in
  * one launch. */
 int orin_gemv_norm_gate_up_swiglu(int type, const void* Wg, const void* Wu, const float* x, const float* norm_w,

@@ -508,4 +508,16 @@ hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
     }
 }
 
+// Matrices of different types over one activation: one launch when every one of them is Q4_K or Q6_K and the
+// matrix-core kernel takes the shape; hipErrorNotSupported otherwise (the caller then launches them one by one).
+hipError_t gemv_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) {
+    if (!gemv_use_mfma() || a.w_up || a.n_seg < 1 || a.n_seg > 3) return hipErrorNotSupported;
+    for (int i = 0; i < a.n_seg; ++i) {
+        if (!gemv_mfma_ok(a.seg[i].type, a)) return hipErrorNotSupported;
+        a.seg[i].row_bytes = weight_row_bytes(a.seg[i].type, a.n_in);
+    }
+    a.mfma_wgs_per_cu = gemv_mfma_wgs_per_cu();
+    return gemv_mfma_mixed_launch(a, cu_count, stream);
+}
+
 } // namespace orin_fa

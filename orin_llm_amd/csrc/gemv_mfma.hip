@@ -268,7 +268,7 @@ struct MF<kQ6_K> {
 // T: weight type.  DUAL: two matrices (gate, up) and SiLU(gate) * up.  Grid: (workgroups, matrices); a
 // workgroup walks the 16-row tiles blockIdx.x, + gridDim.x, ...
 template <int T, bool DUAL, int kWaves>
-__global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a) {
+__device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
     using F = MF<T>;
     using L = Lds<F::kGroup>;
     typedef typename F::Raw Raw;
@@ -277,6 +277,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
     const int n_in = a.n_in, nb = n_in >> 8;
     float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
     const GemvSeg seg = a.seg[blockIdx.y];
+    const size_t row_bytes = a.n_seg_types ? seg.row_bytes : a.row_bytes;
     const int n_tiles = (seg.n_out + 15) >> 4;
     if ((int)blockIdx.x >= n_tiles) return; // (whole workgroup: a shorter matrix of a shared launch)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
         const int row = min(tile * 16 + c.ln, seg.n_out - 1);
         b = min(b, nb - 1);
 #pragma unroll
-        for (int m = 0; m < M; ++m) F::load(wbase[m] + (size_t)row * a.row_bytes + (size_t)b * F::kBlockBytes, c.lg, r[m]);
+        for (int m = 0; m < M; ++m) F::load(wbase[m] + (size_t)row * row_bytes + (size_t)b * F::kBlockBytes, c.lg, r[m]);
     };
     Raw raw_a[M], raw_b[M];
     request(raw_a, blockIdx.x, wave);
@@ -358,6 +359,19 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
     }
 }
 
+template <int T, bool DUAL, int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a) {
+    gemv_mfma_body<T, DUAL, kWaves>(a);
+}
+
+// Matrices of both types in one launch (the q, k, v projections of a file that keeps attn_v in Q6_K): a
+// workgroup belongs to one matrix and runs that matrix's code.
+template <int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void gemv_mfma_mixed_kernel(const GemvArgs a) {
+    if (a.seg[blockIdx.y].type == kQ4_K) gemv_mfma_body<kQ4_K, false, kWaves>(a);
+    else gemv_mfma_body<kQ6_K, false, kWaves>(a);
+}
+
 constexpr size_t kMfmaLdsMax = 96u * 1024u;
 
 template <int T>
@@ -394,6 +408,18 @@ hipError_t allow() {
 
 } // namespace
 
+// Every matrix Q4_K or Q6_K, each its own type (GemvSeg::type, row_bytes filled in by the caller).
+hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) {
+    int max_out = 0;
+    for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
+    const int cap = a.mfma_wgs_per_cu > 0 ? cu_count * a.mfma_wgs_per_cu : (max_out + 15) / 16;
+    const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
+    a.n_seg_types = 1;
+    const size_t lds = max(lds_bytes<kQ4_K>(a.n_in), lds_bytes<kQ6_K>(a.n_in));
+    hipLaunchKernelGGL((gemv_mfma_mixed_kernel<4>), grid, dim3(256), lds, stream, a);
+    return hipGetLastError();
+}
+
 bool gemv_mfma_ok(int type, const GemvArgs& a) {
     if (a.n_in % 256 != 0) return false;
     if (type == kQ4_K) return lds_bytes<kQ4_K>(a.n_in) <= kMfmaLdsMax;
@@ -411,7 +437,9 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow<kQ4_K, false>()) != hipSuccess) return e;
     if ((e = allow<kQ4_K, true>()) != hipSuccess) return e;
     if ((e = allow<kQ6_K, false>()) != hipSuccess) return e;
-    return allow<kQ6_K, true>();
+    if ((e = allow<kQ6_K, true>()) != hipSuccess) return e;
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }
 
 } // namespace orin_fa

@@ -36,7 +36,7 @@ int gemv_call(int type, int n_mat, const void* const* w, const float* const* bia
         const int rc = check_matrix(type, w[i], n_in, n_out[i]);
         if (rc != ORIN_FA_OK) return rc;
         if (!y[i]) return ORIN_FA_E_INVALID;
-        a.seg[i] = GemvSeg{w[i], bias ? bias[i] : nullptr, y[i], n_out[i]};
+        a.seg[i] = GemvSeg{w[i], bias ? bias[i] : nullptr, y[i], n_out[i], type, 0};
     }
     if (w_up) {
         if (n_mat != 1) return ORIN_FA_E_INVALID;
@@ -51,6 +51,29 @@ int gemv_call(int type, int n_mat, const void* const* w, const float* const* bia
     a.n_in = n_in;
     a.accumulate = accumulate;
     return hip_rc(gemv_launch(type, a, lib_cu_count() > 0 ? lib_cu_count() : 256, lib_stream()));
+}
+
+// One launch over matrices of different types, where the matrix-core kernel takes them all; otherwise
+// ORIN_FA_E_INVALID + 1 (not an error: the caller launches them type by type).
+constexpr int kNotMixed = 1;
+int gemv_call_mixed(const int* types, int n_mat, const void* const* w, const float* const* bias, float* const* y,
+                    const int* n_out, const float* x, const float* norm_w, float eps, int n_in) {
+    if (!lib_ready()) return ORIN_FA_E_NOT_INIT;
+    if (n_mat < 1 || n_mat > 3 || !x || !aligned(x, 16) || (norm_w && !aligned(norm_w, 16))) return ORIN_FA_E_INVALID;
+    GemvArgs a{};
+    for (int i = 0; i < n_mat; ++i) {
+        const int rc = check_matrix(types[i], w[i], n_in, n_out[i]);
+        if (rc != ORIN_FA_OK) return rc;
+        if (!y[i]) return ORIN_FA_E_INVALID;
+        a.seg[i] = GemvSeg{w[i], bias ? bias[i] : nullptr, y[i], n_out[i], types[i], 0};
+    }
+    a.n_seg = n_mat;
+    a.x = x;
+    a.norm_w = norm_w;
+    a.eps = eps;
+    a.n_in = n_in;
+    const hipError_t e = gemv_mixed_launch(a, lib_cu_count() > 0 ? lib_cu_count() : 256, lib_stream());
+    return e == hipErrorNotSupported ? kNotMixed : hip_rc(e);
 }
 
 int gemv_one(int type, const void* w, const float* bias, float* y, int n_out, const void* w_up, const float* x,
@@ -143,6 +166,18 @@ int orin_gemv_multi(int type, int n_mat, const void* const* W, const float* cons
     return gemv_call(type, n_mat, W, bias, y, n_out, nullptr, x, norm_w, eps, n_in, accumulate);
 }
 
+int orin_gemv_multi_types(const int* types, int n_mat, const void* const* W, const float* const* bias, float* const* y,
+                          const int* n_out, const float* x, const float* norm_w, float eps, int n_in) {
+    if (!types || !W || !y || !n_out) return ORIN_FA_E_INVALID;
+    int rc = gemv_call_mixed(types, n_mat, W, bias, y, n_out, x, norm_w, eps, n_in);
+    if (rc != kNotMixed) return rc;
+    for (int i = 0; i < n_mat; ++i) { // one launch per matrix
+        const float* bi = bias ? bias[i] : nullptr;
+        if ((rc = gemv_call(types[i], 1, &W[i], &bi, &y[i], &n_out[i], nullptr, x, norm_w, eps, n_in, 0)) != ORIN_FA_OK) return rc;
+    }
+    return ORIN_FA_OK;
+}
+
 int orin_gemv_norm_gate_up_swiglu(int type, const void* Wg, const void* Wu, const float* x, const float* norm_w,
                                   float eps, float* out, int n_in, int n_out) {
     if (!Wu) return ORIN_FA_E_INVALID;
@@ -163,6 +198,11 @@ int orin_decode_layer(const orin_decode_layer_desc* L) {
         float* y[3] = {L->q, L->k, L->v};
         const int n[3] = {nq, nkv, nkv}, t[3] = {L->wq_type, L->wk_type, L->wv_type};
         bool done[3] = {false, false, false};
+        if (t[0] != t[1] || t[1] != t[2]) { // (a file that keeps attn_v in Q6_K beside Q4_K: still one launch)
+            rc = gemv_call_mixed(t, 3, w, b, y, n, L->x, L->attn_norm, L->rms_eps, L->n_embd);
+            if (rc == ORIN_FA_OK) done[0] = done[1] = done[2] = true;
+            else if (rc != kNotMixed) return rc;
+        }
         for (int i = 0; i < 3; ++i) {
             if (done[i]) continue;
             const void* gw[3];

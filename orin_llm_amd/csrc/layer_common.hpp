@@ -17,6 +17,8 @@ struct GemvSeg {
     const float* bias; // or null
     float* y;
     int n_out;
+    int type;         // used by launches that mix types (n_seg_types != 0), with row_bytes
+    size_t row_bytes;
 };
 
 struct GemvArgs {
@@ -30,7 +32,7 @@ struct GemvArgs {
     int accumulate;      // y += instead of y =
     // filled in by the launcher
     size_t row_bytes;
-    int team_waves, wgs_per_cu, mfma_wgs_per_cu;
+    int team_waves, wgs_per_cu, mfma_wgs_per_cu, n_seg_types;
 };
 
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
@@ -41,6 +43,10 @@ hipError_t gemv_launch(int type, GemvArgs args, int cu_count, hipStream_t stream
 bool gemv_mfma_ok(int type, const GemvArgs& args);
 hipError_t gemv_mfma_launch(int type, const GemvArgs& args, int cu_count, hipStream_t stream);
 hipError_t gemv_mfma_allow_lds();
+// Up to three matrices, each Q4_K or Q6_K (GemvSeg::type), in one launch on the matrix cores.
+hipError_t gemv_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
+hipError_t gemv_mfma_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
+bool gemv_use_mfma();
 
 hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream);
 hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream);

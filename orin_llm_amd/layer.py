@@ -42,11 +42,13 @@ def _lib():
         L.orin_swiglu.argtypes = [_vp, _vp, _vp, _int]
         L.orin_gemv_multi.argtypes = [_int, _int, ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
                                       ctypes.POINTER(_int), _vp, _vp, _flt, _int, _int]
+        L.orin_gemv_multi_types.argtypes = [ctypes.POINTER(_int), _int, ctypes.POINTER(_vp), ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                                            ctypes.POINTER(_int), _vp, _vp, _flt, _int]
         L.orin_gemv_norm_gate_up_swiglu.argtypes = [_int, _vp, _vp, _vp, _vp, _flt, _vp, _int, _int]
         L.orin_decode_layer.argtypes = [ctypes.POINTER(DecodeLayerDesc)]
         for n in ("orin_rms_norm", "orin_rms_norm_rows", "orin_quantize_activation", "orin_gemv_q8", "orin_gemv_q8_bias",
                   "orin_gemv_q8_add", "orin_gemv_fused_gate_up_swiglu", "orin_gemv", "orin_dequant_row", "orin_swiglu",
-                  "orin_gemv_multi", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"):
+                  "orin_gemv_multi", "orin_gemv_multi_types", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"):
             getattr(L, n).restype = _int
         _ready = True
     return L
@@ -110,6 +112,14 @@ def gemv_multi(wtype, Ws, biases, ys, n_outs, x, norm_w, eps, n_in, accumulate=F
     arr = lambda xs: (_vp * m)(*[_p(v) for v in xs])  # noqa: E731
     _check("gemv_multi", _lib().orin_gemv_multi(wtype, m, arr(Ws), arr(biases) if biases is not None else None, arr(ys),
                                                 (_int * m)(*n_outs), _p(x), _p(norm_w), eps, n_in, 1 if accumulate else 0))
+
+
+def gemv_multi_types(wtypes, Ws, biases, ys, n_outs, x, norm_w, eps, n_in):
+    """gemv_multi with a type per matrix."""
+    m = len(Ws)
+    arr = lambda xs: (_vp * m)(*[_p(v) for v in xs])  # noqa: E731
+    _check("gemv_multi_types", _lib().orin_gemv_multi_types((_int * m)(*wtypes), m, arr(Ws), arr(biases) if biases is not None else None,
+                                                            arr(ys), (_int * m)(*n_outs), _p(x), _p(norm_w), eps, n_in))
 
 
 def gemv_norm_gate_up_swiglu(wtype, Wg, Wu, x, norm_w, eps, out, n_in, n_out):

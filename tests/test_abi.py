@@ -50,7 +50,7 @@ def test_layer_header_declares_the_expected_entry_points():
     assert _declared_c_functions(LAYER_HDR) == sorted([
         "orin_row_bytes", "orin_rms_norm", "orin_rms_norm_rows", "orin_quantize_activation", "orin_gemv_q8",
         "orin_gemv_q8_bias", "orin_gemv_q8_add", "orin_gemv_fused_gate_up_swiglu", "orin_gemv", "orin_dequant_row",
-        "orin_swiglu", "orin_gemv_multi", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"])
+        "orin_swiglu", "orin_gemv_multi", "orin_gemv_multi_types", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"])
 
 
 def test_library_exports_every_declared_symbol(lib):

@@ -161,6 +161,28 @@ def test_three_projections_in_one_launch(ly, wtype):
         assert vec_err(y.cpu().numpy()[:n], (w_ + ref.gemv(wtype, t[1], x, n_in, n)).astype(np.float64)) < TOL_OP
 
 
+@pytest.mark.parametrize("wtypes", [(lm.Q4_K, lm.Q4_K, lm.Q6_K), (lm.Q6_K, lm.Q4_K, lm.Q6_K), (lm.Q4_K, lm.Q5_K, lm.Q6_K), (lm.Q8_0, lm.F16)])
+@pytest.mark.parametrize("n_in", [1536, 4096])
+def test_projections_of_different_types(ly, wtypes, n_in):
+    """One launch where every type is Q4_K or Q6_K, one per matrix otherwise; same results either way."""
+    import torch
+
+    n_outs = [520, 130, 96][:len(wtypes)]
+    rs = lm.Stream(4500 + sum(wtypes) + n_in)
+    ts = [lm.make_tensor(rs, t, n_in, n) for t, n in zip(wtypes, n_outs)]
+    bs = [rs.sym(n, 0.5) for n in n_outs]
+    x, nw = rs.sym(n_in, 3.0), (1.0 + rs.sym(n_in, 0.3)).astype(np.float32)
+    xn = ref.rms_norm(x, nw, 1e-6)
+    want = [ref.gemv(t[0], t[1], xn, n_in, n) + b for t, b, n in zip(ts, bs, n_outs)]
+    ws = [dev_bytes(t[1], offset=2 if t[0] in (lm.Q8_0, lm.Q6_K) else 0) for t in ts]
+    ys = [out_buf(n) for n in n_outs]
+    ly.gemv_multi_types(list(wtypes), ws, [_dev(b) for b in bs], ys, n_outs, _dev(x), _dev(nw), 1e-6, n_in)
+    torch.cuda.synchronize()
+    for y, w_, n in zip(ys, want, n_outs):
+        got = y.cpu().numpy()
+        assert vec_err(got[:n], w_.astype(np.float64)) < TOL_OP and (got[n:] == 12345.0).all()
+
+
 def test_rms_norm_rows_swiglu_and_in_place(ly):
     import torch
 
