@@ -1,8 +1,9 @@
-// The attention, KV-cache and rotary-embedding slice of the orin_llm operator API, with the reference's own
-// signatures (reference: src/kernels.h:8-10, :55-62, :66-73 and :77-81), implemented for MI355X by
-// liborin_fa.so.  An engine built against the reference header links these symbols
-// unchanged; each forwards to the C ABI in include/orin_fa.h and, like the
-// reference's CUDA_CHECK (src/common.h:14-22), prints and abort()s on failure.
+// The decode layer's slice of the orin_llm operator API -- attention, KV cache, rotary embedding, and the norms
+// and quantised matrix-vector products around them -- with the reference's own signatures (reference:
+// src/kernels.h:8-10, :15-47, :55-62, :66-73 and :77-81), implemented for MI355X by liborin_fa.so.  An engine
+// built against the reference header links these symbols unchanged; each forwards to the C ABI in
+// include/orin_fa.h and include/orin_layer.h and, like the reference's CUDA_CHECK (src/common.h:14-22), prints
+// and abort()s on failure.
 //
 // Pointers are device pointers; kc / vc hold fp16 bit patterns laid out
 // [kv_head][n_ctx][head_dim] for one layer; q / out are fp32 [batch][n_head][head_dim].
@@ -10,6 +11,21 @@
 
 #include <stddef.h>
 #include <stdint.h>
+
+#ifndef ORIN_FA_SHIM_HAVE_DTYPE
+// The weight types, numbered as ggml numbers them (reference: src/common.h:47-54).  An engine that includes
+// its own common.h first defines ORIN_FA_SHIM_HAVE_DTYPE.
+namespace llm {
+enum class DType : uint32_t {
+    F32  = 0,
+    F16  = 1,
+    Q8_0 = 8,
+    Q4_K = 12,
+    Q5_K = 13,
+    Q6_K = 14,
+};
+} // namespace llm
+#endif
 
 namespace llm::cuda {
 
@@ -20,6 +36,26 @@ namespace llm::cuda {
 int init();
 void set_stream(void* stream);
 #endif
+
+void quantize_activation(const float* x, int n_in);
+
+void gemv(DType type, const void* W, const float* x, float* y, int n_in, int n_out);
+
+void gemv_q8(DType type, const void* W, float* y, int n_in, int n_out);
+
+void gemv_q8_bias(DType type, const void* W, const float* bias, float* y, int n_in, int n_out);
+
+void gemv_q8_add(DType type, const void* W, float* y, int n_in, int n_out);
+
+void gemv_fused_gate_up_swiglu(DType type, const void* Wg, const void* Wu,
+                                float* out, int n_in, int n_out);
+
+void dequant_row(DType type, const void* src, float* y, int n);
+
+void rms_norm(const float* x, const float* w, int n, float eps, float* y);
+void rms_norm_rows(const float* x, const float* w, int rows, int cols, float eps, float* y);
+
+void swiglu(float* act, const float* gate, const float* up, int n);
 
 void rope_neox_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors = nullptr);
 

@@ -1,5 +1,5 @@
 // llm::cuda::* entry points with the reference's signatures (reference:
-// src/kernels.h:8-10,55-62,66-73,77-81; definitions src/kernels.cu:1728-1737,1974-2000,2059-2093),
+// src/kernels.h:8-10,15-47,55-62,66-73,77-81; definitions src/kernels.cu:1728-1737,1778-1836,1944-2044,2059-2093),
 // forwarding to the C ABI.  Plain C++: no HIP headers, no device code.
 #include "../../include/orin_llm_amd/kernels.h"
 
@@ -7,6 +7,7 @@
 #include <stdlib.h>
 
 #include "../../include/orin_fa.h"
+#include "../../include/orin_layer.h"
 
 namespace {
 
@@ -33,6 +34,56 @@ int init() {
 
 void set_stream(void* stream) { orin_fa_set_stream(stream); }
 #endif
+
+void quantize_activation(const float* x, int n_in) {
+    const int rc = orin_quantize_activation(x, n_in);
+    if (rc != ORIN_FA_OK) die("quantize_activation", rc);
+}
+
+void gemv(DType type, const void* W, const float* x, float* y, int n_in, int n_out) {
+    const int rc = orin_gemv((int)type, W, x, y, n_in, n_out);
+    if (rc != ORIN_FA_OK) die("gemv", rc);
+}
+
+void gemv_q8(DType type, const void* W, float* y, int n_in, int n_out) {
+    const int rc = orin_gemv_q8((int)type, W, y, n_in, n_out);
+    if (rc != ORIN_FA_OK) die("gemv_q8", rc);
+}
+
+void gemv_q8_bias(DType type, const void* W, const float* bias, float* y, int n_in, int n_out) {
+    const int rc = orin_gemv_q8_bias((int)type, W, bias, y, n_in, n_out);
+    if (rc != ORIN_FA_OK) die("gemv_q8_bias", rc);
+}
+
+void gemv_q8_add(DType type, const void* W, float* y, int n_in, int n_out) {
+    const int rc = orin_gemv_q8_add((int)type, W, y, n_in, n_out);
+    if (rc != ORIN_FA_OK) die("gemv_q8_add", rc);
+}
+
+void gemv_fused_gate_up_swiglu(DType type, const void* Wg, const void* Wu, float* out, int n_in, int n_out) {
+    const int rc = orin_gemv_fused_gate_up_swiglu((int)type, Wg, Wu, out, n_in, n_out);
+    if (rc != ORIN_FA_OK) die("gemv_fused_gate_up_swiglu", rc);
+}
+
+void dequant_row(DType type, const void* src, float* y, int n) {
+    const int rc = orin_dequant_row((int)type, src, y, n);
+    if (rc != ORIN_FA_OK) die("dequant_row", rc);
+}
+
+void rms_norm(const float* x, const float* w, int n, float eps, float* y) {
+    const int rc = orin_rms_norm(x, w, n, eps, y);
+    if (rc != ORIN_FA_OK) die("rms_norm", rc);
+}
+
+void rms_norm_rows(const float* x, const float* w, int rows, int cols, float eps, float* y) {
+    const int rc = orin_rms_norm_rows(x, w, rows, cols, eps, y);
+    if (rc != ORIN_FA_OK) die("rms_norm_rows", rc);
+}
+
+void swiglu(float* act, const float* gate, const float* up, int n) {
+    const int rc = orin_swiglu(act, gate, up, n);
+    if (rc != ORIN_FA_OK) die("swiglu", rc);
+}
 
 void rope_neox_batch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads, const float* freq_factors) {
     const int rc = orin_fa_rope_batch(x, rows, head_dim, n_rot, theta, n_past, heads, freq_factors, 1);

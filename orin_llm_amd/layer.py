@@ -151,8 +151,18 @@ def decode_layer(desc):
     _check("decode_layer", _lib().orin_decode_layer(ctypes.byref(desc)))
 
 
-def decode_layer_calls(hp, L, bufs, kc, vc, d_pos, n_ctx):
-    """The reference's decode_layer, call for call (src/model_gpu.cu:251-293).  bufs additionally holds xn, xn2."""
+def decode_layer_calls(hp, L, bufs, kc, vc, d_pos, n_ctx, ops=None):
+    """The reference's decode_layer, call for call (src/model_gpu.cu:251-293).  bufs additionally holds xn, xn2.
+    ops: an object with the operators under the reference's names (default: this module and kernels)."""
+    if ops is not None:
+        return _decode_layer_calls(ops, ops, hp, L, bufs, kc, vc, d_pos, n_ctx)
+    import sys
+    return _decode_layer_calls(sys.modules[__name__], _k, hp, L, bufs, kc, vc, d_pos, n_ctx)
+
+
+def _decode_layer_calls(o, ka, hp, L, bufs, kc, vc, d_pos, n_ctx):
+    rms_norm, rms_norm_rows, quantize_activation, swiglu = o.rms_norm, o.rms_norm_rows, o.quantize_activation, o.swiglu
+    gemv_q8, gemv_q8_bias, gemv_q8_add, gemv_fused_gate_up_swiglu = o.gemv_q8, o.gemv_q8_bias, o.gemv_q8_add, o.gemv_fused_gate_up_swiglu
     ne, nh, nkv, hd, nff = hp["n_embd"], hp["n_head"], hp["n_kv"], hp["head_dim"], hp["n_ff"]
     eps, scale = hp["rms_eps"], 1.0 / float(hd) ** 0.5
     x, xn, xn2, q, k, v, attn, act = (bufs[n] for n in ("x", "xn", "xn2", "q", "k", "v", "attn", "act"))
@@ -170,11 +180,11 @@ def decode_layer_calls(hp, L, bufs, kc, vc, d_pos, n_ctx):
         rms_norm_rows(q, L["q_norm"], nh, hd, eps, q)
     if L.get("k_norm") is not None:
         rms_norm_rows(k, L["k_norm"], nkv, hd, eps, k)
-    rope_ind = _k.rope_neox_ind if hp["neox"] else _k.rope_normal_ind
+    rope_ind = ka.rope_neox_ind if hp["neox"] else ka.rope_normal_ind
     rope_ind(q, nh, hd, hp["n_rot"], hp["rope_theta"], d_pos, hp.get("freq_factors_dev"))
     rope_ind(k, nkv, hd, hp["n_rot"], hp["rope_theta"], d_pos, hp.get("freq_factors_dev"))
-    _k.kv_store_ind(kc, vc, k, v, nkv, hd, n_ctx, d_pos)
-    _k.flash_attention_decode_ind(q, kc, vc, attn, nh, nkv, hd, n_ctx, d_pos, scale)
+    ka.kv_store_ind(kc, vc, k, v, nkv, hd, n_ctx, d_pos)
+    ka.flash_attention_decode_ind(q, kc, vc, attn, nh, nkv, hd, n_ctx, d_pos, scale)
     quantize_activation(attn, nh * hd)
     gemv_q8_add(L["wo"][0], L["wo"][1], x, nh * hd, ne)
     rms_norm(x, L["ffn_norm"], ne, eps, xn2)

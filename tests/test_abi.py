@@ -124,6 +124,16 @@ def test_shim_symbols_have_the_reference_manglings():
         "_ZN3llm4cuda8kv_shiftEPtS1_iiiiii",
         "_ZN3llm4cuda4initEv",
         "_ZN3llm4cuda10set_streamEPv",
+        "_ZN3llm4cuda19quantize_activationEPKfi",
+        "_ZN3llm4cuda4gemvENS_5DTypeEPKvPKfPfii",
+        "_ZN3llm4cuda7gemv_q8ENS_5DTypeEPKvPfii",
+        "_ZN3llm4cuda12gemv_q8_biasENS_5DTypeEPKvPKfPfii",
+        "_ZN3llm4cuda11gemv_q8_addENS_5DTypeEPKvPfii",
+        "_ZN3llm4cuda25gemv_fused_gate_up_swigluENS_5DTypeEPKvS3_Pfii",
+        "_ZN3llm4cuda11dequant_rowENS_5DTypeEPKvPfi",
+        "_ZN3llm4cuda8rms_normEPKfS2_ifPf",
+        "_ZN3llm4cuda13rms_norm_rowsEPKfS2_iifPf",
+        "_ZN3llm4cuda6swigluEPfPKfS3_i",
     ]
     for s in expected:
         assert s in syms, s
@@ -139,7 +149,9 @@ def _decl(text, name):
 def test_shim_header_matches_reference_declarations():
     ref, ours = open(REF_HDR).read(), open(SHIM_HDR).read()
     for name in ("flash_attention", "flash_attention_decode_ind", "kv_store_batch", "kv_store_ind", "kv_shift",
-                 "rope_neox_batch", "rope_normal_batch", "rope_neox_ind", "rope_normal_ind"):
+                 "rope_neox_batch", "rope_normal_batch", "rope_neox_ind", "rope_normal_ind",
+                 "quantize_activation", "gemv", "gemv_q8", "gemv_q8_bias", "gemv_q8_add", "gemv_fused_gate_up_swiglu",
+                 "dequant_row", "rms_norm", "rms_norm_rows", "swiglu"):
         assert _decl(ours, name) == _decl(ref, name)
 
 
@@ -167,6 +179,18 @@ int main(int argc, char**) {
         llm::cuda::kv_store_ind(kc, vc, k, v, 2, 128, 4096, d_pos);
         llm::cuda::flash_attention_decode_ind(q, kc, vc, out, 12, 2, 128, 4096, d_pos, 0.088f);
         llm::cuda::kv_shift(kc, vc, 28, 2, 128, 4096, 4, 2046);
+        // the rest of the decode layer (reference: src/model_gpu.cu:251-293, 303-306)
+        const void* W = nullptr; float* x = nullptr; float* y = nullptr; const float* w = nullptr;
+        llm::cuda::dequant_row(llm::DType::Q4_K, W, x, 1536);
+        llm::cuda::rms_norm(x, w, 1536, 1e-6f, y);
+        llm::cuda::quantize_activation(y, 1536);
+        llm::cuda::gemv_q8(llm::DType::Q4_K, W, q, 1536, 1536);
+        llm::cuda::gemv_q8_bias(llm::DType::Q6_K, W, w, v, 1536, 256);
+        llm::cuda::rms_norm_rows(q, w, 12, 128, 1e-6f, q);
+        llm::cuda::gemv_q8_add(llm::DType::Q4_K, W, x, 1536, 1536);
+        llm::cuda::gemv_fused_gate_up_swiglu(llm::DType::Q4_K, W, W, y, 1536, 8960);
+        llm::cuda::swiglu(y, y, y, 8960);
+        llm::cuda::gemv(llm::DType::Q6_K, W, x, y, 1536, 151936);
     }
     return 0;
 }

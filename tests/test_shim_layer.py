@@ -159,3 +159,91 @@ def test_decode_steps_through_the_shim_replayed_from_a_graph(shim):
             if l not in (0, 13, n_layer - 1):
                 k_ref = ref.rope_batch(k[l], D, D, THETA, pos, G, None, True)
                 ref.kv_store_f16(kcs[l], vcs[l], k_ref[None], v[l][None], G, D, n_ctx, pos, 1)
+
+
+# ---------------------------------------------------------------- the whole decode step
+
+LAYER_SHIM = {  # the rest of what decode_layer calls (reference: src/model_gpu.cu:251-293, 303-306)
+    "rope_normal_ind": ("_ZN3llm4cuda15rope_normal_indEPfiiifPKiPKf", [vp, ci, ci, ci, cf, vp, vp]),
+    "quantize_activation": ("_ZN3llm4cuda19quantize_activationEPKfi", [vp, ci]),
+    "gemv": ("_ZN3llm4cuda4gemvENS_5DTypeEPKvPKfPfii", [ci, vp, vp, vp, ci, ci]),
+    "gemv_q8": ("_ZN3llm4cuda7gemv_q8ENS_5DTypeEPKvPfii", [ci, vp, vp, ci, ci]),
+    "gemv_q8_bias": ("_ZN3llm4cuda12gemv_q8_biasENS_5DTypeEPKvPKfPfii", [ci, vp, vp, vp, ci, ci]),
+    "gemv_q8_add": ("_ZN3llm4cuda11gemv_q8_addENS_5DTypeEPKvPfii", [ci, vp, vp, ci, ci]),
+    "gemv_fused_gate_up_swiglu": ("_ZN3llm4cuda25gemv_fused_gate_up_swigluENS_5DTypeEPKvS3_Pfii", [ci, vp, vp, vp, ci, ci]),
+    "dequant_row": ("_ZN3llm4cuda11dequant_rowENS_5DTypeEPKvPfi", [ci, vp, vp, ci]),
+    "rms_norm": ("_ZN3llm4cuda8rms_normEPKfS2_ifPf", [vp, vp, ci, cf, vp]),
+    "rms_norm_rows": ("_ZN3llm4cuda13rms_norm_rowsEPKfS2_iifPf", [vp, vp, ci, ci, cf, vp]),
+    "swiglu": ("_ZN3llm4cuda6swigluEPfPKfS3_i", [vp, vp, vp, ci]),
+}
+
+
+@pytest.mark.parametrize("name", ["qwen2", "llama"])
+def test_whole_decode_step_through_the_shim_replayed_from_a_graph(shim, name):
+    """The reference's forward_capture (src/model_gpu.cu:295-316) over a small quantised model: embedding
+    row, every layer call for call, last norm, output matrix -- through the llm::cuda symbols, captured once
+    and replayed per token with the embedding row and the position updated in place -- against the logits of
+    the unmodified reference CPU build."""
+    import os
+    import sys
+
+    import torch
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, os.path.join(here, "golden"))
+    import layer_model as lm
+    from orin_llm_amd import kernels, layer as ly
+    from test_gpu_layer import make_bufs, upload, vec_err
+
+    lib = ctypes.CDLL(kernels.LIB_PATH)
+
+    class Ops:  # the operators under the reference's names, taking tensors
+        pass
+
+    ops = Ops()
+    table = dict(SHIM)
+    table.update(LAYER_SHIM)
+    for fname, (sym, argtypes) in table.items():
+        f = getattr(lib, sym)
+        f.argtypes, f.restype = argtypes, (ci if fname == "init" else None)
+
+        def call(*args, _f=f):
+            _f(*[a.data_ptr() if hasattr(a, "data_ptr") else a for a in args])
+        setattr(ops, fname, call)
+
+    golden = np.load(os.path.join(here, "golden", "layer_reference.npz"))
+    n_tok, n_ctx = (int(v) for v in golden["meta"])
+    model = lm.build(name)
+    hp, layers, top = upload(model)
+    bufs = make_bufs(hp)
+    ne, nv, nl = hp["n_embd"], hp["n_vocab"], hp["n_layer"]
+    kc = torch.zeros((nl, hp["n_kv"], n_ctx, hp["head_dim"]), dtype=torch.int16, device="cuda")
+    vc = torch.zeros_like(kc)
+    d_pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    et, eraw = top["token_embd"]
+    rb = ref.row_bytes(et, ne)
+    emb_row = torch.zeros(rb + 16, dtype=torch.uint8, device="cuda")[:rb]
+
+    def step():
+        ops.dequant_row(et, emb_row, bufs["x"], ne)
+        for l in range(nl):
+            ly.decode_layer_calls(hp, layers[l], bufs, kc[l], vc[l], d_pos, n_ctx, ops=ops)
+        ops.rms_norm(bufs["x"], top["output_norm"], ne, hp["rms_eps"], bufs["xn"])
+        ops.gemv(top["output"][0], top["output"][1], bufs["xn"], bufs["logits"], ne, nv)
+
+    stream, graph, worst = torch.cuda.Stream(), None, 0.0
+    for t in range(n_tok):
+        emb_row.copy_(eraw[t * rb:(t + 1) * rb])
+        d_pos.fill_(t)
+        torch.cuda.synchronize()
+        if graph is None:
+            shim.set_stream(stream.cuda_stream)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                step()
+            shim.set_stream(torch.cuda.current_stream().cuda_stream)
+        graph.replay()
+        torch.cuda.synchronize()
+        worst = max(worst, vec_err(bufs["logits"].cpu().numpy(), golden["logits_" + name][t].astype(np.float64)))
+    print(f"{name} through the shim, graph replay: vs reference logits {worst:.2e}", flush=True)
+    assert worst < 1e-2
