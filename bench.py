@@ -117,7 +117,7 @@ ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qw
         "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
         "qwen1.5b-decode-32k-cutoffs", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
-TARGETS = ["decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
+TARGETS = ["qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
 
 
@@ -1246,9 +1246,13 @@ def main():
                 rf = a["roofline"]
                 t = dict(frac=round(rf["frac"], 4), achieved=round(rf["achieved"], 1), unit=rf["unit"],
                          launch_us=round(rf["launch_us"], 2))
-                if "fused_two_level_us" in rf:
+                if "layer_us" in rf:
+                    t = dict(layer_us=round(rf["layer_us"], 2), layer_frac=round(rf["layer_frac"], 4),
+                             layer_us_reference_call_sequence=round(rf["layer_us_reference_call_sequence"], 2),
+                             err=float(f"{a['parity']['err_row']:.2e}"))
+                elif "fused_two_level_us" in rf:
                     t = dict(two_launch_us=round(rf["two_launch_us"], 2), fused_two_level_us=round(rf["fused_two_level_us"], 2))
-                elif a["parity"]:
+                elif a["parity"] and "layer_us" not in rf:
                     t["err_row"] = float(f"{a['parity']['err_row']:.2e}")
                     t["err_floor1pct"] = float(f"{a['parity']['err_floor1pct']:.2e}")
                 if "tiny_kernel_launch_to_launch_us" in rf:
