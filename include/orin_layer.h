@@ -15,9 +15,10 @@
  * activations and outputs 16-byte aligned.  ORIN_FA_E_INVALID otherwise.
  *
  * Arithmetic: the reference's GPU operators round the activation to int8 in blocks of 32 before a
- * product (quantize_activation + dp4a).  These keep it in fp32 and decode the weights to the exact
- * fp32 values of the reference's CPU backend (src/model_cpu.cpp:70-167), so results agree with that
- * backend up to the order of the fp32 sum.
+ * product (quantize_activation + dp4a).  These keep it at fp32 precision (as fp32, or as three int8
+ * digits of a 24-bit integer per sub-block on the matrix cores) and use the weights' exact values as the
+ * reference's CPU backend decodes them (src/model_cpu.cpp:70-167), so results agree with that backend up to
+ * the order of an fp32 sum.
  */
 #ifndef ORIN_LAYER_H
 #define ORIN_LAYER_H
@@ -70,6 +71,12 @@ int orin_dequant_row(int type, const void* src, float* y, int n);
 /* Replaces llm::cuda::swiglu (reference: src/kernels.h:47, src/kernels.cu:1702-1707, 2041-2044):
  * act[i] = silu(gate[i]) * up[i]. */
 int orin_swiglu(float* act, const float* gate, const float* up, int n);
+
+/* Products over the block types (Q4_K, Q5_K, Q6_K, Q8_0) run on the matrix cores where the row length is a
+ * multiple of 256 (the activation carried as three int8 digits per sub-block, integer matrix instructions, the
+ * blocks' scales applied in fp32) and on the vector ALU otherwise, as F16 and F32 always do.  on = 0 keeps
+ * everything on the vector ALU: for comparisons and tests; the results agree to the order of an fp32 sum. */
+void orin_gemv_use_matrix_cores(int on);
 
 /* ---- forms with no counterpart in the reference: fewer launches per layer ---- */
 

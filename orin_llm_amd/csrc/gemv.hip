@@ -468,14 +468,17 @@ int gemv_mfma_wgs_per_cu() {
     return v;
 }
 
-// ORIN_GEMV_NO_MFMA=1 keeps every type on the vector-ALU kernel (for comparisons).
+// Whether block types go to the matrix-core kernel (default) or stay on the vector-ALU kernel
+// (orin_gemv_use_matrix_cores(0), or ORIN_GEMV_NO_MFMA=1 in the environment: for comparisons and tests).
+static int g_use_mfma = -1;
 bool gemv_use_mfma() {
-    static const bool v = [] {
+    if (g_use_mfma < 0) {
         const char* e = getenv("ORIN_GEMV_NO_MFMA");
-        return !(e && e[0] == '1');
-    }();
-    return v;
+        g_use_mfma = !(e && e[0] == '1');
+    }
+    return g_use_mfma != 0;
 }
+void gemv_set_use_mfma(bool on) { g_use_mfma = on ? 1 : 0; }
 
 size_t weight_row_bytes(int type, int n) {
     switch (type) {

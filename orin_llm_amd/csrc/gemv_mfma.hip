@@ -1,12 +1,13 @@
-// Matrix-vector products over Q4_K and Q6_K weight rows on the matrix cores of gfx950 (MI355X).
+// Matrix-vector products over quantised weight rows (Q4_K, Q5_K, Q6_K, Q8_0) on the matrix cores of gfx950
+// (MI355X).
 //
 // The vector-ALU kernel of gemv.hip spends about three instructions per weight (byte to float,
 // multiply-add, unpacking) and is bound by them at twice the time HBM needs for the bytes.  Here
 // the multiply-adds run as integer matrix instructions and the vector ALU only assembles the
 // weights' bytes and applies the blocks' scales:
 //
-//   * The activation is cut, per sub-block of the weight format (32 elements for Q4_K, 16 for
-//     Q6_K), into three signed 8-bit digits of a 24-bit integer, x = s (65536 d0 + 256 d1 + d2)
+//   * The activation is cut, per sub-block of the weight format (16 elements for Q6_K, 32 for
+//     the others), into three signed 8-bit digits of a 24-bit integer, x = s (65536 d0 + 256 d1 + d2)
 //     with s = max|x| / (2^23 - 2^16): what the reference does with one digit (quantize_q8_1_k,
 //     reference: src/kernels.cu:136-157), carried to the precision of an fp32 mantissa.  Every
 //     workgroup builds the digits once, in LDS (together with the RMS norm, when that is folded
@@ -17,8 +18,8 @@
 //     accumulator therefore holds, for a row of weights, the exact integer sums of four sub-blocks
 //     against the three digits, already separated: lane (n, g) receives the three sums of
 //     sub-block g.  They are recombined in fp32 and multiplied by the sub-block's scales:
-//     d * scale * sum - dmin * min * sum(x) for Q4_K, d * scale * (sum - 32 sum(x)) for Q6_K
-//     (reference CPU statements: src/model_cpu.cpp:70-89, 115-142).
+//     d * scale * sum - dmin * min * sum(x) for Q4_K and Q5_K, d * scale * (sum - 32 sum(x)) for Q6_K,
+//     d * sum for Q8_0 (reference CPU statements: src/model_cpu.cpp:70-152).
 //   * Loads are made with four neighbouring lanes on 64 consecutive bytes of a row (lane = 4 * row +
 //     piece: the vector cache then sees 16 runs per instruction; with the matrix instruction's own
 //     lane order, lane = row + 16 * piece, it sees 64 separate 16-byte requests and the kernel runs
@@ -142,22 +143,26 @@ struct LaneCtx {
 template <int T>
 struct MF;
 
-// Q4_K (reference: src/quant.h:14-21): per 128-element half of a block, the lane's 16 bytes of nibbles
-// are 16 elements of sub-block 2 (g / 2) (low nibbles) and of 2 (g / 2) + 1 (high nibbles); the two
+// Q4_K and Q5_K (reference: src/quant.h:14-31): per 128-element half of a block, the lane's 16 bytes of
+// nibbles are 16 elements of sub-block 2 (g / 2) (low nibbles) and of 2 (g / 2) + 1 (high nibbles); the two
 // matrix instructions of a half add into one accumulator whose row group p is sub-block p of the half.
-template <>
-struct MF<kQ4_K> {
-    static constexpr int kGroup = 32, kBlockBytes = 144;
+// Q5_K keeps a fifth bit per element in 32 bytes behind the header: bit p of byte e belongs to element e of
+// sub-block p.
+template <bool FIVE>
+struct MFK45 {
+    static constexpr int kGroup = 32, kBlockBytes = FIVE ? 176 : 144, kQs = FIVE ? 48 : 16;
     struct Raw {
         u32x4 hdr, q1, q2; // a block's header and this lane's 16 bytes of each half of its nibbles
+        u32x4 qh;          // (Q5_K) the 16 bytes of fifth bits that cover this lane's elements
     };
     struct Addr {
         int lo_base, hi_base, lo_step, hi_step; // LDS byte offsets of this lane's A operands; a lane whose row is zero reads the 16 zero bytes, stride 0
     };
     static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
         r.hdr = *reinterpret_cast<const u32x4*>(blk);
-        r.q1 = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * lg);
-        r.q2 = *reinterpret_cast<const u32x4*>(blk + 80 + 16 * lg);
+        if constexpr (FIVE) r.qh = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * (lg & 1));
+        r.q1 = *reinterpret_cast<const u32x4*>(blk + kQs + 16 * lg);
+        r.q2 = *reinterpret_cast<const u32x4*>(blk + kQs + 64 + 16 * lg);
     }
     static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
         const int ap = c.am >> 2, ad = c.am & 3, g = c.g;
@@ -177,6 +182,11 @@ struct MF<kQ4_K> {
         // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
         const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
         const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
+        u32x4 fifth = {0u, 0u, 0u, 0u};
+        if constexpr (FIVE) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fifth[i] = from_lane(c.src_lane4, r.qh[i]) >> (2 * (c.g >> 1));
+        }
         float out = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -188,13 +198,78 @@ struct MF<kQ4_K> {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const unsigned q = from_lane(c.src_lane4, qs[i]);
-                lo[i] = (int)(q & 0x0f0f0f0fu);
-                hi[i] = (int)((q >> 4) & 0x0f0f0f0fu);
+                unsigned l = q & 0x0f0f0f0fu, u = (q >> 4) & 0x0f0f0f0fu;
+                if constexpr (FIVE) { // sub-blocks 4 h + 2 (g / 2) and + 1: bits 4 h and 4 h + 1 of the shifted bytes
+                    const unsigned f = fifth[i] >> (4 * h);
+                    l |= (f & 0x01010101u) << 4;
+                    u |= (f & 0x02020202u) << 3;
+                }
+                lo[i] = (int)l;
+                hi[i] = (int)u;
             }
             i32x4 acc = {0, 0, 0, 0};
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, lo, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, hi, acc, 0, 0, 0);
             out += (d * sc[h]) * (digits_sum(acc) * xp.scale) - (dmin * mn[h]) * xp.sum;
+        }
+        return out;
+    }
+};
+template <>
+struct MF<kQ4_K> : MFK45<false> {};
+template <>
+struct MF<kQ5_K> : MFK45<true> {};
+
+// Q8_0 (reference: src/quant.h:42-45; blocks of 34 bytes, 2-byte aligned): eight blocks make up the 256
+// elements the kernel walks at a time.  Per 128-element half, the lane's 16 bytes are half of block
+// 2 run + g / 2 of the half, for run = 0, 1: one matrix instruction per run, both adding into one accumulator
+// whose row group p is block p of the half.
+template <>
+struct MF<kQ8_0> {
+    static constexpr int kGroup = 32, kBlockBytes = 272;
+    struct Raw {
+        u32x4 q[2][2]; // [half][run]
+        unsigned d[2]; // scales of blocks lg and 4 + lg
+    };
+    typedef MFK45<false>::Addr Addr;
+    template <typename V>
+    struct __attribute__((packed, aligned(2))) Loose {
+        V v;
+    };
+    static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int run = 0; run < 2; ++run)
+                r.q[h][run] = reinterpret_cast<const Loose<u32x4>*>(blk + 34 * (4 * h + 2 * run + (lg >> 1)) + 2 + 16 * (lg & 1))->v;
+            r.d[h] = *reinterpret_cast<const uint16_t*>(blk + 34 * (4 * h + lg));
+        }
+    }
+    static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
+        const int ap = c.am >> 2, ad = c.am & 3, g = c.g;
+        const bool live = ad < 3 && (ap & 1) == (g >> 1);
+        const int elem = 32 * ap + 16 * (g & 1);
+        const bool r0 = live && (ap >> 1) == 0, r1 = live && (ap >> 1) == 1;
+        return Addr{r0 ? ad * c.n_in + elem : c.zero_off, r1 ? ad * c.n_in + elem : c.zero_off, r0 ? 256 : 0, r1 ? 256 : 0};
+    }
+    static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
+        float out = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const i32x4 a0 = *reinterpret_cast<const i32x4*>(c.smem + ad.lo_base + b * ad.lo_step + (ad.lo_step ? 128 * h : 0));
+            const i32x4 a1 = *reinterpret_cast<const i32x4*>(c.smem + ad.hi_base + b * ad.hi_step + (ad.hi_step ? 128 * h : 0));
+            const XPair xp = c.pairs[8 * b + 4 * h + c.g];
+            const float d = half_of(from_lane(c.src_lane4, r.d[h]));
+            i32x4 w0, w1;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                w0[i] = (int)from_lane(c.src_lane4, r.q[h][0][i]);
+                w1[i] = (int)from_lane(c.src_lane4, r.q[h][1][i]);
+            }
+            i32x4 acc = {0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, w0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, w1, acc, 0, 0, 0);
+            out += d * (digits_sum(acc) * xp.scale);
         }
         return out;
     }
@@ -364,12 +439,16 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
     gemv_mfma_body<T, DUAL, kWaves>(a);
 }
 
-// Matrices of both types in one launch (the q, k, v projections of a file that keeps attn_v in Q6_K): a
-// workgroup belongs to one matrix and runs that matrix's code.
+// Matrices of different block types in one launch (the q, k, v projections of a file that keeps attn_v in
+// Q6_K): a workgroup belongs to one matrix and runs that matrix's code.
 template <int kWaves>
 __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_mixed_kernel(const GemvArgs a) {
-    if (a.seg[blockIdx.y].type == kQ4_K) gemv_mfma_body<kQ4_K, false, kWaves>(a);
-    else gemv_mfma_body<kQ6_K, false, kWaves>(a);
+    switch (a.seg[blockIdx.y].type) {
+    case kQ4_K: gemv_mfma_body<kQ4_K, false, kWaves>(a); break;
+    case kQ5_K: gemv_mfma_body<kQ5_K, false, kWaves>(a); break;
+    case kQ6_K: gemv_mfma_body<kQ6_K, false, kWaves>(a); break;
+    default: gemv_mfma_body<kQ8_0, false, kWaves>(a); break;
+    }
 }
 
 constexpr size_t kMfmaLdsMax = 96u * 1024u;
@@ -408,7 +487,7 @@ hipError_t allow() {
 
 } // namespace
 
-// Every matrix Q4_K or Q6_K, each its own type (GemvSeg::type, row_bytes filled in by the caller).
+// Every matrix of a block type (Q4_K, Q5_K, Q6_K, Q8_0), each its own type (GemvSeg::type, row_bytes filled in by the caller).
 hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) {
     int max_out = 0;
     for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
@@ -422,13 +501,19 @@ hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) 
 
 bool gemv_mfma_ok(int type, const GemvArgs& a) {
     if (a.n_in % 256 != 0) return false;
-    if (type == kQ4_K) return lds_bytes<kQ4_K>(a.n_in) <= kMfmaLdsMax;
+    if (type == kQ4_K || type == kQ5_K || type == kQ8_0) return lds_bytes<kQ4_K>(a.n_in) <= kMfmaLdsMax;
     if (type == kQ6_K) return lds_bytes<kQ6_K>(a.n_in) <= kMfmaLdsMax;
     return false;
 }
 
 hipError_t gemv_mfma_launch(int type, const GemvArgs& a, int cu_count, hipStream_t stream) {
-    return type == kQ4_K ? launch<kQ4_K>(a, cu_count, stream) : launch<kQ6_K>(a, cu_count, stream);
+    switch (type) {
+    case kQ4_K: return launch<kQ4_K>(a, cu_count, stream);
+    case kQ5_K: return launch<kQ5_K>(a, cu_count, stream);
+    case kQ6_K: return launch<kQ6_K>(a, cu_count, stream);
+    case kQ8_0: return launch<kQ8_0>(a, cu_count, stream);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 // More than 64 KB of LDS per workgroup (rows longer than about 16k elements) needs to be allowed once.
@@ -438,6 +523,10 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow<kQ4_K, true>()) != hipSuccess) return e;
     if ((e = allow<kQ6_K, false>()) != hipSuccess) return e;
     if ((e = allow<kQ6_K, true>()) != hipSuccess) return e;
+    if ((e = allow<kQ5_K, false>()) != hipSuccess) return e;
+    if ((e = allow<kQ5_K, true>()) != hipSuccess) return e;
+    if ((e = allow<kQ8_0, false>()) != hipSuccess) return e;
+    if ((e = allow<kQ8_0, true>()) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }

@@ -95,6 +95,8 @@ using namespace orin_fa;
 
 extern "C" {
 
+void orin_gemv_use_matrix_cores(int on) { gemv_set_use_mfma(on != 0); }
+
 size_t orin_row_bytes(int type, int n) { return n < 0 ? 0 : weight_row_bytes(type, n); }
 
 int orin_rms_norm(const float* x, const float* w, int n, float eps, float* y) {

@@ -47,6 +47,7 @@ hipError_t gemv_mfma_allow_lds();
 hipError_t gemv_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
 hipError_t gemv_mfma_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
 bool gemv_use_mfma();
+void gemv_set_use_mfma(bool on);
 
 hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream);
 hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream);

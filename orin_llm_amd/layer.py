@@ -28,6 +28,8 @@ def _lib():
     global _ready
     L = _k.lib()
     if not _ready:
+        L.orin_gemv_use_matrix_cores.argtypes = [_int]
+        L.orin_gemv_use_matrix_cores.restype = None
         L.orin_row_bytes.argtypes = [_int, _int]
         L.orin_row_bytes.restype = ctypes.c_size_t
         L.orin_rms_norm.argtypes = [_vp, _vp, _int, _flt, _vp]
@@ -60,6 +62,11 @@ _p = _k._ptr
 def _check(what, rc):
     if rc != 0:
         raise _k.OrinFaError(what, rc)
+
+
+def use_matrix_cores(on):
+    """Block types on the matrix cores (default) or on the vector ALU (for comparisons and tests)."""
+    _lib().orin_gemv_use_matrix_cores(1 if on else 0)
 
 
 def row_bytes(wtype, n):

@@ -48,7 +48,7 @@ def test_measurement_aids_sit_in_their_own_header():
 
 def test_layer_header_declares_the_expected_entry_points():
     assert _declared_c_functions(LAYER_HDR) == sorted([
-        "orin_row_bytes", "orin_rms_norm", "orin_rms_norm_rows", "orin_quantize_activation", "orin_gemv_q8",
+        "orin_row_bytes", "orin_gemv_use_matrix_cores", "orin_rms_norm", "orin_rms_norm_rows", "orin_quantize_activation", "orin_gemv_q8",
         "orin_gemv_q8_bias", "orin_gemv_q8_add", "orin_gemv_fused_gate_up_swiglu", "orin_gemv", "orin_dequant_row",
         "orin_swiglu", "orin_gemv_multi", "orin_gemv_multi_types", "orin_gemv_norm_gate_up_swiglu", "orin_decode_layer"])
 

@@ -54,15 +54,29 @@ def out_buf(n, fill=12345.0, pad=4):
     return torch.full((n + pad,), fill, dtype=torch.float32, device="cuda")
 
 
-# rows that exercise every team shape: (n_in, waves per row, slots per lane)
+# rows that exercise every team shape of the vector-ALU kernel: (n_in, waves per row, slots per lane); on the
+# matrix cores the same lengths are 1 ... 74 blocks per row, shared among four waves
 SHAPES = [(256, 1, 1), (1536, 1, 1), (2048, 1, 1), (4096, 1, 2), (6144, 1, 3), (8960, 2, 3), (14336, 4, 2), (18944, 4, 3)]
 
 
-@pytest.mark.parametrize("wtype", TYPES)
+@pytest.fixture(params=["matrix cores", "vector ALU"])
+def unit(request, ly):
+    ly.use_matrix_cores(request.param == "matrix cores")
+    yield request.param
+    ly.use_matrix_cores(True)
+
+
+# (F32 and F16 rows are always on the vector ALU)
+TYPE_UNITS = [(t, "vector ALU") for t in TYPES] + [(t, "matrix cores") for t in (lm.Q8_0, lm.Q4_K, lm.Q5_K, lm.Q6_K)]
+
+
+@pytest.mark.parametrize("wtype,where", TYPE_UNITS)
 @pytest.mark.parametrize("n_in,kw,slots", SHAPES)
-def test_gemv_against_the_oracle(ly, wtype, n_in, kw, slots):
+def test_gemv_against_the_oracle(ly, wtype, where, n_in, kw, slots):
     import torch
 
+    unit = where
+    ly.use_matrix_cores(where == "matrix cores")
     n_out = 37 if n_in > 4096 else 131
     rs = lm.Stream(1000 + wtype * 31 + n_in)
     t = lm.make_tensor(rs, wtype, n_in, n_out)
@@ -75,7 +89,8 @@ def test_gemv_against_the_oracle(ly, wtype, n_in, kw, slots):
     got = y.cpu().numpy()
     assert (got[n_out:] == 12345.0).all(), "rows past n_out were written"
     e = vec_err(got[:n_out], want)
-    print(f"gemv {lm.TYPE_NAME[wtype]} n_in {n_in} (waves {kw}, slots {slots}): err {e:.2e}", flush=True)
+    ly.use_matrix_cores(True)
+    print(f"gemv {lm.TYPE_NAME[wtype]} n_in {n_in} on the {unit}: err {e:.2e}", flush=True)
     assert e < TOL_OP
 
 
@@ -110,9 +125,23 @@ def test_staged_products_bias_add_and_snapshot(ly, wtype):
         ly.gemv_q8(wtype, w, y, n_in // 2 if wtype == lm.F16 else 1280, n_out)
 
 
+def test_q8_0_rows_that_are_not_whole_256s_stay_on_the_vector_alu(ly):
+    """Q8_0 blocks are 32 elements: a row of 1568 is legal and does not fit the matrix-core kernel's 256-element steps."""
+    import torch
+
+    n_in, n_out = 1568, 50
+    rs = lm.Stream(1234)
+    t = lm.make_tensor(rs, lm.Q8_0, n_in, n_out)
+    x = rs.sym(n_in, 1.0)
+    y = out_buf(n_out)
+    ly.gemv(lm.Q8_0, dev_bytes(t[1], offset=2), _dev(x), y, n_in, n_out)
+    torch.cuda.synchronize()
+    assert vec_err(y.cpu().numpy()[:n_out], ref.gemv(lm.Q8_0, t[1], x, n_in, n_out).astype(np.float64)) < TOL_OP
+
+
 @pytest.mark.parametrize("wtype", [lm.Q8_0, lm.Q4_K, lm.Q5_K, lm.Q6_K])
 @pytest.mark.parametrize("n_in", [1536, 8960])
-def test_gate_up_swiglu_staged_and_with_the_norm_folded_in(ly, wtype, n_in):
+def test_gate_up_swiglu_staged_and_with_the_norm_folded_in(ly, unit, wtype, n_in):
     import torch
 
     n_out = 90
@@ -138,7 +167,7 @@ def test_gate_up_swiglu_staged_and_with_the_norm_folded_in(ly, wtype, n_in):
 
 
 @pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q6_K])
-def test_three_projections_in_one_launch(ly, wtype):
+def test_three_projections_in_one_launch(ly, unit, wtype):
     """q, k, v of different heights over one normalised activation, with biases; and accumulated."""
     import torch
 
@@ -163,8 +192,9 @@ def test_three_projections_in_one_launch(ly, wtype):
 
 @pytest.mark.parametrize("wtypes", [(lm.Q4_K, lm.Q4_K, lm.Q6_K), (lm.Q6_K, lm.Q4_K, lm.Q6_K), (lm.Q4_K, lm.Q5_K, lm.Q6_K), (lm.Q8_0, lm.F16)])
 @pytest.mark.parametrize("n_in", [1536, 4096])
-def test_projections_of_different_types(ly, wtypes, n_in):
-    """One launch where every type is Q4_K or Q6_K, one per matrix otherwise; same results either way."""
+def test_projections_of_different_types(ly, unit, wtypes, n_in):
+    """One launch where every type is a block type and the matrix cores are in use, one per matrix otherwise; same
+    results either way."""
     import torch
 
     n_outs = [520, 130, 96][:len(wtypes)]
