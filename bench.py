@@ -1102,20 +1102,21 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
     _, dev_calls_ms, forms_calls = time_eager_and_graph(torch, kernels, one_step_calls, max(3, steps // 2), min(warmup, 2))
     us_layer_calls = dev_calls_ms * 1e3 / (max(3, steps // 2) * layers)
 
-    # Each launch of layer 0 alone, by event pairs (eager, cold-ish: the other layers ran in between).
+    # Each kind of launch by itself: the same launch of every layer back to back between one pair of events (every
+    # layer has its own weights and cache, so the bytes come from HBM), per launch; a few ten nanoseconds of launch
+    # gap included.
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    Lw, k0, v0 = model[0]
+    scale_f = float(1.0 / np.sqrt(d))
     launches = {
-        "norm + q,k,v (one launch)": lambda: ly.gemv_multi_types([Q4, Q4, Q6], [Lw["wq"][1], Lw["wk"][1], Lw["wv"][1]],
-                                                                  [Lw.get("bq"), Lw.get("bk"), Lw.get("bv")], [bufs["q"], bufs["k"], bufs["v"]],
-                                                                  [H * d, G * d, G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
-        "rope + store + attention (two launches)": lambda: kernels.flash_attention_decode_rope_store_ind(
-            bufs["q"], bufs["k"], bufs["v"], k0, v0, bufs["attn"], H, G, d, n_ctx, dpos, float(1.0 / np.sqrt(d)), d, s["theta"],
-            None, bool(s["neox"]), angles),
-        "output projection (+=)": lambda: ly.gemv_multi(Q4, [Lw["wo"][1]], None, [bufs["x"]], [ne], bufs["attn"], None, 0.0, H * d, True),
-        "norm + gate/up + SwiGLU": lambda: ly.gemv_norm_gate_up_swiglu(Q4, Lw["ffn_gate"][1], Lw["ffn_up"][1], bufs["x"], Lw["ffn_norm"], 1e-6,
-                                                                      bufs["act"], ne, nff),
-        "down projection (+=)": lambda: ly.gemv_multi(Q6, [Lw["ffn_down"][1]], None, [bufs["x"]], [ne], bufs["act"], None, 0.0, nff, True),
+        "norm + q,k,v (one launch)": lambda Lw, k, v: ly.gemv_multi_types(
+            [Q4, Q4, Q6], [Lw["wq"][1], Lw["wk"][1], Lw["wv"][1]], [Lw.get("bq"), Lw.get("bk"), Lw.get("bv")],
+            [bufs["q"], bufs["k"], bufs["v"]], [H * d, G * d, G * d], bufs["x"], Lw["attn_norm"], 1e-6, ne),
+        "rope + store + attention (two launches)": lambda Lw, k, v: kernels.flash_attention_decode_rope_store_ind(
+            bufs["q"], bufs["k"], bufs["v"], k, v, bufs["attn"], H, G, d, n_ctx, dpos, scale_f, d, s["theta"], None, bool(s["neox"]), angles),
+        "output projection (+=)": lambda Lw, k, v: ly.gemv_multi(Q4, [Lw["wo"][1]], None, [bufs["x"]], [ne], bufs["attn"], None, 0.0, H * d, True),
+        "norm + gate/up + SwiGLU": lambda Lw, k, v: ly.gemv_norm_gate_up_swiglu(Q4, Lw["ffn_gate"][1], Lw["ffn_up"][1], bufs["x"], Lw["ffn_norm"],
+                                                                               1e-6, bufs["act"], ne, nff),
+        "down projection (+=)": lambda Lw, k, v: ly.gemv_multi(Q6, [Lw["ffn_down"][1]], None, [bufs["x"]], [ne], bufs["act"], None, 0.0, nff, True),
     }
     launch_bytes = {"norm + q,k,v (one launch)": ly.row_bytes(Q4, ne) * (H + G) * d + ly.row_bytes(Q6, ne) * G * d,
                     "rope + store + attention (two launches)": kv_bytes, "output projection (+=)": ly.row_bytes(Q4, H * d) * ne,
@@ -1123,17 +1124,27 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
     launch_us = {}
     bufs["x"].copy_(x0)
     for what, fn in launches.items():
+        g = torch.cuda.CUDAGraph()  # (a graph, so that the host's launch rate does not price the short ones)
+        try:
+            with torch.cuda.graph(g):
+                kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+                for Lw, k, v in model:
+                    fn(Lw, k, v)
+        finally:
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
         ts = []
-        for rep in range(7):
-            for dsc in descs[1:4]:  # other layers' weights through the caches in between
-                ly.decode_layer(dsc)
+        for rep in range(6):
+            torch.cuda.synchronize()
             ev[0].record()
-            fn()
+            g.replay()
             ev[1].record()
             torch.cuda.synchronize()
-            ts.append(ev[0].elapsed_time(ev[1]) * 1e3)
+            ts.append(ev[0].elapsed_time(ev[1]) * 1e3 / layers)
+        del g
+        bufs["x"].copy_(x0)  # (the accumulating launches have moved it)
         launch_us[what] = dict(us=round(float(np.median(ts)), 2), MB=round(launch_bytes[what] / 1e6, 2),
                                GBps=round(launch_bytes[what] / (float(np.median(ts)) * 1e-6) / 1e9, 1))
+    Lw, k0, v0 = model[0]
 
     # Parity: layer 0 from x0, against the oracle's operators in the reference's order (fp16 cache).
     bufs["x"].copy_(x0)
