@@ -50,24 +50,11 @@ struct Lds {
 // Digits of the (optionally normalised) activation into LDS, in groups of G elements.  Thread t takes
 // elements 8 t .. 8 t + 7 of every 2048; the G / 8 threads of a group meet by DPP moves inside their quad.
 template <int G, int kWaves>
-__device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red) {
+__device__ float stage_digits(const GemvArgs& a, unsigned char* smem, float* red) {
+    // With the RMS norm folded in, the digits are those of x * w; the norm's scalar 1 / sqrt(mean(x^2) + eps),
+    // which needs the whole vector, multiplies the finished row sums instead (returned): one pass over x.
     const int n_in = a.n_in, tid = threadIdx.x;
-    float rinv = 1.0f;
-    if (a.norm_w) {
-        float ss = 0.0f;
-        for (int e = tid * 8; e < n_in; e += kWaves * 64 * 8) {
-            const float4 u = *reinterpret_cast<const float4*>(a.x + e), v = *reinterpret_cast<const float4*>(a.x + e + 4);
-            ss += u.x * u.x + u.y * u.y + u.z * u.z + u.w * u.w + v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-        }
-        ss = wave_sum(ss);
-        if ((tid & 63) == 0) red[tid >> 6] = ss;
-        __syncthreads();
-        ss = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) ss += red[w];
-        __syncthreads();
-        rinv = 1.0f / sqrtf(ss / (float)n_in + a.eps);
-    }
+    float ss = 0.0f;
     XPair* pairs = reinterpret_cast<XPair*>(smem + Lds<G>::pairs_off(n_in));
     for (int e = tid * 8; e < n_in; e += kWaves * 64 * 8) {
         float x[8];
@@ -78,7 +65,10 @@ __device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red)
             *reinterpret_cast<float4*>(g) = *reinterpret_cast<const float4*>(a.norm_w + e);
             *reinterpret_cast<float4*>(g + 4) = *reinterpret_cast<const float4*>(a.norm_w + e + 4);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = x[i] * rinv * g[i];
+            for (int i = 0; i < 8; ++i) {
+                ss += x[i] * x[i];
+                x[i] *= g[i];
+            }
         }
         float mx = 0.0f, sum = 0.0f;
 #pragma unroll
@@ -119,7 +109,18 @@ __device__ void stage_digits(const GemvArgs& a, unsigned char* smem, float* red)
         if ((tid & (G / 8 - 1)) == 0) pairs[e / G] = XPair{scale, sum};
     }
     if (tid < 4) reinterpret_cast<unsigned*>(smem + Lds<G>::zero_off(n_in))[tid] = 0u;
+    if (!a.norm_w) {
+        __syncthreads();
+        return 1.0f;
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
+    ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) ss += red[w];
+    __syncthreads(); // (red is reused for the row sums)
+    return 1.0f / sqrtf(ss / (float)n_in + a.eps);
 }
 
 __device__ __forceinline__ float half_of(unsigned bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
@@ -378,7 +379,7 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
     request(raw_a, blockIdx.x, wave);
     __builtin_amdgcn_sched_barrier(0);
 
-    stage_digits<F::kGroup, kWaves>(a, smem, red);
+    const float rinv = stage_digits<F::kGroup, kWaves>(a, smem, red);
 
     const typename F::Addr addr = F::addr(c);
     float rowacc[M];
@@ -423,6 +424,7 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
                 v[m] = 0.0f;
 #pragma unroll
                 for (int w = 0; w < kWaves; ++w) v[m] += red[(w * M + m) * 16 + threadIdx.x];
+                v[m] *= rinv;
             }
             float y = v[0];
             if constexpr (DUAL) y = y / (1.0f + expf(-y)) * v[1]; // SiLU(gate) * up
