@@ -499,6 +499,10 @@ hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
     if (a.row_bytes == 0 || a.n_in % 32 != 0 || a.n_seg < 1 || a.n_seg > 3) return hipErrorInvalidValue;
     if (a.wgs_per_cu < 1) a.wgs_per_cu = gemv_wgs_per_cu();
     a.mfma_wgs_per_cu = gemv_mfma_wgs_per_cu();
+    {
+        static const int ks = [] { const char* e = getenv("ORIN_GEMV_KSPLIT"); return e ? atoi(e) : 0; }();
+        a.k_split_override = ks;
+    }
     if (gemv_use_mfma() && gemv_mfma_ok(type, a)) return gemv_mfma_launch(type, a, cu_count, stream);
     switch (type) {
     case kF32: return launch_type<kF32>(a, cu_count, stream);

@@ -50,20 +50,23 @@ struct Lds {
 // Digits of the (optionally normalised) activation into LDS, in groups of G elements.  Thread t takes
 // elements 8 t .. 8 t + 7 of every 2048; the G / 8 threads of a group meet by DPP moves inside their quad.
 template <int G, int kWaves>
-__device__ float stage_digits(const GemvArgs& a, unsigned char* smem, float* red) {
-    // With the RMS norm folded in, the digits are those of x * w; the norm's scalar 1 / sqrt(mean(x^2) + eps),
-    // which needs the whole vector, multiplies the finished row sums instead (returned): one pass over x.
-    const int n_in = a.n_in, tid = threadIdx.x;
+__device__ float stage_digits(const GemvArgs& a, int first, int n_in, unsigned char* smem, float* red) {
+    // Elements [first, first + n_in) of the activation.  With the RMS norm folded in (whole rows only), the
+    // digits are those of x * w; the norm's scalar 1 / sqrt(mean(x^2) + eps), which needs the whole vector,
+    // multiplies the finished row sums instead (returned): one pass over x.
+    const int tid = threadIdx.x;
+    const float* const ax = a.x + first;
+    const float* const aw = a.norm_w ? a.norm_w + first : nullptr;
     float ss = 0.0f;
     XPair* pairs = reinterpret_cast<XPair*>(smem + Lds<G>::pairs_off(n_in));
     for (int e = tid * 8; e < n_in; e += kWaves * 64 * 8) {
         float x[8];
-        *reinterpret_cast<float4*>(x) = *reinterpret_cast<const float4*>(a.x + e);
-        *reinterpret_cast<float4*>(x + 4) = *reinterpret_cast<const float4*>(a.x + e + 4);
-        if (a.norm_w) {
+        *reinterpret_cast<float4*>(x) = *reinterpret_cast<const float4*>(ax + e);
+        *reinterpret_cast<float4*>(x + 4) = *reinterpret_cast<const float4*>(ax + e + 4);
+        if (aw) {
             float g[8];
-            *reinterpret_cast<float4*>(g) = *reinterpret_cast<const float4*>(a.norm_w + e);
-            *reinterpret_cast<float4*>(g + 4) = *reinterpret_cast<const float4*>(a.norm_w + e + 4);
+            *reinterpret_cast<float4*>(g) = *reinterpret_cast<const float4*>(aw + e);
+            *reinterpret_cast<float4*>(g + 4) = *reinterpret_cast<const float4*>(aw + e + 4);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 ss += x[i] * x[i];
@@ -109,7 +112,7 @@ __device__ float stage_digits(const GemvArgs& a, unsigned char* smem, float* red
         if ((tid & (G / 8 - 1)) == 0) pairs[e / G] = XPair{scale, sum};
     }
     if (tid < 4) reinterpret_cast<unsigned*>(smem + Lds<G>::zero_off(n_in))[tid] = 0u;
-    if (!a.norm_w) {
+    if (!aw) {
         __syncthreads();
         return 1.0f;
     }
@@ -350,7 +353,12 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
     typedef typename F::Raw Raw;
     constexpr int M = DUAL ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int n_in = a.n_in, nb = n_in >> 8;
+    // gridDim.z workgroups share a tile's blocks (a matrix with few tiles and long rows, accumulating into y):
+    // this one takes blocks [b0, b0 + nb), stages that part of the activation only, and adds its row sums to
+    // y atomically.  gridDim.z = 1: the whole row, stored.
+    const int nb_row = a.n_in >> 8;
+    const int b0 = (int)blockIdx.z * nb_row / (int)gridDim.z, nb = ((int)blockIdx.z + 1) * nb_row / (int)gridDim.z - b0;
+    const int n_in = nb << 8; // (elements this workgroup works on: LDS is laid out for them)
     float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
     const GemvSeg seg = a.seg[blockIdx.y];
     const size_t row_bytes = a.n_seg_types ? seg.row_bytes : a.row_bytes;
@@ -373,13 +381,13 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
         const int row = min(tile * 16 + c.ln, seg.n_out - 1);
         b = min(b, nb - 1);
 #pragma unroll
-        for (int m = 0; m < M; ++m) F::load(wbase[m] + (size_t)row * row_bytes + (size_t)b * F::kBlockBytes, c.lg, r[m]);
+        for (int m = 0; m < M; ++m) F::load(wbase[m] + (size_t)row * row_bytes + (size_t)(b0 + b) * F::kBlockBytes, c.lg, r[m]);
     };
     Raw raw_a[M], raw_b[M];
     request(raw_a, blockIdx.x, wave);
     __builtin_amdgcn_sched_barrier(0);
 
-    const float rinv = stage_digits<F::kGroup, kWaves>(a, smem, red);
+    const float rinv = stage_digits<F::kGroup, kWaves>(a, b0 << 8, n_in, smem, red);
 
     const typename F::Addr addr = F::addr(c);
     float rowacc[M];
@@ -428,9 +436,14 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs& a) {
             }
             float y = v[0];
             if constexpr (DUAL) y = y / (1.0f + expf(-y)) * v[1]; // SiLU(gate) * up
-            if (seg.bias) y += seg.bias[r];
-            if (a.accumulate) y += seg.y[r];
-            seg.y[r] = y;
+            if (gridDim.z > 1) { // (a share of the row: y already holds what is accumulated into)
+                if (seg.bias && blockIdx.z == 0) y += seg.bias[r];
+                atomicAdd(seg.y + r, y);
+            } else {
+                if (seg.bias) y += seg.bias[r];
+                if (a.accumulate) y += seg.y[r];
+                seg.y[r] = y;
+            }
         }
         __syncthreads(); // (the partial sums are free for the next tile)
     }
@@ -466,14 +479,22 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
     // Eight waves a workgroup where the tiles would not give every SIMD a second wave and a row has the
     // blocks to share out (a down projection: few rows, long ones).
-    const bool wide = (int)(grid.x * grid.y) <= cu_count && a.n_in / 256 >= 16;
-    const size_t lds = lds_bytes<T>(a.n_in);
+    dim3 g3 = grid;
+    // A matrix with too few tiles to fill the chip whose rows are long, accumulating into y without a norm (output
+    // and down projections): 2 or 4 workgroups share a tile's blocks, each staging its own part of the activation.
+    const int nb_row = a.n_in / 256;
+    int ks = 1;
+    if (a.accumulate && !a.w_up && !a.norm_w && (int)(grid.x * grid.y) <= cu_count) ks = nb_row >= 32 ? 4 : nb_row >= 12 ? 2 : 1;
+    if (a.k_split_override > 0) ks = a.accumulate && !a.w_up && !a.norm_w ? min(a.k_split_override, nb_row) : 1;
+    g3.z = ks;
+    const bool wide = ks == 1 && (int)(grid.x * grid.y) <= cu_count && nb_row >= 16;
+    const size_t lds = lds_bytes<T>((nb_row + ks - 1) / ks * 256);
     if (a.w_up) {
-        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 8>), grid, dim3(512), lds, stream, a);
-        else hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 4>), grid, dim3(256), lds, stream, a);
+        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 8>), g3, dim3(512), lds, stream, a);
+        else hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 4>), g3, dim3(256), lds, stream, a);
     } else {
-        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 8>), grid, dim3(512), lds, stream, a);
-        else hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 4>), grid, dim3(256), lds, stream, a);
+        if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 8>), g3, dim3(512), lds, stream, a);
+        else hipLaunchKernelGGL((gemv_mfma_kernel<T, false, 4>), g3, dim3(256), lds, stream, a);
     }
     return hipGetLastError();
 }

@@ -32,7 +32,7 @@ struct GemvArgs {
     int accumulate;      // y += instead of y =
     // filled in by the launcher
     size_t row_bytes;
-    int team_waves, wgs_per_cu, mfma_wgs_per_cu, n_seg_types;
+    int team_waves, wgs_per_cu, mfma_wgs_per_cu, n_seg_types, k_split_override;
 };
 
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
