@@ -477,8 +477,6 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
     const int cap = a.mfma_wgs_per_cu > 0 ? cu_count * a.mfma_wgs_per_cu : (max_out + 15) / 16;
     const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
-    // Eight waves a workgroup where the tiles would not give every SIMD a second wave and a row has the
-    // blocks to share out (a down projection: few rows, long ones).
     dim3 g3 = grid;
     // A matrix with too few tiles to fill the chip whose rows are long, accumulating into y without a norm (output
     // and down projections): 2 or 4 workgroups share a tile's blocks, each staging its own part of the activation.
@@ -487,7 +485,9 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     if (a.accumulate && !a.w_up && !a.norm_w && (int)(grid.x * grid.y) <= cu_count) ks = nb_row >= 32 ? 4 : nb_row >= 12 ? 2 : 1;
     if (a.k_split_override > 0) ks = a.accumulate && !a.w_up && !a.norm_w ? min(a.k_split_override, nb_row) : 1;
     g3.z = ks;
-    const bool wide = ks == 1 && (int)(grid.x * grid.y) <= cu_count && nb_row >= 16;
+    // Eight waves a workgroup where a row has the blocks to share out and a workgroup has one tile only (a
+    // second tile would have amortised the staging instead).
+    const bool wide = ks == 1 && nb_row >= 16 && !a.w_up && (int)grid.x == (max_out + 15) / 16;
     const size_t lds = lds_bytes<T>((nb_row + ks - 1) / ks * 256);
     if (a.w_up) {
         if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 8>), g3, dim3(512), lds, stream, a);
@@ -518,7 +518,9 @@ hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) 
     const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
     a.n_seg_types = 1;
     const size_t lds = max(lds_bytes<kQ4_K>(a.n_in), lds_bytes<kQ6_K>(a.n_in));
-    hipLaunchKernelGGL((gemv_mfma_mixed_kernel<4>), grid, dim3(256), lds, stream, a);
+    const bool wide = a.n_in / 256 >= 16 && (int)grid.x == (max_out + 15) / 16; // (as in launch() above)
+    if (wide) hipLaunchKernelGGL((gemv_mfma_mixed_kernel<8>), grid, dim3(512), lds, stream, a);
+    else hipLaunchKernelGGL((gemv_mfma_mixed_kernel<4>), grid, dim3(256), lds, stream, a);
     return hipGetLastError();
 }
 
@@ -550,6 +552,8 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow<kQ5_K, true>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, false>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, true>()) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<8>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }
