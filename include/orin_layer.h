@@ -104,7 +104,9 @@ int orin_gemv_norm_gate_up_swiglu(int type, const void* Wg, const void* Wu, cons
  * Projections of different types take a launch each; a rotary layout the fused attention call does
  * not take (NeoX pairing with n_rot < head_dim) goes through the separate rope and store calls.
  * x is updated in place; q, k, v, attn, act (and up_tmp, needed only when ffn_gate and ffn_up
- * differ in type) are scratch the caller provides; k and v leave un-rotated / as projected. */
+ * differ in type) are scratch the caller provides; k and v leave un-rotated / as projected.
+ * A descriptor with a missing pointer or a non-positive size returns ORIN_FA_E_INVALID before
+ * anything is launched; shapes a kernel cannot take are refused by the launch that meets them. */
 typedef struct orin_decode_layer_desc {
     int n_embd, n_head, n_kv, head_dim, n_ff, n_ctx, n_rot, neox;
     float rms_eps, rope_theta, scale;

@@ -191,6 +191,8 @@ int orin_decode_layer(const orin_decode_layer_desc* L) {
     if (!L || !L->x || !L->q || !L->k || !L->v || !L->attn || !L->act || !L->attn_norm || !L->ffn_norm || !L->d_pos)
         return ORIN_FA_E_INVALID;
     if (L->n_embd <= 0 || L->n_head <= 0 || L->n_kv <= 0 || L->head_dim <= 0 || L->n_ff <= 0) return ORIN_FA_E_INVALID;
+    if (!L->wq || !L->wk || !L->wv || !L->wo || !L->ffn_gate || !L->ffn_up || !L->ffn_down || !L->kc || !L->vc) return ORIN_FA_E_INVALID;
+    if (L->gate_type != L->up_type && !L->up_tmp) return ORIN_FA_E_INVALID; // (checked here so that nothing has run when it fails)
     const int nq = L->n_head * L->head_dim, nkv = L->n_kv * L->head_dim;
     int rc;
     // ---- attn_norm + q, k, v projections: matrices of one type share a launch ----
@@ -243,7 +245,6 @@ int orin_decode_layer(const orin_decode_layer_desc* L) {
         rc = gemv_one(L->gate_type, L->ffn_gate, nullptr, L->act, L->n_ff, L->ffn_up, L->x, L->ffn_norm, L->rms_eps, L->n_embd, 0);
         if (rc != ORIN_FA_OK) return rc;
     } else {
-        if (!L->up_tmp) return ORIN_FA_E_INVALID;
         if ((rc = gemv_one(L->gate_type, L->ffn_gate, nullptr, L->act, L->n_ff, nullptr, L->x, L->ffn_norm, L->rms_eps, L->n_embd, 0)) != ORIN_FA_OK) return rc;
         if ((rc = gemv_one(L->up_type, L->ffn_up, nullptr, L->up_tmp, L->n_ff, nullptr, L->x, L->ffn_norm, L->rms_eps, L->n_embd, 0)) != ORIN_FA_OK) return rc;
         if ((rc = orin_swiglu(L->act, L->act, L->up_tmp, L->n_ff)) != ORIN_FA_OK) return rc;

@@ -90,6 +90,13 @@ VARIANTS = {
                   embd=Q8_0, output=Q4_K,
                   types=[dict(wq=Q4_K, wk=Q4_K, wv=Q4_K, wo=Q4_K, ffn_gate=Q5_K, ffn_up=Q5_K, ffn_down=Q5_K),
                          dict(wq=Q8_0, wk=Q6_K, wv=Q5_K, wo=Q6_K, ffn_gate=Q6_K, ffn_up=Q8_0, ffn_down=Q6_K)]),
+    # NeoX pairing over half the head only (the layout the fused attention call does not take), tied Q6_K embedding,
+    # gate and up of one type
+    "qwen2p": dict(arch="qwen2", seed=404, n_embd=512, n_head=4, n_kv=1, head_dim=128, n_ff=512, n_layer=2,
+                   n_vocab=72, n_rot=64, theta=1.0e4, eps=1.0e-6, bias=True, qk_norm=False, factors=False,
+                   embd=Q6_K, output=None,
+                   types=[dict(wq=Q5_K, wk=Q5_K, wv=Q5_K, wo=Q6_K, ffn_gate=Q8_0, ffn_up=Q8_0, ffn_down=Q4_K),
+                          dict(wq=Q4_K, wk=Q6_K, wv=Q6_K, wo=Q8_0, ffn_gate=Q6_K, ffn_up=Q6_K, ffn_down=Q5_K)]),
 }
 N_TOKENS = 12
 

@@ -267,6 +267,40 @@ def test_rejects_bad_arguments(ly):
             call()
 
 
+def test_decode_layer_rejects_what_it_cannot_run(ly):
+    """Missing buffers, and gate/up of different types without the scratch vector for the up product."""
+    import torch
+
+    from orin_llm_amd.kernels import OrinFaError
+
+    model = lm.build("qwen2")   # layer 0: ffn_gate Q4_K, ffn_up Q5_K
+    hp, layers, _ = upload(model)
+    bufs = make_bufs(hp)
+    kc = torch.zeros((hp["n_kv"], 32, hp["head_dim"]), dtype=torch.int16, device="cuda")
+    vc, d_pos = torch.zeros_like(kc), torch.zeros(1, dtype=torch.int32, device="cuda")
+    bufs["x"].copy_(_dev(np.linspace(-1.0, 1.0, hp["n_embd"], dtype=np.float32)))
+    x_before = bufs["x"].clone()
+    for drop in ("x", "attn", "act", "up_tmp"):
+        b = dict(bufs)
+        b[drop] = None
+        with pytest.raises(OrinFaError):
+            ly.decode_layer(ly.make_desc(hp, layers[0], b, kc, vc, d_pos, 32))
+    with pytest.raises(OrinFaError):
+        ly.decode_layer(ly.make_desc(hp, layers[0], bufs, kc, vc, None, 32))
+    with pytest.raises(OrinFaError):
+        ly.decode_layer(ly.make_desc(hp, layers[0], bufs, kc, None, d_pos, 32))
+    no_down = dict(layers[0])
+    no_down["ffn_down"] = (lm.Q6_K, None)
+    with pytest.raises(OrinFaError):
+        ly.decode_layer(ly.make_desc(hp, no_down, bufs, kc, vc, d_pos, 32))
+    desc = ly.make_desc(hp, layers[0], bufs, kc, vc, d_pos, 32)
+    desc.n_ff = 0
+    with pytest.raises(OrinFaError):
+        ly.decode_layer(desc)
+    torch.cuda.synchronize()
+    assert torch.equal(bufs["x"], x_before)   # every one of them is refused before anything is launched
+
+
 # ---------------------------------------------------------------- whole models
 
 def upload(model):
