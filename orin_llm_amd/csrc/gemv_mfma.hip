@@ -28,6 +28,8 @@
 //     in LDS at the end; blocks are requested one iteration ahead, across row tiles.
 #include "layer_common.hpp"
 
+#include <stdlib.h>
+
 namespace orin_fa {
 namespace {
 
@@ -47,8 +49,51 @@ struct Lds {
     static __host__ __device__ size_t bytes(int n_in) { return (size_t)red_off(n_in) + kMaxWaves * 2 * 16 * 4; }
 };
 
+// Eight consecutive elements (x, already multiplied by the norm's weights) of a group of G into the digit planes;
+// the G / 8 threads of a group sit in one quad (n_in is a multiple of 32, so a quad is never split) and meet
+// by DPP moves.
+template <int G>
+__device__ __forceinline__ void digits8(const float (&x)[8], int e, int n_in, unsigned char* smem, XPair* pairs, int tid) {
+    float mx = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        mx = fmaxf(mx, fabsf(x[i]));
+        sum += x[i];
+    }
+    mx = fmaxf(mx, dpp_xor_step(mx, 0));
+    sum += dpp_xor_step(sum, 0);
+    if constexpr (G == 32) {
+        mx = fmaxf(mx, dpp_xor_step(mx, 1));
+        sum += dpp_xor_step(sum, 1);
+    }
+    const float scale = mx > 0.0f ? mx / kDigitRange : 1.0f;
+    const float inv = 1.0f / scale;
+    // X + 0x808080 carries 128 into each of the three byte positions, so its bytes are the signed
+    // digits plus 128 (byte k of X + 0x808080 is ((X >> 8 k) + 128) & 255 with the lower digits'
+    // carries already taken out); the exclusive-or takes the 128 off again, byte by byte.
+    unsigned z[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = ((unsigned)((int)rintf(x[i] * inv)) + 0x808080u) ^ 0x808080u;
+    // byte k of four consecutive elements into one word of plane 2 - k (plane 0 holds the top digits)
+    u32x2 plane[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const unsigned pick = (unsigned)k | ((unsigned)(4 + k) << 8); // byte k of the second operand, then of the first
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            const unsigned t01 = __builtin_amdgcn_perm(z[4 * w + 1], z[4 * w + 0], pick);
+            const unsigned t23 = __builtin_amdgcn_perm(z[4 * w + 3], z[4 * w + 2], pick);
+            plane[2 - k][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+        }
+    }
+    *reinterpret_cast<u32x2*>(smem + e) = plane[0];
+    *reinterpret_cast<u32x2*>(smem + n_in + e) = plane[1];
+    *reinterpret_cast<u32x2*>(smem + 2 * n_in + e) = plane[2];
+    if ((tid & (G / 8 - 1)) == 0) pairs[e / G] = XPair{scale, sum};
+}
+
 // Digits of the (optionally normalised) activation into LDS, in groups of G elements.  Thread t takes
-// elements 8 t .. 8 t + 7 of every 2048; the G / 8 threads of a group meet by DPP moves inside their quad.
+// elements 8 t .. 8 t + 7 of every kWaves * 512.
 template <int G, int kWaves>
 __device__ float stage_digits(const GemvArgs& a, int first, int n_in, unsigned char* smem, float* red) {
     // Elements [first, first + n_in) of the activation.  With the RMS norm folded in (whole rows only), the
@@ -73,43 +118,7 @@ __device__ float stage_digits(const GemvArgs& a, int first, int n_in, unsigned c
                 x[i] *= g[i];
             }
         }
-        float mx = 0.0f, sum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            mx = fmaxf(mx, fabsf(x[i]));
-            sum += x[i];
-        }
-        // a group's threads sit in one quad (n_in is a multiple of 32, so a quad is never split)
-        mx = fmaxf(mx, dpp_xor_step(mx, 0));
-        sum += dpp_xor_step(sum, 0);
-        if constexpr (G == 32) {
-            mx = fmaxf(mx, dpp_xor_step(mx, 1));
-            sum += dpp_xor_step(sum, 1);
-        }
-        const float scale = mx > 0.0f ? mx / kDigitRange : 1.0f;
-        const float inv = 1.0f / scale;
-        // X + 0x808080 carries 128 into each of the three byte positions, so its bytes are the signed
-        // digits plus 128 (byte k of X + 0x808080 is ((X >> 8 k) + 128) & 255 with the lower digits'
-        // carries already taken out); the exclusive-or takes the 128 off again, byte by byte.
-        unsigned z[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) z[i] = ((unsigned)((int)rintf(x[i] * inv)) + 0x808080u) ^ 0x808080u;
-        // byte k of four consecutive elements into one word of plane 2 - k (plane 0 holds the top digits)
-        u32x2 plane[3];
-#pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            const unsigned pick = (unsigned)k | ((unsigned)(4 + k) << 8); // byte k of the second operand, then of the first
-#pragma unroll
-            for (int w = 0; w < 2; ++w) {
-                const unsigned t01 = __builtin_amdgcn_perm(z[4 * w + 1], z[4 * w + 0], pick);
-                const unsigned t23 = __builtin_amdgcn_perm(z[4 * w + 3], z[4 * w + 2], pick);
-                plane[2 - k][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
-            }
-        }
-        *reinterpret_cast<u32x2*>(smem + e) = plane[0];
-        *reinterpret_cast<u32x2*>(smem + n_in + e) = plane[1];
-        *reinterpret_cast<u32x2*>(smem + 2 * n_in + e) = plane[2];
-        if ((tid & (G / 8 - 1)) == 0) pairs[e / G] = XPair{scale, sum};
+        digits8<G>(x, e, n_in, smem, pairs, tid);
     }
     if (tid < 4) reinterpret_cast<unsigned*>(smem + Lds<G>::zero_off(n_in))[tid] = 0u;
     if (!aw) {
@@ -126,6 +135,15 @@ __device__ float stage_digits(const GemvArgs& a, int first, int n_in, unsigned c
     return 1.0f / sqrtf(ss / (float)n_in + a.eps);
 }
 
+// A workgroup barrier that waits for this wave's LDS traffic only: weight requests in flight stay in flight.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// 16-byte loads of the kernels that fetch 64 bytes of each of 16 rows per instruction: ordinary ones, because the
+// neighbouring pieces of a line are fetched by other instructions and meet in the CU's cache (as streaming loads,
+// which pass that cache, these kernels take half as long again).  p may be 2-byte aligned.
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+__device__ __forceinline__ u32x4 load16(const unsigned char* p) { return *reinterpret_cast<const u32x4_a2*>(p); }
+__device__ __forceinline__ u32x4 load16_aligned(const unsigned char* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ float half_of(unsigned bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
 __device__ __forceinline__ unsigned from_lane(int src_lane4, unsigned v) {
     return (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)v);
@@ -163,10 +181,10 @@ struct MFK45 {
         int lo_base, hi_base, lo_step, hi_step; // LDS byte offsets of this lane's A operands; a lane whose row is zero reads the 16 zero bytes, stride 0
     };
     static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
-        r.hdr = *reinterpret_cast<const u32x4*>(blk);
-        if constexpr (FIVE) r.qh = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * (lg & 1));
-        r.q1 = *reinterpret_cast<const u32x4*>(blk + kQs + 16 * lg);
-        r.q2 = *reinterpret_cast<const u32x4*>(blk + kQs + 64 + 16 * lg);
+        r.hdr = load16_aligned(blk);
+        if constexpr (FIVE) r.qh = load16_aligned(blk + 16 + 16 * (lg & 1));
+        r.q1 = load16_aligned(blk + kQs + 16 * lg);
+        r.q2 = load16_aligned(blk + kQs + 64 + 16 * lg);
     }
     static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
         const int ap = c.am >> 2, ad = c.am & 3, g = c.g;
@@ -181,27 +199,36 @@ struct MFK45 {
         const unsigned mine = ((r.hdr.y >> (8 * c.lg)) & 0xffu) | (((r.hdr.z >> (8 * c.lg)) & 0xffu) << 8) |
                               (((r.hdr.w >> (8 * c.lg)) & 0xffu) << 16);
         const unsigned dd = from_lane(c.src_lane4, r.hdr.x), bb = from_lane(c.src_lane4, mine);
+        u32x4 fifth = {0u, 0u, 0u, 0u}, q1, q2;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (FIVE) fifth[i] = from_lane(c.src_lane4, r.qh[i]) >> (2 * (c.g >> 1));
+            q1[i] = from_lane(c.src_lane4, r.q1[i]);
+            q2[i] = from_lane(c.src_lane4, r.q2[i]);
+        }
+        return math(dd, bb, q1, q2, fifth, c, ad, b);
+    }
+    // In lane (n, g): dd = the block's two fp16 scales, bb = bytes g of the three words of packed six-bit pairs,
+    // q1 / q2 = piece g of each half of the nibbles, fifth = the fifth bits of this lane's elements shifted down
+    // to bit 0 (Q5_K).
+    static __device__ __forceinline__ float math(unsigned dd, unsigned bb, const u32x4& q1, const u32x4& q2, const u32x4& fifth,
+                                                 const LaneCtx& c, const Addr& ad, int b) {
         const float d = half_of(dd & 0xffffu), dmin = half_of(dd >> 16);
         const unsigned b0 = bb & 0xffu, b1 = (bb >> 8) & 0xffu, b2 = (bb >> 16) & 0xffu;
         // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
         const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
         const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
-        u32x4 fifth = {0u, 0u, 0u, 0u};
-        if constexpr (FIVE) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fifth[i] = from_lane(c.src_lane4, r.qh[i]) >> (2 * (c.g >> 1));
-        }
         float out = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + ad.lo_base + b * ad.lo_step + (ad.lo_step ? 128 * h : 0));
             const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + ad.hi_base + b * ad.hi_step + (ad.hi_step ? 128 * h : 0));
             const XPair xp = c.pairs[8 * b + 4 * h + c.g];
-            const u32x4 qs = h ? r.q2 : r.q1;
+            const u32x4 qs = h ? q2 : q1;
             i32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const unsigned q = from_lane(c.src_lane4, qs[i]);
+                const unsigned q = qs[i];
                 unsigned l = q & 0x0f0f0f0fu, u = (q >> 4) & 0x0f0f0f0fu;
                 if constexpr (FIVE) { // sub-blocks 4 h + 2 (g / 2) and + 1: bits 4 h and 4 h + 1 of the shifted bytes
                     const unsigned f = fifth[i] >> (4 * h);
@@ -245,7 +272,7 @@ struct MF<kQ8_0> {
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
             for (int run = 0; run < 2; ++run)
-                r.q[h][run] = reinterpret_cast<const Loose<u32x4>*>(blk + 34 * (4 * h + 2 * run + (lg >> 1)) + 2 + 16 * (lg & 1))->v;
+                r.q[h][run] = load16(blk + 34 * (4 * h + 2 * run + (lg >> 1)) + 2 + 16 * (lg & 1));
             r.d[h] = *reinterpret_cast<const uint16_t*>(blk + 34 * (4 * h + lg));
         }
     }
@@ -301,10 +328,10 @@ struct MF<kQ6_K> {
     static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            r.ql[h] = reinterpret_cast<const Loose<u32x4>*>(blk + 64 * h + 16 * lg)->v;
-            r.qh[h] = reinterpret_cast<const Loose<u32x4>*>(blk + 128 + 32 * h + 16 * (lg & 1))->v;
+            r.ql[h] = load16(blk + 64 * h + 16 * lg);
+            r.qh[h] = load16(blk + 128 + 32 * h + 16 * (lg & 1));
         }
-        r.sc = reinterpret_cast<const Loose<u32x4>*>(blk + 192)->v;
+        r.sc = load16(blk + 192);
         r.d = *reinterpret_cast<const uint16_t*>(blk + 208);
     }
     static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
@@ -454,6 +481,253 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
     gemv_mfma_body<T, DUAL, kWaves>(a);
 }
 
+// Q4_K and Q5_K rows read in long runs.  The kernel above fetches, per load instruction, 64 bytes of each of 16
+// rows; this machine's memory path moves that pattern at 4.4 TB/s where lane-linear runs of 288 bytes move at
+// 5.4 TB/s and of 576 bytes at 5.5 TB/s (a read-only stand-in with these patterns over the 66 MB of a Llama-3-8B
+// gate/up pair: 15.0, 12.3 and 11.9 us a launch; a plain read 12.3, with streaming loads 11.0).  Here a wave's
+// item is CB consecutive blocks of each of a tile's 16 rows, of one matrix, fetched as (row, 16-byte piece) slots
+// in row-major order, lane after lane, with streaming loads: runs of CB * 144 (176) bytes, every line requested by
+// one instruction.  The pieces pass through a wave-private LDS buffer (rows padded to an odd number of pieces, so
+// that the 16 rows a matrix-instruction operand is read from lie in 16 different bank groups) and come back in
+// the matrix instruction's lane order: no lane permutations.  Two items per wave are on their way or in use;
+// chunks w, w + kWaves, ... of a tile's blocks are wave w's, and so are those chunks' digits of the activation,
+// which the wave makes for itself: no wave waits for another before the first tile's end, where the norm's sum
+// of squares is put together as well.  Barriers wait for LDS only, row sums leave through stores and atomic adds
+// without a return value, a tile's bias values travel with its items: nothing in the loop waits for anything but
+// the oldest item.  Requires whole 16-row tiles.  (Deeper request queues, three and four items a wave, were
+// slower in both kernels: what bounds them after the loads is the vector ALU, about 95 instructions per block
+// and wave for the nibbles, the six-bit pairs and the digit sums.)
+constexpr int kRowsMaxCb = 2; // blocks of a row in an item, at most
+constexpr int kRowsRedBytes = 2 * kMaxWaves * 2 * 16 * 4 + 64; // two sets of partial row sums (tiles alternate: one barrier a tile), the waves' sums of squares
+
+template <bool FIVE, int CB>
+struct RowsGeom {
+    static constexpr int P = MFK45<FIVE>::kBlockBytes / 16; // pieces of a block
+    static constexpr int kRowPieces = CB * P;                // pieces of a row in an item
+    static constexpr int R = kRowPieces | 1;                 // LDS row stride, pieces
+    static constexpr int NL = (16 * kRowPieces + 63) / 64;   // load instructions an item
+    static constexpr int kWaveBytes = (16 * R + 1) * 16;     // (one more piece: where lanes past the item's end write)
+    static __host__ __device__ size_t lds_bytes(int n_in, int waves) {
+        return (size_t)Lds<32>::red_off(n_in) + kRowsRedBytes + (size_t)waves * kWaveBytes;
+    }
+};
+
+template <bool FIVE, bool DUAL, int kWaves, int CB>
+__device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
+    using F = MFK45<FIVE>;
+    using L = Lds<32>;
+    using G = RowsGeom<FIVE, CB>;
+    constexpr int M = DUAL ? 2 : 1, P = G::P, R = G::R, NL = G::NL;
+    constexpr int kQ = F::kQs / 16; // piece of a block's first nibbles
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int nb_row = a.n_in >> 8;
+    const int b0 = (int)blockIdx.z * nb_row / (int)gridDim.z, nb = ((int)blockIdx.z + 1) * nb_row / (int)gridDim.z - b0;
+    const int n_in = nb << 8;
+    float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
+    const GemvSeg seg = a.seg[blockIdx.y];
+    const unsigned row_bytes = (unsigned)a.row_bytes;
+    const int n_tiles = seg.n_out >> 4;
+    if ((int)blockIdx.x >= n_tiles) return; // (whole workgroup: a shorter matrix of a shared launch)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // (scalar: what follows from it stays in scalar registers)
+    unsigned char* const transit = smem + L::red_off(n_in) + kRowsRedBytes + wave * G::kWaveBytes;
+    LaneCtx c;
+    c.n = lane & 15; c.g = lane >> 4; c.ln = 0; c.lg = 0; c.src_lane4 = 0;
+    c.am = lane & 15;
+    c.smem = smem;
+    c.pairs = reinterpret_cast<const XPair*>(smem + L::pairs_off(n_in));
+    c.n_in = n_in;
+    c.zero_off = L::zero_off(n_in);
+    const unsigned char* const wbase[2] = {static_cast<const unsigned char*>(seg.w),
+                                           static_cast<const unsigned char*>(DUAL ? a.w_up : seg.w)};
+    const int n_chunks = (nb + CB - 1) / CB;
+    const int my_chunks = wave < n_chunks ? (n_chunks - wave + kWaves - 1) / kWaves : 0;
+    const int n_mine = (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int total = n_mine * my_chunks * M;
+    // slot 64 i + lane of an item: (row, piece), row-major
+    unsigned goff[NL];
+    int loff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int s = 64 * i + lane, row = s / G::kRowPieces, piece = s - row * G::kRowPieces;
+        goff[i] = row < 16 ? (unsigned)row * row_bytes + (unsigned)piece * 16u : 0xffffffffu; // (past the end: cut to the item's last piece below)
+        loff[i] = row < 16 ? (row * R + piece) * 16 : 16 * R * 16;
+    }
+
+    // ---- requests ----
+    int rq_tile = blockIdx.x, rq_c = wave;
+    constexpr int kRing = 2; // items on their way or in use (M divides it: an item's matrix is its slot's)
+    u32x4 buf[kRing][NL];
+    float bias_v[kRing];
+    auto request = [&](u32x4 (&r)[NL], float& bias, int m) {
+        const int cb = min(CB, nb - rq_c * CB);
+        // pieces past the chunk's end in rows above the last are the row's next blocks or the next row's first (fetched,
+        // never used); in the last row they are cut to the last piece
+        const unsigned limit = 15u * row_bytes + (unsigned)(cb * P - 1) * 16u;
+        const unsigned char* const base = wbase[m] + (size_t)rq_tile * 16 * row_bytes + (size_t)(b0 + rq_c * CB) * F::kBlockBytes;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + min(goff[i], limit))) /* whole runs, read once: streaming */;
+        }
+        bias = *(seg.bias ? seg.bias + rq_tile * 16 + c.n : a.x); // (always a load: the same count on every path)
+        if (m == M - 1) {
+            rq_c += kWaves;
+            if (rq_c >= n_chunks) {
+                rq_c = wave;
+                rq_tile += (int)gridDim.x;
+            }
+        }
+    };
+    // ---- the activation's digits: every wave makes those of its own chunks (it multiplies no others), so
+    // nothing waits for another wave before the first tile's end; the norm's sum of squares is put together
+    // there.  The first chunk's loads go out ahead of the weight requests (loads return in order). ----
+    float* const wave_ss = red + 2 * kMaxWaves * 2 * 16;
+    {
+        const float* const ax = a.x + (b0 << 8);
+        const float* const aw = a.norm_w ? a.norm_w + (b0 << 8) : nullptr;
+        XPair* const pairs = reinterpret_cast<XPair*>(smem + L::pairs_off(n_in));
+        float ss = 0.0f;
+        auto fetch = [&](const float* p, int e, float (&v)[8]) {
+            *reinterpret_cast<float4*>(v) = *reinterpret_cast<const float4*>(p + e);
+            *reinterpret_cast<float4*>(v + 4) = *reinterpret_cast<const float4*>(p + e + 4);
+        };
+        auto digits = [&](float (&x)[8], const float (&g)[8], int e) {
+            if (aw) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    ss += x[i] * x[i];
+                    x[i] *= g[i];
+                }
+            }
+            digits8<32>(x, e, n_in, smem, pairs, lane);
+        };
+        constexpr int kPasses = (CB * 256 + 511) / 512; // 512 elements a pass
+        float x0[kPasses][8] = {}, g0[kPasses][8] = {};
+        const int first_end = min((wave + 1) * CB * 256, n_in);
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const int e = wave * CB * 256 + ps * 512 + lane * 8;
+            if (e < first_end) {
+                fetch(ax, e, x0[ps]);
+                if (aw) fetch(aw, e, g0[ps]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kRing; ++j)
+            if (j < total) request(buf[j], bias_v[j], j % M);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ps = 0; ps < kPasses; ++ps) {
+            const int e = wave * CB * 256 + ps * 512 + lane * 8;
+            if (e < first_end) digits(x0[ps], g0[ps], e);
+        }
+        for (int ch = wave + kWaves; ch < n_chunks; ch += kWaves) { // (rows longer than kWaves chunks: these loads queue behind the weights)
+            const int end = min((ch + 1) * CB * 256, n_in);
+            for (int e = ch * CB * 256 + lane * 8; e < end; e += 512) {
+                float x[8], g[8] = {};
+                fetch(ax, e, x);
+                if (aw) fetch(aw, e, g);
+                digits(x, g, e);
+            }
+        }
+        if (lane < 4) reinterpret_cast<unsigned*>(smem + L::zero_off(n_in))[lane] = 0u; // (every wave writes the same zeros)
+        ss = wave_sum(ss);
+        if (lane == 0) wave_ss[wave] = ss;
+    }
+    const bool has_norm = a.norm_w != nullptr;
+    const float norm_n = (float)n_in, norm_eps = a.eps;
+
+    const typename F::Addr addr = F::addr(c);
+    int set = 0;
+    auto tile_end = [&](int tile, const float (&rowacc)[M], float bias) {
+        float* const mine = red + set * (kMaxWaves * 2 * 16);
+        set ^= 1;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float t = xor_sum(rowacc[m]);
+            if (c.g == 0) mine[(wave * M + m) * 16 + c.n] = t;
+        }
+        lds_barrier();
+        if (threadIdx.x < 16) {
+            const int r = tile * 16 + (int)threadIdx.x;
+            float rinv = 1.0f;
+            if (has_norm) { // (every wave has left its sum of squares before its first barrier here)
+                float ss = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) ss += wave_ss[w];
+                rinv = 1.0f / sqrtf(ss / norm_n + norm_eps);
+            }
+            float v[M];
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                v[m] = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) v[m] += mine[(w * M + m) * 16 + threadIdx.x];
+                v[m] *= rinv;
+            }
+            float y = v[0];
+            if constexpr (DUAL) y = y / (1.0f + expf(-y)) * v[1]; // SiLU(gate) * up
+            if (seg.bias && blockIdx.z == 0) y += bias;
+            if (gridDim.z > 1 || a.accumulate) atomicAdd(seg.y + r, y); // (one writer a row and share: with one share the sum is the plain one)
+            else seg.y[r] = y;
+        }
+    };
+    if (my_chunks == 0) { // (fewer chunks than waves: this wave only keeps the barriers' count)
+        const float zero[M] = {};
+        for (int t = 0; t < n_mine; ++t) tile_end((int)blockIdx.x + t * (int)gridDim.x, zero, 0.0f);
+        return;
+    }
+    int cs_tile = blockIdx.x, cs_c = wave;
+    float rowacc[M] = {};
+    auto consume = [&](const u32x4 (&r)[NL], float bias, int m) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(transit + loff[i]) = r[i];
+        const int cb = min(CB, nb - cs_c * CB);
+        float v = 0.0f;
+        for (int j = 0; j < cb; ++j) {
+            const unsigned char* const blk = transit + (c.n * R + j * P) * 16;
+            const u32x4 hdr = *reinterpret_cast<const u32x4*>(blk);
+            const u32x4 q1 = *reinterpret_cast<const u32x4*>(blk + (kQ + c.g) * 16);
+            const u32x4 q2 = *reinterpret_cast<const u32x4*>(blk + (kQ + 4 + c.g) * 16);
+            u32x4 fifth = {0u, 0u, 0u, 0u};
+            if constexpr (FIVE) fifth = *reinterpret_cast<const u32x4*>(blk + (1 + (c.g & 1)) * 16) >> (unsigned)(2 * (c.g >> 1));
+            const unsigned bb = ((hdr.y >> (8 * c.g)) & 0xffu) | (((hdr.z >> (8 * c.g)) & 0xffu) << 8) | (((hdr.w >> (8 * c.g)) & 0xffu) << 16);
+            v += F::math(hdr.x, bb, q1, q2, fifth, c, addr, cs_c * CB + j);
+        }
+        rowacc[m] += v;
+        if (m == M - 1) {
+            cs_c += kWaves;
+            if (cs_c >= n_chunks) {
+                tile_end(cs_tile, rowacc, bias);
+                cs_c = wave;
+                cs_tile += (int)gridDim.x;
+#pragma unroll
+                for (int mm = 0; mm < M; ++mm) rowacc[mm] = 0.0f;
+            }
+        }
+    };
+    // Steady state: every item consumed is followed by the request kRing items on, which exists: no branch around
+    // a load, so the compiler's wait counts are exact.
+    int k = 0;
+    for (; k + 2 * kRing <= total; k += kRing) {
+#pragma unroll
+        for (int j = 0; j < kRing; ++j) {
+            consume(buf[j], bias_v[j], j % M);
+            request(buf[j], bias_v[j], j % M);
+        }
+    }
+    // the last two or three items (or the only one)
+    if (k < total) consume(buf[0], bias_v[0], 0);
+    if (k + 2 < total) request(buf[0], bias_v[0], 0);
+    if (k + 1 < total) consume(buf[1], bias_v[1], M - 1);
+    if (k + 2 < total) consume(buf[0], bias_v[0], 0);
+}
+
+template <bool FIVE, bool DUAL, int kWaves, int CB>
+__global__ __launch_bounds__(kWaves * 64) void gemv_rows_kernel(const GemvArgs a) {
+    gemv_rows_body<FIVE, DUAL, kWaves, CB>(a);
+}
+
 // Matrices of different block types in one launch (the q, k, v projections of a file that keeps attn_v in
 // Q6_K): a workgroup belongs to one matrix and runs that matrix's code.
 template <int kWaves>
@@ -470,6 +744,45 @@ constexpr size_t kMfmaLdsMax = 96u * 1024u;
 
 template <int T>
 size_t lds_bytes(int n_in) { return Lds<MF<T>::kGroup>::bytes(n_in); }
+
+// The long-run kernel where it applies: Q4_K / Q5_K, whole 16-row tiles, LDS within the limit.
+bool rows_enabled() {
+    static const bool on = getenv("ORIN_GEMV_NO_ROWS") == nullptr;
+    return on;
+}
+// Its workgroups per CU: three (staging is each wave's own business there, so a workgroup more costs little and
+// hides more of the others' waits); ORIN_GEMV_MFMA_WGS_PER_CU overrides as for the other kernel.
+int rows_wgs_per_cu(int given) {
+    static const bool env = getenv("ORIN_GEMV_MFMA_WGS_PER_CU") != nullptr;
+    return env ? given : 3;
+}
+
+template <bool FIVE, bool DUAL, int kWaves, int CB>
+bool launch_rows_as(const GemvArgs& a, dim3 grid, int n_in_wg, hipStream_t stream) {
+    const size_t lds = RowsGeom<FIVE, CB>::lds_bytes(n_in_wg, kWaves);
+    if (lds > kMfmaLdsMax) return false;
+    hipLaunchKernelGGL((gemv_rows_kernel<FIVE, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, a);
+    return true;
+}
+
+template <bool FIVE>
+bool launch_rows(const GemvArgs& a, dim3 grid, bool wide, int nb_wg, hipStream_t stream) {
+    if (!rows_enabled()) return false;
+    for (int i = 0; i < a.n_seg; ++i)
+        if (a.seg[i].n_out % 16 != 0) return false;
+    const int n_in_wg = nb_wg * 256;
+    if (wide) { // (eight waves: never two matrices)
+        return (nb_wg + 7) / 8 <= 1 ? launch_rows_as<FIVE, false, 8, 1>(a, grid, n_in_wg, stream)
+                                    : launch_rows_as<FIVE, false, 8, 2>(a, grid, n_in_wg, stream);
+    }
+    // runs of 288 (352) bytes read within a few percent of longer ones, and the wave's last item, which nothing
+    // overlaps, is half as long as with four blocks
+    const int cb = min(kRowsMaxCb, (nb_wg + 3) / 4);
+    if (a.w_up) {
+        return cb == 1 ? launch_rows_as<FIVE, true, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<FIVE, true, 4, 2>(a, grid, n_in_wg, stream);
+    }
+    return cb == 1 ? launch_rows_as<FIVE, false, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<FIVE, false, 4, 2>(a, grid, n_in_wg, stream);
+}
 
 template <int T>
 hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
@@ -488,6 +801,13 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     // Eight waves a workgroup where a row has the blocks to share out and a workgroup has one tile only (a
     // second tile would have amortised the staging instead).
     const bool wide = ks == 1 && nb_row >= 16 && !a.w_up && (int)grid.x == (max_out + 15) / 16;
+    if constexpr (T == kQ4_K || T == kQ5_K) {
+        const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu);
+        dim3 gr = g3;
+        gr.x = min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16);
+        const bool wide_r = ks == 1 && nb_row >= 16 && !a.w_up && (int)gr.x == (max_out + 15) / 16;
+        if (launch_rows<T == kQ5_K>(a, gr, wide_r, (nb_row + ks - 1) / ks, stream)) return hipGetLastError();
+    }
     const size_t lds = lds_bytes<T>((nb_row + ks - 1) / ks * 256);
     if (a.w_up) {
         if (wide) hipLaunchKernelGGL((gemv_mfma_kernel<T, true, 8>), g3, dim3(512), lds, stream, a);
@@ -506,6 +826,23 @@ hipError_t allow() {
     if (e != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_kernel<T, DUAL, 8>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+}
+
+template <bool FIVE, bool DUAL, int kWaves, int CB>
+hipError_t allow_rows() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_kernel<FIVE, DUAL, kWaves, CB>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+}
+
+template <bool FIVE>
+hipError_t allow_rows_all() {
+    hipError_t e;
+    if ((e = allow_rows<FIVE, false, 8, 1>()) != hipSuccess) return e;
+    if ((e = allow_rows<FIVE, false, 8, 2>()) != hipSuccess) return e;
+    if ((e = allow_rows<FIVE, false, 4, 1>()) != hipSuccess) return e;
+    if ((e = allow_rows<FIVE, false, 4, 2>()) != hipSuccess) return e;
+    if ((e = allow_rows<FIVE, true, 4, 1>()) != hipSuccess) return e;
+    return allow_rows<FIVE, true, 4, 2>();
 }
 
 } // namespace
@@ -552,6 +889,8 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow<kQ5_K, true>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, false>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, true>()) != hipSuccess) return e;
+    if ((e = allow_rows_all<false>()) != hipSuccess) return e;
+    if ((e = allow_rows_all<true>()) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<8>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),

@@ -213,6 +213,51 @@ def test_projections_of_different_types(ly, unit, wtypes, n_in):
         assert vec_err(got[:n], w_.astype(np.float64)) < TOL_OP and (got[n:] == 12345.0).all()
 
 
+# Q4_K / Q5_K matrices made of whole 16-row tiles go to the kernel that reads rows in long runs: 1 ... 74 blocks
+# per row (one or two blocks per item, chunks shared among four or eight waves, ragged last chunks), few and many
+# tiles (one per workgroup, several per workgroup), every epilogue.
+LONG_RUN_SHAPES = [(256, 48), (512, 16), (1536, 12800), (1792, 64), (3584, 512), (4096, 4096), (8960, 96), (14336, 256), (18944, 32)]
+
+
+@pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q5_K])
+@pytest.mark.parametrize("n_in,n_out", LONG_RUN_SHAPES)
+def test_whole_tiles_in_long_runs(ly, wtype, n_in, n_out):
+    import torch
+
+    ly.use_matrix_cores(True)
+    rs = lm.Stream(7000 + wtype * 131 + n_in + n_out)
+    t = lm.make_tensor(rs, wtype, n_in, n_out)
+    x = rs.sym(n_in, 1.0)
+    nw = (1.0 + rs.sym(n_in, 0.3)).astype(np.float32)
+    bias, y0 = rs.sym(n_out, 0.5), rs.sym(n_out, 1.0)
+    w, dx = dev_bytes(t[1]), _dev(x)
+    plain = ref.gemv(wtype, t[1], x, n_in, n_out).astype(np.float64)
+    normed = ref.gemv(wtype, t[1], ref.rms_norm(x, nw, 1e-5), n_in, n_out).astype(np.float64)
+    errs = {}
+    y = out_buf(n_out)
+    ly.gemv(wtype, w, dx, y, n_in, n_out)
+    errs["plain"] = (y, plain)
+    yb = out_buf(n_out)
+    ly.gemv_multi(wtype, [w], [_dev(bias)], [yb], [n_out], dx, _dev(nw), 1e-5, n_in)
+    errs["norm + bias"] = (yb, normed + bias)
+    ya = _dev(np.concatenate([y0, np.full(4, 12345.0, np.float32)]))
+    ly.gemv_multi(wtype, [w], None, [ya], [n_out], dx, None, 0.0, n_in, True)   # (few tiles and long rows: shares of a row)
+    errs["accumulate"] = (ya, plain + y0)
+    if n_out <= 4096:
+        up = lm.make_tensor(rs, wtype, n_in, n_out)
+        yg = out_buf(n_out)
+        ly.gemv_norm_gate_up_swiglu(wtype, w, dev_bytes(up[1]), dx, _dev(nw), 1e-5, yg, n_in, n_out)
+        u = ref.gemv(wtype, up[1], ref.rms_norm(x, nw, 1e-5), n_in, n_out)
+        errs["gate/up"] = (yg, ref.swiglu(normed.astype(np.float32), u).astype(np.float64))
+    torch.cuda.synchronize()
+    for what, (got_t, want) in errs.items():
+        got = got_t.cpu().numpy()
+        assert (got[n_out:] == 12345.0).all(), f"{what}: rows past n_out were written"
+        e = vec_err(got[:n_out], want)
+        print(f"{lm.TYPE_NAME[wtype]} {n_in} x {n_out} {what}: err {e:.2e}", flush=True)
+        assert e < TOL_OP, what
+
+
 def test_rms_norm_rows_swiglu_and_in_place(ly):
     import torch
 
