@@ -208,6 +208,20 @@ struct MFK45 {
         }
         return math(dd, bb, q1, q2, fifth, c, ad, b);
     }
+    // A block laid out in LDS piece after piece (the kernel that reads rows in long runs): piece k is the block's
+    // bytes 16 k ...
+    static constexpr int kPieces = kBlockBytes / 16;
+    static constexpr bool kAligned = true;
+    static __host__ __device__ constexpr int piece_off(int k) { return 16 * k; }
+    static __device__ __forceinline__ float from_lds(const unsigned char* blk, const LaneCtx& c, const Addr& ad, int b) {
+        const u32x4 hdr = *reinterpret_cast<const u32x4*>(blk);
+        const u32x4 q1 = *reinterpret_cast<const u32x4*>(blk + kQs + 16 * c.g);
+        const u32x4 q2 = *reinterpret_cast<const u32x4*>(blk + kQs + 64 + 16 * c.g);
+        u32x4 fifth = {0u, 0u, 0u, 0u};
+        if constexpr (FIVE) fifth = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * (c.g & 1)) >> (unsigned)(2 * (c.g >> 1));
+        const unsigned bb = ((hdr.y >> (8 * c.g)) & 0xffu) | (((hdr.z >> (8 * c.g)) & 0xffu) << 8) | (((hdr.w >> (8 * c.g)) & 0xffu) << 16);
+        return math(hdr.x, bb, q1, q2, fifth, c, ad, b);
+    }
     // In lane (n, g): dd = the block's two fp16 scales, bb = bytes g of the three words of packed six-bit pairs,
     // q1 / q2 = piece g of each half of the nibbles, fifth = the fifth bits of this lane's elements shifted down
     // to bit 0 (Q5_K).
@@ -344,7 +358,42 @@ struct MF<kQ6_K> {
         const unsigned mine = ((r.sc.x >> (8 * c.lg)) & 0xffu) | (((r.sc.y >> (8 * c.lg)) & 0xffu) << 8) |
                               (((r.sc.z >> (8 * c.lg)) & 0xffu) << 16) | (((r.sc.w >> (8 * c.lg)) & 0xffu) << 24);
         const unsigned ss = from_lane(c.src_lane4, mine);
-        const float d = half_of(from_lane(c.src_lane4, r.d));
+        const unsigned dd = from_lane(c.src_lane4, r.d);
+        u32x4 ql[2], qh[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ql[h][i] = from_lane(c.src_lane4, r.ql[h][i]);
+                qh[h][i] = from_lane(c.src_lane4, r.qh[h][i]);
+            }
+        }
+        return math(ss, dd, ql, qh, c, ad, b);
+    }
+    // A block laid out in LDS piece after piece (the kernel that reads rows in long runs): pieces 0 ... 12 are the
+    // block's bytes 16 k ..., piece 13 its last 16 bytes (194 ... 209: the fp16 scale in its last two), so that no
+    // piece reaches past the block.
+    static constexpr int kPieces = 14;
+    static constexpr bool kAligned = false;
+    static __host__ __device__ constexpr int piece_off(int k) { return k < 13 ? 16 * k : 194; }
+    static __device__ __forceinline__ float from_lds(const unsigned char* blk, const LaneCtx& c, const Addr& ad, int b) {
+        const u32x4 sc = *reinterpret_cast<const u32x4*>(blk + 192);
+        const unsigned ss = ((sc.x >> (8 * c.g)) & 0xffu) | (((sc.y >> (8 * c.g)) & 0xffu) << 8) | (((sc.z >> (8 * c.g)) & 0xffu) << 16) |
+                            (((sc.w >> (8 * c.g)) & 0xffu) << 24);
+        const unsigned dd = *reinterpret_cast<const unsigned*>(blk + 13 * 16 + 12) >> 16;
+        u32x4 ql[2], qh[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            ql[h] = *reinterpret_cast<const u32x4*>(blk + 64 * h + 16 * c.g);
+            qh[h] = *reinterpret_cast<const u32x4*>(blk + 128 + 32 * h + 16 * (c.g & 1));
+        }
+        return math(ss, dd, ql, qh, c, ad, b);
+    }
+    // In lane (n, g): ss = the scales 8 h + g and 8 h + 4 + g of both halves (a byte each), dd = the block's fp16
+    // scale, ql / qh = piece g of each half's low nibbles and the piece of high bit pairs that covers it.
+    static __device__ __forceinline__ float math(unsigned ss, unsigned dd, const u32x4 (&ql)[2], const u32x4 (&qh)[2], const LaneCtx& c,
+                                                 const Addr& ad, int b) {
+        const float d = half_of(dd & 0xffffu);
         const int s1 = 2 * (c.g >> 1);
         float out = 0.0f;
 #pragma unroll
@@ -356,7 +405,7 @@ struct MF<kQ6_K> {
             i32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const unsigned l = from_lane(c.src_lane4, r.ql[h][i]), u = from_lane(c.src_lane4, r.qh[h][i]) >> s1;
+                const unsigned l = ql[h][i], u = qh[h][i] >> s1;
                 lo[i] = (int)((l & 0x0f0f0f0fu) | ((u & 0x03030303u) << 4));
                 hi[i] = (int)(((l >> 4) & 0x0f0f0f0fu) | (((u >> 4) & 0x03030303u) << 4));
             }
@@ -500,32 +549,31 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
 constexpr int kRowsMaxCb = 2; // blocks of a row in an item, at most
 constexpr int kRowsRedBytes = 2 * kMaxWaves * 2 * 16 * 4 + 64; // two sets of partial row sums (tiles alternate: one barrier a tile), the waves' sums of squares
 
-template <bool FIVE, int CB>
+template <int T, int CB>
 struct RowsGeom {
-    static constexpr int P = MFK45<FIVE>::kBlockBytes / 16; // pieces of a block
+    static constexpr int P = MF<T>::kPieces;                 // pieces of a block
     static constexpr int kRowPieces = CB * P;                // pieces of a row in an item
     static constexpr int R = kRowPieces | 1;                 // LDS row stride, pieces
     static constexpr int NL = (16 * kRowPieces + 63) / 64;   // load instructions an item
     static constexpr int kWaveBytes = (16 * R + 1) * 16;     // (one more piece: where lanes past the item's end write)
     static __host__ __device__ size_t lds_bytes(int n_in, int waves) {
-        return (size_t)Lds<32>::red_off(n_in) + kRowsRedBytes + (size_t)waves * kWaveBytes;
+        return (size_t)Lds<MF<T>::kGroup>::red_off(n_in) + kRowsRedBytes + (size_t)waves * kWaveBytes;
     }
 };
 
-template <bool FIVE, bool DUAL, int kWaves, int CB>
+template <int T, bool DUAL, int kWaves, int CB>
 __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
-    using F = MFK45<FIVE>;
-    using L = Lds<32>;
-    using G = RowsGeom<FIVE, CB>;
+    using F = MF<T>;
+    using L = Lds<F::kGroup>;
+    using G = RowsGeom<T, CB>;
     constexpr int M = DUAL ? 2 : 1, P = G::P, R = G::R, NL = G::NL;
-    constexpr int kQ = F::kQs / 16; // piece of a block's first nibbles
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int nb_row = a.n_in >> 8;
     const int b0 = (int)blockIdx.z * nb_row / (int)gridDim.z, nb = ((int)blockIdx.z + 1) * nb_row / (int)gridDim.z - b0;
     const int n_in = nb << 8;
     float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
     const GemvSeg seg = a.seg[blockIdx.y];
-    const unsigned row_bytes = (unsigned)a.row_bytes;
+    const unsigned row_bytes = (unsigned)(a.n_seg_types ? seg.row_bytes : a.row_bytes);
     const int n_tiles = seg.n_out >> 4;
     if ((int)blockIdx.x >= n_tiles) return; // (whole workgroup: a shorter matrix of a shared launch)
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // (scalar: what follows from it stays in scalar registers)
@@ -548,8 +596,8 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     int loff[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        const int s = 64 * i + lane, row = s / G::kRowPieces, piece = s - row * G::kRowPieces;
-        goff[i] = row < 16 ? (unsigned)row * row_bytes + (unsigned)piece * 16u : 0xffffffffu; // (past the end: cut to the item's last piece below)
+        const int s = 64 * i + lane, row = s / G::kRowPieces, piece = s - row * G::kRowPieces, blk = piece / P;
+        goff[i] = row < 16 ? (unsigned)row * row_bytes + (unsigned)(blk * F::kBlockBytes + F::piece_off(piece - blk * P)) : 0xffffffffu; // (past the end: cut to the item's last piece below)
         loff[i] = row < 16 ? (row * R + piece) * 16 : 16 * R * 16;
     }
 
@@ -562,11 +610,13 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         const int cb = min(CB, nb - rq_c * CB);
         // pieces past the chunk's end in rows above the last are the row's next blocks or the next row's first (fetched,
         // never used); in the last row they are cut to the last piece
-        const unsigned limit = 15u * row_bytes + (unsigned)(cb * P - 1) * 16u;
+        const unsigned limit = 15u * row_bytes + (unsigned)((cb - 1) * F::kBlockBytes + F::piece_off(P - 1));
         const unsigned char* const base = wbase[m] + (size_t)rq_tile * 16 * row_bytes + (size_t)(b0 + rq_c * CB) * F::kBlockBytes;
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
-            r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + min(goff[i], limit))) /* whole runs, read once: streaming */;
+            // whole runs, read once: streaming loads
+            if constexpr (F::kAligned) r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + min(goff[i], limit)));
+            else r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a2*>(base + min(goff[i], limit)));
         }
         bias = *(seg.bias ? seg.bias + rq_tile * 16 + c.n : a.x); // (always a load: the same count on every path)
         if (m == M - 1) {
@@ -598,7 +648,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
                     x[i] *= g[i];
                 }
             }
-            digits8<32>(x, e, n_in, smem, pairs, lane);
+            digits8<F::kGroup>(x, e, n_in, smem, pairs, lane);
         };
         constexpr int kPasses = (CB * 256 + 511) / 512; // 512 elements a pass
         float x0[kPasses][8] = {}, g0[kPasses][8] = {};
@@ -684,16 +734,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(transit + loff[i]) = r[i];
         const int cb = min(CB, nb - cs_c * CB);
         float v = 0.0f;
-        for (int j = 0; j < cb; ++j) {
-            const unsigned char* const blk = transit + (c.n * R + j * P) * 16;
-            const u32x4 hdr = *reinterpret_cast<const u32x4*>(blk);
-            const u32x4 q1 = *reinterpret_cast<const u32x4*>(blk + (kQ + c.g) * 16);
-            const u32x4 q2 = *reinterpret_cast<const u32x4*>(blk + (kQ + 4 + c.g) * 16);
-            u32x4 fifth = {0u, 0u, 0u, 0u};
-            if constexpr (FIVE) fifth = *reinterpret_cast<const u32x4*>(blk + (1 + (c.g & 1)) * 16) >> (unsigned)(2 * (c.g >> 1));
-            const unsigned bb = ((hdr.y >> (8 * c.g)) & 0xffu) | (((hdr.z >> (8 * c.g)) & 0xffu) << 8) | (((hdr.w >> (8 * c.g)) & 0xffu) << 16);
-            v += F::math(hdr.x, bb, q1, q2, fifth, c, addr, cs_c * CB + j);
-        }
+        for (int j = 0; j < cb; ++j) v += F::from_lds(transit + (c.n * R + j * P) * 16, c, addr, cs_c * CB + j);
         rowacc[m] += v;
         if (m == M - 1) {
             cs_c += kWaves;
@@ -723,9 +764,9 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     if (k + 2 < total) consume(buf[0], bias_v[0], 0);
 }
 
-template <bool FIVE, bool DUAL, int kWaves, int CB>
+template <int T, bool DUAL, int kWaves, int CB>
 __global__ __launch_bounds__(kWaves * 64) void gemv_rows_kernel(const GemvArgs a) {
-    gemv_rows_body<FIVE, DUAL, kWaves, CB>(a);
+    gemv_rows_body<T, DUAL, kWaves, CB>(a);
 }
 
 // Matrices of different block types in one launch (the q, k, v projections of a file that keeps attn_v in
@@ -745,7 +786,7 @@ constexpr size_t kMfmaLdsMax = 96u * 1024u;
 template <int T>
 size_t lds_bytes(int n_in) { return Lds<MF<T>::kGroup>::bytes(n_in); }
 
-// The long-run kernel where it applies: Q4_K / Q5_K, whole 16-row tiles, LDS within the limit.
+// The long-run kernel where it applies: Q4_K / Q5_K / Q6_K, whole 16-row tiles, LDS within the limit.
 bool rows_enabled() {
     static const bool on = getenv("ORIN_GEMV_NO_ROWS") == nullptr;
     return on;
@@ -757,31 +798,31 @@ int rows_wgs_per_cu(int given) {
     return env ? given : 3;
 }
 
-template <bool FIVE, bool DUAL, int kWaves, int CB>
+template <int T, bool DUAL, int kWaves, int CB>
 bool launch_rows_as(const GemvArgs& a, dim3 grid, int n_in_wg, hipStream_t stream) {
-    const size_t lds = RowsGeom<FIVE, CB>::lds_bytes(n_in_wg, kWaves);
+    const size_t lds = RowsGeom<T, CB>::lds_bytes(n_in_wg, kWaves);
     if (lds > kMfmaLdsMax) return false;
-    hipLaunchKernelGGL((gemv_rows_kernel<FIVE, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, a);
+    hipLaunchKernelGGL((gemv_rows_kernel<T, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, a);
     return true;
 }
 
-template <bool FIVE>
+template <int T>
 bool launch_rows(const GemvArgs& a, dim3 grid, bool wide, int nb_wg, hipStream_t stream) {
     if (!rows_enabled()) return false;
     for (int i = 0; i < a.n_seg; ++i)
         if (a.seg[i].n_out % 16 != 0) return false;
     const int n_in_wg = nb_wg * 256;
     if (wide) { // (eight waves: never two matrices)
-        return (nb_wg + 7) / 8 <= 1 ? launch_rows_as<FIVE, false, 8, 1>(a, grid, n_in_wg, stream)
-                                    : launch_rows_as<FIVE, false, 8, 2>(a, grid, n_in_wg, stream);
+        return (nb_wg + 7) / 8 <= 1 ? launch_rows_as<T, false, 8, 1>(a, grid, n_in_wg, stream)
+                                    : launch_rows_as<T, false, 8, 2>(a, grid, n_in_wg, stream);
     }
     // runs of 288 (352) bytes read within a few percent of longer ones, and the wave's last item, which nothing
     // overlaps, is half as long as with four blocks
     const int cb = min(kRowsMaxCb, (nb_wg + 3) / 4);
     if (a.w_up) {
-        return cb == 1 ? launch_rows_as<FIVE, true, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<FIVE, true, 4, 2>(a, grid, n_in_wg, stream);
+        return cb == 1 ? launch_rows_as<T, true, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<T, true, 4, 2>(a, grid, n_in_wg, stream);
     }
-    return cb == 1 ? launch_rows_as<FIVE, false, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<FIVE, false, 4, 2>(a, grid, n_in_wg, stream);
+    return cb == 1 ? launch_rows_as<T, false, 4, 1>(a, grid, n_in_wg, stream) : launch_rows_as<T, false, 4, 2>(a, grid, n_in_wg, stream);
 }
 
 template <int T>
@@ -801,12 +842,17 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     // Eight waves a workgroup where a row has the blocks to share out and a workgroup has one tile only (a
     // second tile would have amortised the staging instead).
     const bool wide = ks == 1 && nb_row >= 16 && !a.w_up && (int)grid.x == (max_out + 15) / 16;
-    if constexpr (T == kQ4_K || T == kQ5_K) {
+    if constexpr (T == kQ4_K || T == kQ5_K || T == kQ6_K) {
         const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu);
         dim3 gr = g3;
         gr.x = min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16);
-        const bool wide_r = ks == 1 && nb_row >= 16 && !a.w_up && (int)gr.x == (max_out + 15) / 16;
-        if (launch_rows<T == kQ5_K>(a, gr, wide_r, (nb_row + ks - 1) / ks, stream)) return hipGetLastError();
+        // (its LDS buffers let three workgroups of four waves share a CU: no more shares of a row than are resident at once)
+        int ks_r = ks;
+        if (a.k_split_override <= 0)
+            while (ks_r > 1 && (int)(gr.x * gr.y) * ks_r > cu_count * 3) ks_r /= 2;
+        gr.z = ks_r;
+        const bool wide_r = ks_r == 1 && nb_row >= 16 && !a.w_up && (int)gr.x == (max_out + 15) / 16;
+        if (launch_rows<T>(a, gr, wide_r, (nb_row + ks_r - 1) / ks_r, stream)) return hipGetLastError();
     }
     const size_t lds = lds_bytes<T>((nb_row + ks - 1) / ks * 256);
     if (a.w_up) {
@@ -828,21 +874,21 @@ hipError_t allow() {
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }
 
-template <bool FIVE, bool DUAL, int kWaves, int CB>
+template <int T, bool DUAL, int kWaves, int CB>
 hipError_t allow_rows() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_kernel<FIVE, DUAL, kWaves, CB>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_kernel<T, DUAL, kWaves, CB>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }
 
-template <bool FIVE>
+template <int T>
 hipError_t allow_rows_all() {
     hipError_t e;
-    if ((e = allow_rows<FIVE, false, 8, 1>()) != hipSuccess) return e;
-    if ((e = allow_rows<FIVE, false, 8, 2>()) != hipSuccess) return e;
-    if ((e = allow_rows<FIVE, false, 4, 1>()) != hipSuccess) return e;
-    if ((e = allow_rows<FIVE, false, 4, 2>()) != hipSuccess) return e;
-    if ((e = allow_rows<FIVE, true, 4, 1>()) != hipSuccess) return e;
-    return allow_rows<FIVE, true, 4, 2>();
+    if ((e = allow_rows<T, false, 8, 1>()) != hipSuccess) return e;
+    if ((e = allow_rows<T, false, 8, 2>()) != hipSuccess) return e;
+    if ((e = allow_rows<T, false, 4, 1>()) != hipSuccess) return e;
+    if ((e = allow_rows<T, false, 4, 2>()) != hipSuccess) return e;
+    if ((e = allow_rows<T, true, 4, 1>()) != hipSuccess) return e;
+    return allow_rows<T, true, 4, 2>();
 }
 
 } // namespace
@@ -889,8 +935,9 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow<kQ5_K, true>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, false>()) != hipSuccess) return e;
     if ((e = allow<kQ8_0, true>()) != hipSuccess) return e;
-    if ((e = allow_rows_all<false>()) != hipSuccess) return e;
-    if ((e = allow_rows_all<true>()) != hipSuccess) return e;
+    if ((e = allow_rows_all<kQ4_K>()) != hipSuccess) return e;
+    if ((e = allow_rows_all<kQ5_K>()) != hipSuccess) return e;
+    if ((e = allow_rows_all<kQ6_K>()) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<8>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),

@@ -213,13 +213,13 @@ def test_projections_of_different_types(ly, unit, wtypes, n_in):
         assert vec_err(got[:n], w_.astype(np.float64)) < TOL_OP and (got[n:] == 12345.0).all()
 
 
-# Q4_K / Q5_K matrices made of whole 16-row tiles go to the kernel that reads rows in long runs: 1 ... 74 blocks
+# Q4_K / Q5_K / Q6_K matrices made of whole 16-row tiles go to the kernel that reads rows in long runs: 1 ... 74 blocks
 # per row (one or two blocks per item, chunks shared among four or eight waves, ragged last chunks), few and many
 # tiles (one per workgroup, several per workgroup), every epilogue.
 LONG_RUN_SHAPES = [(256, 48), (512, 16), (1536, 12800), (1792, 64), (3584, 512), (4096, 4096), (8960, 96), (14336, 256), (18944, 32)]
 
 
-@pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q5_K])
+@pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q5_K, lm.Q6_K])
 @pytest.mark.parametrize("n_in,n_out", LONG_RUN_SHAPES)
 def test_whole_tiles_in_long_runs(ly, wtype, n_in, n_out):
     import torch
@@ -230,7 +230,8 @@ def test_whole_tiles_in_long_runs(ly, wtype, n_in, n_out):
     x = rs.sym(n_in, 1.0)
     nw = (1.0 + rs.sym(n_in, 0.3)).astype(np.float32)
     bias, y0 = rs.sym(n_out, 0.5), rs.sym(n_out, 1.0)
-    w, dx = dev_bytes(t[1]), _dev(x)
+    odd = 2 if wtype == lm.Q6_K else 0   # (the 2-byte-aligned type at an odd spot)
+    w, dx = dev_bytes(t[1], offset=odd), _dev(x)
     plain = ref.gemv(wtype, t[1], x, n_in, n_out).astype(np.float64)
     normed = ref.gemv(wtype, t[1], ref.rms_norm(x, nw, 1e-5), n_in, n_out).astype(np.float64)
     errs = {}
@@ -246,7 +247,7 @@ def test_whole_tiles_in_long_runs(ly, wtype, n_in, n_out):
     if n_out <= 4096:
         up = lm.make_tensor(rs, wtype, n_in, n_out)
         yg = out_buf(n_out)
-        ly.gemv_norm_gate_up_swiglu(wtype, w, dev_bytes(up[1]), dx, _dev(nw), 1e-5, yg, n_in, n_out)
+        ly.gemv_norm_gate_up_swiglu(wtype, w, dev_bytes(up[1], offset=odd), dx, _dev(nw), 1e-5, yg, n_in, n_out)
         u = ref.gemv(wtype, up[1], ref.rms_norm(x, nw, 1e-5), n_in, n_out)
         errs["gate/up"] = (yg, ref.swiglu(normed.astype(np.float32), u).astype(np.float64))
     torch.cuda.synchronize()
