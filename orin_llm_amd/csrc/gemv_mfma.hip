@@ -781,6 +781,16 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_mixed_kernel(const Gemv
     }
 }
 
+// The same for the kernel that reads rows in long runs (no Q8_0 there).
+template <int kWaves, int CB>
+__global__ __launch_bounds__(kWaves * 64) void gemv_rows_mixed_kernel(const GemvArgs a) {
+    switch (a.seg[blockIdx.y].type) {
+    case kQ4_K: gemv_rows_body<kQ4_K, false, kWaves, CB>(a); break;
+    case kQ5_K: gemv_rows_body<kQ5_K, false, kWaves, CB>(a); break;
+    default: gemv_rows_body<kQ6_K, false, kWaves, CB>(a); break;
+    }
+}
+
 constexpr size_t kMfmaLdsMax = 96u * 1024u;
 
 template <int T>
@@ -848,8 +858,10 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
         gr.x = min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16);
         // (its LDS buffers let three workgroups of four waves share a CU: no more shares of a row than are resident at once)
         int ks_r = ks;
-        if (a.k_split_override <= 0)
+        if (a.k_split_override <= 0) {
+            if (ks == 1 && nb_row >= 6 && a.accumulate && !a.w_up && !a.norm_w && (int)(grid.x * grid.y) <= cu_count) ks_r = 2; // (shorter rows too: a share is cheap here)
             while (ks_r > 1 && (int)(gr.x * gr.y) * ks_r > cu_count * 3) ks_r /= 2;
+        }
         gr.z = ks_r;
         const bool wide_r = ks_r == 1 && nb_row >= 16 && !a.w_up && (int)gr.x == (max_out + 15) / 16;
         if (launch_rows<T>(a, gr, wide_r, (nb_row + ks_r - 1) / ks_r, stream)) return hipGetLastError();
@@ -900,6 +912,29 @@ hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) 
     const int cap = a.mfma_wgs_per_cu > 0 ? cu_count * a.mfma_wgs_per_cu : (max_out + 15) / 16;
     const dim3 grid(min((max_out + 15) / 16, cap), a.n_seg);
     a.n_seg_types = 1;
+    bool rows = rows_enabled();
+    for (int i = 0; i < a.n_seg; ++i) rows = rows && a.seg[i].n_out % 16 == 0 && a.seg[i].type != kQ8_0;
+    if (rows) {
+        const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu), nb = a.n_in / 256;
+        const dim3 gr(min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16), a.n_seg);
+        const bool wide_r = nb >= 16 && (int)gr.x == (max_out + 15) / 16;
+        // (the largest of the types' layouts: Q6_K's digits in groups of 16, Q5_K's 11 pieces a block are within Q6_K's 14)
+        if (wide_r) {
+            const size_t lds = RowsGeom<kQ6_K, 2>::lds_bytes(a.n_in, 8);
+            if (lds <= kMfmaLdsMax) {
+                if ((nb + 7) / 8 <= 1) hipLaunchKernelGGL((gemv_rows_mixed_kernel<8, 1>), gr, dim3(512), lds, stream, a);
+                else hipLaunchKernelGGL((gemv_rows_mixed_kernel<8, 2>), gr, dim3(512), lds, stream, a);
+                return hipGetLastError();
+            }
+        } else {
+            const size_t lds = RowsGeom<kQ6_K, 2>::lds_bytes(a.n_in, 4);
+            if (lds <= kMfmaLdsMax) {
+                if ((nb + 3) / 4 <= 1) hipLaunchKernelGGL((gemv_rows_mixed_kernel<4, 1>), gr, dim3(256), lds, stream, a);
+                else hipLaunchKernelGGL((gemv_rows_mixed_kernel<4, 2>), gr, dim3(256), lds, stream, a);
+                return hipGetLastError();
+            }
+        }
+    }
     const size_t lds = max(lds_bytes<kQ4_K>(a.n_in), lds_bytes<kQ6_K>(a.n_in));
     const bool wide = a.n_in / 256 >= 16 && (int)grid.x == (max_out + 15) / 16; // (as in launch() above)
     if (wide) hipLaunchKernelGGL((gemv_mfma_mixed_kernel<8>), grid, dim3(512), lds, stream, a);
@@ -938,6 +973,10 @@ hipError_t gemv_mfma_allow_lds() {
     if ((e = allow_rows_all<kQ4_K>()) != hipSuccess) return e;
     if ((e = allow_rows_all<kQ5_K>()) != hipSuccess) return e;
     if ((e = allow_rows_all<kQ6_K>()) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_mixed_kernel<8, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_mixed_kernel<8, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_mixed_kernel<4, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
+    if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_mixed_kernel<4, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     if ((e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<8>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),

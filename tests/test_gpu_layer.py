@@ -191,13 +191,14 @@ def test_three_projections_in_one_launch(ly, unit, wtype):
 
 
 @pytest.mark.parametrize("wtypes", [(lm.Q4_K, lm.Q4_K, lm.Q6_K), (lm.Q6_K, lm.Q4_K, lm.Q6_K), (lm.Q4_K, lm.Q5_K, lm.Q6_K), (lm.Q8_0, lm.F16)])
-@pytest.mark.parametrize("n_in", [1536, 4096])
-def test_projections_of_different_types(ly, unit, wtypes, n_in):
+@pytest.mark.parametrize("n_in", [256, 1536, 4096])
+@pytest.mark.parametrize("heights", [(520, 130, 96), (512, 128, 96), (4096, 1024, 1024)])
+def test_projections_of_different_types(ly, unit, wtypes, n_in, heights):
     """One launch where every type is a block type and the matrix cores are in use, one per matrix otherwise; same
-    results either way."""
+    results either way.  (Heights that are whole 16-row tiles go to the kernel that reads rows in long runs.)"""
     import torch
 
-    n_outs = [520, 130, 96][:len(wtypes)]
+    n_outs = list(heights)[:len(wtypes)]
     rs = lm.Stream(4500 + sum(wtypes) + n_in)
     ts = [lm.make_tensor(rs, t, n_in, n) for t, n in zip(wtypes, n_outs)]
     bs = [rs.sym(n, 0.5) for n in n_outs]
