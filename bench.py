@@ -1184,7 +1184,7 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
                            cache_MB_per_layer=round(kv_bytes / 1e6, 2), launch="graph" if forms["graph"]["device_ms_per_step"] <= forms["eager"]["device_ms_per_step"] else "eager"),
                roofline=dict(bound="hbm", achieved=launch_bytes[main_key] / (launch_us[main_key]["us"] * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9,
                              unit="GB/s", frac=launch_bytes[main_key] / (launch_us[main_key]["us"] * 1e-6) / PEAK_BYTES, traffic=None,
-                             kernel="gemv_kernel<Q4_K, dual> (norm + gate/up + SwiGLU)", launch_us=launch_us[main_key]["us"],
+                             kernel="gemv_rows_kernel<Q4_K, two matrices> (norm + gate/up + SwiGLU)", launch_us=launch_us[main_key]["us"],
                              bytes_per_launch=launch_bytes[main_key], layer_us=us_layer, layer_frac=bytes_layer / (us_layer * 1e-6) / PEAK_BYTES,
                              layer_us_reference_call_sequence=us_layer_calls, launches=launch_us),
                parity=dict(err_row=err, err_floor1pct=err, cache_row_err=cache_err,

@@ -29,6 +29,9 @@ FLAGS = [
     # behind a trip to memory (the attention kernels put what their first loads need there)
     "-mllvm", "-amdgpu-kernarg-preload-count=14",
 ]
+# Per source: the matrix-vector kernels' matrix instructions leave their sums in vector registers (the default puts
+# them in accumulation registers, from which the vector ALU has to fetch each with a move before it can use it).
+EXTRA_FLAGS = {"gemv_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 # The prefill kernel's hand-placed instruction stream (matrix-result and vector-write wait states counted by
@@ -59,7 +62,7 @@ def build(verbose=False):
     check_toolchain()
     os.makedirs(OBJ_DIR, exist_ok=True)
     objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in SOURCES]
-    cmds = [[HIPCC] + FLAGS + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
+    cmds = [[HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(s), []) + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
     stamped = {s: os.path.join(OBJ_DIR, os.path.basename(s) + ".stamps.o") for s in SOURCES if os.path.basename(s) in STAMPED}
     cmds += [[HIPCC] + FLAGS + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
     dec = next(s for s in SOURCES if os.path.basename(s) == "fa_decode.hip")
