@@ -75,6 +75,10 @@ WORKLOADS = {
     # partials), its partials merged by a second kernel, as the library does, or inside the launch by a two-level
     # last-arriver reduction over write-through stores and relaxed atomics -- what fusing the combine would cost
     "decode-handoff-mock": (None, "handoff", 0, 32 << 20),
+    # not part of the path: read-only stand-ins for the loads of a matrix-vector kernel over a Q4_K gate/up pair of
+    # Llama-3-8B's shape (2 x 14336 rows x 16 blocks, 66 MB), by load pattern -- 64 bytes of each of 16 rows per
+    # instruction, or lane-linear runs of one, two or four whole blocks of a row
+    "weights-read-patterns": (None, "patterns", 0, (14336, 16)),
     # The whole decode layer around the path (norms, quantised projections, rotary embedding, cache store,
     # attention, feed-forward block): one token through every layer of the model, replayed as one graph.
     # Weights are random blocks in the mix of a Q4_K_M file (Q4_K; attn_v and ffn_down Q6_K).
@@ -783,6 +787,56 @@ def run_read(torch, kernels, name, steps, warmup, with_cpu):
                 parity=None)
 
 
+def run_patterns(torch, kernels, name, steps, warmup, with_cpu):
+    """What the load pattern of a matrix-vector kernel costs by itself: a pair of Q4_K-shaped matrices read by
+    kernels that compute nothing, launched back to back in a graph over buffers that rotate through more memory than
+    the last-level cache holds.  One step = 16 launches; value and roofline are the best pattern's."""
+    n_rows, n_blocks = WORKLOADS[name][3]
+    mat = n_rows * n_blocks * 144
+    nbytes = 2 * mat
+    launches = 16
+    n_buf = max(launches, int(np.ceil(1.2e9 / nbytes)))
+    pool = torch.empty(n_buf * nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    names = {0: "64 B of each of 16 rows per instruction", 1: "runs of 144 B", 2: "runs of 288 B", 4: "runs of 576 B"}
+    out, wall_best, best_us = {}, None, None
+    for pattern, label in names.items():
+        for wgs_per_cu in (2, 3):
+            g = torch.cuda.CUDAGraph()
+            try:
+                with torch.cuda.graph(g):
+                    kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+                    for k in range(launches):
+                        kernels.bench_read_pattern(pool[(k % n_buf) * nbytes:], mat, n_rows, n_blocks, pattern, wgs_per_cu * kernels.cu_count())
+            finally:
+                kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            for _ in range(max(1, warmup)):
+                g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            e0.record()
+            for _ in range(steps):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+            us = e0.elapsed_time(e1) * 1e3 / (steps * launches)
+            del g
+            out[f"{label}, {wgs_per_cu} workgroups per CU"] = dict(us=round(us, 2), GBps=round(nbytes / (us * 1e-6) / 1e9, 1))
+            if best_us is None or us < best_us:
+                best_us, wall_best, best = us, wall, f"{label}, {wgs_per_cu} workgroups per CU"
+    del pool
+    torch.cuda.empty_cache()
+    return dict(value=nbytes * launches * steps / wall_best / 1e9, unit="GB/s", ms_per_step=wall_best / steps * 1e3,
+                config=dict(workload=name, shape=f"2 x {n_rows} rows x {n_blocks} blocks of 144 B", bytes_per_launch=nbytes,
+                            launches_per_step=launches, buffers_rotated=n_buf),
+                roofline=dict(bound="hbm", achieved=nbytes / (best_us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=nbytes / (best_us * 1e-6) / PEAK_BYTES, traffic=float(nbytes),
+                              kernel=f"read_pattern_kernel ({best}; reads only, not part of the path)", launch_us=best_us,
+                              launch_us_by_pattern=out, bytes_per_launch=nbytes),
+                parity=None)
+
+
 # Stage marks of the kernels (slot, what has happened by then), in the order a wave passes them.
 PREFILL_STAGES = [(0, "entry"), (9, "queries and first K tile requested"), (10, "first V tile and second K tile requested"),
                   (1, "queries in registers"), (2, "first two score tiles"), (3, "first weights"), (4, "main loop done"),
@@ -1198,7 +1252,7 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
 
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"decode_layer": run_decode_layer, "prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
+    fn = {"decode_layer": run_decode_layer, "prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "patterns": run_patterns, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 

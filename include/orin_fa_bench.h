@@ -28,6 +28,14 @@ int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t*
  * decode step's cache read costs when nothing else is done with the bytes.  Asynchronous. */
 int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread);
 
+/* One launch, on the library's stream, of a kernel that only reads a pair of Q4_K-shaped matrices (n_rows rows of
+ * n_blocks 144-byte blocks each; the second matrix mat_bytes behind the first; w 16-byte aligned, n_rows a multiple
+ * of 16, n_blocks of 8) the way a matrix-vector kernel would: workgroups of four waves over 16-row tiles.
+ * pattern 0: per load instruction 64 bytes of each of 16 rows (header, and a piece of each half of a block's nibbles);
+ * pattern 1, 2, 4: runs of that many whole blocks of a row, lane after lane, with streaming loads.  What the load
+ * pattern alone costs, nothing computed.  Asynchronous. */
+int orin_fa_bench_read_pattern(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups);
+
 /* A stand-in for one split-KV decode step, to price the two ways of merging its partial results:
  * 256 workgroups stream orin_fa_bench_handoff_stream_bytes() (32 MiB) at src and leave 784-float
  * partial results that are then added up into out[784] -- fused = 0: by a second kernel (two

@@ -126,6 +126,66 @@ __global__ __launch_bounds__(256) void handoff_combine_kernel(const float* part1
     if (lane == 0) *reinterpret_cast<f4*>(out + e * 4) = sum;
 }
 
+// ---- what the load pattern of a matrix-vector kernel costs ----
+// Read-only stand-ins over a pair of Q4_K-shaped matrices (rows of n_blocks 144-byte blocks, the second matrix
+// `mat_bytes` behind the first): a workgroup of four waves walks 16-row tiles, wave w takes every fourth chunk of a
+// tile's blocks, and everything loaded is folded into a word that is never stored.
+//   RUN = 0: per instruction 64 bytes of each of 16 rows -- lane = 4 row + piece: a block's 16-byte header, and a
+//            16-byte piece of each half of its nibbles (three instructions a block and matrix).
+//   RUN = 1, 2, 4: a chunk of RUN blocks of each of the 16 rows as (row, 16-byte piece) slots in row-major order,
+//            lane after lane: runs of 144 RUN bytes, every line asked for by one instruction; streaming loads.
+template <int RUN>
+__global__ __launch_bounds__(256) void read_pattern_kernel(const unsigned char* w, size_t mat_bytes, int n_rows, int n_blocks, unsigned* sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row_bytes = (size_t)n_blocks * 144;
+    const int n_tiles = n_rows / 16;
+    unsigned acc = 0;
+    if constexpr (RUN == 0) {
+        const int ln = lane >> 2, lg = lane & 3;
+        for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+            for (int b = wave; b < n_blocks; b += 8) { // two blocks in flight
+                u32x4 r[12];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int bb = min(b + 4 * u, n_blocks - 1);
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) {
+                        const unsigned char* blk = w + m * mat_bytes + (size_t)(tile * 16 + ln) * row_bytes + (size_t)bb * 144;
+                        r[6 * u + 3 * m] = *reinterpret_cast<const u32x4*>(blk);
+                        r[6 * u + 3 * m + 1] = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * lg);
+                        r[6 * u + 3 * m + 2] = *reinterpret_cast<const u32x4*>(blk + 80 + 16 * lg);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 12; ++i) acc ^= r[i].x ^ r[i].y ^ r[i].z ^ r[i].w;
+            }
+        }
+    } else {
+        constexpr int RP = RUN * 9, NL = (16 * RP + 63) / 64;
+        unsigned off[NL];
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int s = min(64 * i + lane, 16 * RP - 1), row = s / RP, piece = s - row * RP;
+            off[i] = (unsigned)(row * row_bytes) + (unsigned)piece * 16u;
+        }
+        const int n_chunks = n_blocks / RUN;
+        for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+            for (int c = wave; c < n_chunks; c += 4) {
+#pragma unroll
+                for (int m = 0; m < 2; ++m) { // (one matrix's chunk at a time, as the product kernel's items are)
+                    const unsigned char* base = w + m * mat_bytes + (size_t)tile * 16 * row_bytes + (size_t)c * RUN * 144;
+                    u32x4 r[NL];
+#pragma unroll
+                    for (int i = 0; i < NL; ++i) r[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + off[i]));
+#pragma unroll
+                    for (int i = 0; i < NL; ++i) acc ^= r[i].x ^ r[i].y ^ r[i].z ^ r[i].w;
+                }
+            }
+        }
+    }
+    if (acc == 0x9E3779B9u) *sink = acc;
+}
+
 } // namespace
 
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream) {
@@ -172,6 +232,22 @@ hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out,
 
 hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream) {
     hipLaunchKernelGGL(tiny_kernel, dim3(1), dim3(64), 0, stream, src, sink);
+    return hipGetLastError();
+}
+
+
+// pattern: 0 (64 bytes of each of 16 rows per instruction), or the run length in blocks (1, 2, 4)
+hipError_t read_pattern_launch(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups, unsigned* sink,
+                               hipStream_t stream) {
+    if (n_rows % 16 != 0 || n_blocks % 8 != 0 || workgroups < 1) return hipErrorInvalidValue;
+    const unsigned char* p = static_cast<const unsigned char*>(w);
+    switch (pattern) {
+    case 0: hipLaunchKernelGGL(read_pattern_kernel<0>, dim3(workgroups), dim3(256), 0, stream, p, mat_bytes, n_rows, n_blocks, sink); break;
+    case 1: hipLaunchKernelGGL(read_pattern_kernel<1>, dim3(workgroups), dim3(256), 0, stream, p, mat_bytes, n_rows, n_blocks, sink); break;
+    case 2: hipLaunchKernelGGL(read_pattern_kernel<2>, dim3(workgroups), dim3(256), 0, stream, p, mat_bytes, n_rows, n_blocks, sink); break;
+    case 4: hipLaunchKernelGGL(read_pattern_kernel<4>, dim3(workgroups), dim3(256), 0, stream, p, mat_bytes, n_rows, n_blocks, sink); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

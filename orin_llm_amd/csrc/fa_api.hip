@@ -389,6 +389,13 @@ int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread) 
     return hip_code(hbm_read_launch(src, bytes, loads_per_thread, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
 }
 
+int orin_fa_bench_read_pattern(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups) {
+    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
+    if (!w || (reinterpret_cast<uintptr_t>(w) & 15u) || mat_bytes < (size_t)n_rows * n_blocks * 144 || (mat_bytes & 15u)) return ORIN_FA_E_INVALID;
+    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
+    return hip_code(read_pattern_launch(w, mat_bytes, n_rows, n_blocks, pattern, workgroups, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
+}
+
 int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out) {
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
     if (!src || !scratch || !out) return ORIN_FA_E_INVALID;

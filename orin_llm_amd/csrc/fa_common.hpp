@@ -87,6 +87,8 @@ hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* 
 
 // Measurement aids (bench_aids.hip).
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream);
+hipError_t read_pattern_launch(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups, unsigned* sink,
+                               hipStream_t stream);
 hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream);
 
 // ---- timeline build (-DORIN_FA_STAMPS, liborin_fa_stamps.so; a measurement aid) ----

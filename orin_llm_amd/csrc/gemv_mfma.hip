@@ -530,22 +530,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
     gemv_mfma_body<T, DUAL, kWaves>(a);
 }
 
-// Q4_K and Q5_K rows read in long runs.  The kernel above fetches, per load instruction, 64 bytes of each of 16
-// rows; this machine's memory path moves that pattern at 4.4 TB/s where lane-linear runs of 288 bytes move at
-// 5.4 TB/s and of 576 bytes at 5.5 TB/s (a read-only stand-in with these patterns over the 66 MB of a Llama-3-8B
-// gate/up pair: 15.0, 12.3 and 11.9 us a launch; a plain read 12.3, with streaming loads 11.0).  Here a wave's
-// item is CB consecutive blocks of each of a tile's 16 rows, of one matrix, fetched as (row, 16-byte piece) slots
-// in row-major order, lane after lane, with streaming loads: runs of CB * 144 (176) bytes, every line requested by
-// one instruction.  The pieces pass through a wave-private LDS buffer (rows padded to an odd number of pieces, so
-// that the 16 rows a matrix-instruction operand is read from lie in 16 different bank groups) and come back in
-// the matrix instruction's lane order: no lane permutations.  Two items per wave are on their way or in use;
-// chunks w, w + kWaves, ... of a tile's blocks are wave w's, and so are those chunks' digits of the activation,
-// which the wave makes for itself: no wave waits for another before the first tile's end, where the norm's sum
-// of squares is put together as well.  Barriers wait for LDS only, row sums leave through stores and atomic adds
-// without a return value, a tile's bias values travel with its items: nothing in the loop waits for anything but
-// the oldest item.  Requires whole 16-row tiles.  (Deeper request queues, three and four items a wave, were
-// slower in both kernels: what bounds them after the loads is the vector ALU, about 95 instructions per block
-// and wave for the nibbles, the six-bit pairs and the digit sums.)
+// Q4_K, Q5_K and Q6_K rows read in long runs.  The kernel above fetches, per load instruction, 64 bytes of each of
+// 16 rows; this machine's memory path moves that pattern at 4.6-4.7 TB/s where lane-linear runs of two whole blocks
+// of a row (288 bytes) move at 5.5-5.8 TB/s, as fast as a plain streaming read (the read-only stand-ins of
+// bench_aids.hip over the 66 MB of a Llama-3-8B gate/up pair, `bench.py --workload weights-read-patterns`: 14.1-14.4
+// us a launch against 11.5-12.0; runs of one block 13.5, of four blocks 17.9).  Here a wave's item is CB <= 2
+// consecutive blocks of each of a tile's 16 rows, of one matrix, fetched as (row, 16-byte piece) slots in row-major
+// order, lane after lane, with streaming loads: every line is asked for by one instruction.  The pieces pass
+// through a wave-private LDS buffer (rows padded to an odd number of pieces, so that the 16 rows a
+// matrix-instruction operand is read from lie in 16 different bank groups) and come back in the matrix
+// instruction's lane order: no lane permutations.  Two items per wave are on their way or in use; chunks w, w +
+// kWaves, ... of a tile's blocks are wave w's, and so are those chunks' digits of the activation, which the wave
+// makes for itself: no wave waits for another before the first tile's end, where the norm's sum of squares is put
+// together as well.  Barriers wait for LDS only, row sums leave through stores and atomic adds without a return
+// value, a tile's bias values travel with its items: nothing in the loop waits for anything but the oldest item.
+// Requires whole 16-row tiles.  (Deeper request queues, three and four items a wave, were slower in both kernels,
+// and so were four-block items: what bounds the kernels after the loads is the vector ALU, about 85 instructions
+// per block and wave for the nibbles, the six-bit pairs and the digit sums.)
 constexpr int kRowsMaxCb = 2; // blocks of a row in an item, at most
 constexpr int kRowsRedBytes = 2 * kMaxWaves * 2 * 16 * 4 + 64; // two sets of partial row sums (tiles alternate: one barrier a tile), the waves' sums of squares
 

@@ -74,6 +74,8 @@ def lib():
         L.orin_fa_decode_ind_timed.restype = _int
         L.orin_fa_bench_hbm_read.argtypes = [_vp, ctypes.c_size_t, _int]
         L.orin_fa_bench_hbm_read.restype = _int
+        L.orin_fa_bench_read_pattern.argtypes = [_vp, ctypes.c_size_t, _int, _int, _int, _int]
+        L.orin_fa_bench_read_pattern.restype = _int
         L.orin_fa_bench_handoff.argtypes = [_vp, _int, _vp, _vp]
         L.orin_fa_bench_handoff.restype = _int
         L.orin_fa_bench_handoff_scratch_bytes.argtypes = []
@@ -256,6 +258,13 @@ def bench_hbm_read(src, nbytes, loads_per_thread=16):
     rc = lib().orin_fa_bench_hbm_read(_ptr(src), int(nbytes), int(loads_per_thread))
     if rc != 0:
         raise OrinFaError("bench_hbm_read", rc)
+
+
+def bench_read_pattern(w, mat_bytes, n_rows, n_blocks, pattern, workgroups):
+    """Measurement aid: one launch of a read-only stand-in for a matrix-vector kernel's loads over a pair of Q4_K-shaped matrices."""
+    rc = lib().orin_fa_bench_read_pattern(_ptr(w), int(mat_bytes), int(n_rows), int(n_blocks), int(pattern), int(workgroups))
+    if rc != 0:
+        raise OrinFaError("bench_read_pattern", rc)
 
 
 def bench_tiny_launch():

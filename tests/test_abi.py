@@ -42,7 +42,7 @@ def test_header_declares_the_expected_entry_points():
 
 def test_measurement_aids_sit_in_their_own_header():
     assert _declared_c_functions(BENCH_HDR) == sorted([
-        "orin_fa_decode_ind_timed", "orin_fa_bench_hbm_read", "orin_fa_bench_tiny_launch", "orin_fa_bench_handoff",
+        "orin_fa_decode_ind_timed", "orin_fa_bench_hbm_read", "orin_fa_bench_read_pattern", "orin_fa_bench_tiny_launch", "orin_fa_bench_handoff",
         "orin_fa_bench_handoff_scratch_bytes", "orin_fa_bench_handoff_stream_bytes", "orin_fa_bench_stamps"])
 
 
