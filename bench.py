@@ -119,7 +119,7 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
         "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
-        "qwen1.5b-decode-32k-cutoffs", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
+        "qwen1.5b-decode-32k-cutoffs", "weights-read-patterns", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too

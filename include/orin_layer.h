@@ -50,7 +50,10 @@ int orin_quantize_activation(const float* x, int n_in);
 
 /* Replace llm::cuda::gemv_q8 / gemv_q8_bias / gemv_q8_add (reference: src/kernels.h:21-27,
  * src/kernels.cu:1786-1806, 1825-1836): y = W xs, y = W xs + bias, y += W xs, with xs the activation of the
- * last orin_quantize_activation call (whose n_in must equal this n_in). */
+ * last orin_quantize_activation call (whose n_in must equal this n_in).  The accumulating form may add a row's sum
+ * to y in several shares with atomic adds (long rows of a matrix with few rows): y must be written by nothing else
+ * while the launch runs, and the order in which a row's shares are added is not fixed (the last bits of y may
+ * differ from run to run; with one share the result is the plain sum). */
 int orin_gemv_q8(int type, const void* W, float* y, int n_in, int n_out);
 int orin_gemv_q8_bias(int type, const void* W, const float* bias, float* y, int n_in, int n_out);
 int orin_gemv_q8_add(int type, const void* W, float* y, int n_in, int n_out);
