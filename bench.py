@@ -85,6 +85,10 @@ WORKLOADS = {
     "qwen1.5b-decode-layer-32k": ("qwen1.5b", "decode_layer", 32768, 32768),
     "llama8b-decode-layer-8k": ("llama8b", "decode_layer", 8192, 8192),
     "qwen7b-decode-layer-32k": ("qwen7b", "decode_layer", 32768, 32767),
+    # The end of a decode step (reference: src/model_gpu.cu:303-306): the last norm and the output matrix over the
+    # residual stream, one token.  Output matrix Q6_K, as a Q4_K_M file keeps it; (vocabulary size)
+    "llama8b-logits": ("llama8b", "logits", 0, 128256),
+    "qwen1.5b-logits": ("qwen1.5b", "logits", 0, 151936),
     # not timed: where a kernel's microseconds go, from the timeline build of the library (the attention kernels'
     # stage marks store the wall clock there; medians over the waves of one launch, cold inputs)
     "llama8b-prefill512-d4096-timeline": ("llama8b", "timeline", 8192, ("prefill", 4096, 512)),
@@ -119,7 +123,7 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
         "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
-        "qwen1.5b-decode-32k-cutoffs", "weights-read-patterns", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
+        "qwen1.5b-decode-32k-cutoffs", "weights-read-patterns", "llama8b-logits", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -1250,9 +1254,89 @@ def run_decode_layer(torch, kernels, name, steps, warmup, with_cpu):
     return res
 
 
+def run_logits(torch, kernels, name, steps, warmup, with_cpu):
+    """One step = the last RMS norm and the output matrix (Q6_K, vocabulary x n_embd) over one token's residual
+    stream: orin_rms_norm + orin_gemv, as the reference ends a decode step (src/model_gpu.cu:303-306); replayed
+    from a graph over copies of the matrix that rotate through more memory than the last-level cache holds.
+    value = bytes of the matrix per second."""
+    from oracle import ref
+    from orin_llm_amd import layer as ly
+
+    shape_name, _, _, n_vocab = WORKLOADS[name]
+    ne = SHAPES[shape_name]["n_embd"]
+    wt = ly.Q6_K
+    nbytes = ly.row_bytes(wt, ne) * n_vocab
+    n_copies = max(2, int(np.ceil(0.6e9 / nbytes)))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(777)
+    ws = [random_weight(torch, gen, wt, ne, n_vocab) for _ in range(n_copies)]
+    x = torch.randn(ne, generator=gen, device="cuda")
+    nw = 1.0 + 0.1 * torch.randn(ne, generator=gen, device="cuda")
+    xn, y = torch.zeros(ne, device="cuda"), torch.zeros(n_vocab, device="cuda")
+    k = 0
+
+    def one_step():
+        nonlocal k
+        ly.rms_norm(x, nw, ne, 1e-6, xn)
+        ly.gemv(wt, ws[k % n_copies], xn, y, ne, n_vocab)
+        k += 1
+
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+            for _ in range(n_copies):
+                one_step()
+    finally:
+        kernels.set_stream(torch.cuda.current_stream().cuda_stream)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(max(1, warmup)):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us = e0.elapsed_time(e1) * 1e3 / (steps * n_copies)
+    del g
+    # parity: a sample of rows of the last matrix used, against the oracle's product over the oracle's norm
+    k = 0
+    one_step()
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    rb = ly.row_bytes(wt, ne)
+    xh, nwh = x.cpu().numpy(), nw.cpu().numpy()
+    t_cpu = time.perf_counter()
+    xnh = ref.rms_norm(xh, nwh, 1e-6)
+    rows = sorted(set([0, 1, 15, 16, n_vocab // 2, n_vocab - 17, n_vocab - 1]) | set(int(r) for r in np.random.default_rng(5).integers(0, n_vocab - 256, 41)))
+    err, n_rows = 0.0, 0
+    for r in rows:
+        m = min(256, n_vocab - r)
+        want = ref.gemv(wt, ws[0][r * rb:(r + m) * rb].cpu().numpy(), xnh, ne, m).astype(np.float64)
+        err = max(err, float(np.abs(got[r:r + m] - want).max() / max(np.abs(want).max(), 1e-30)))
+        n_rows += m
+    cpu_s = time.perf_counter() - t_cpu
+    res = dict(value=nbytes * n_copies * steps / wall / 1e9, unit="GB/s", ms_per_step=wall / steps * 1e3 / n_copies,
+               config=dict(workload=name, shape=f"n_embd {ne}, vocabulary {n_vocab}", weights="Q6_K", MB=round(nbytes / 1e6, 1),
+                           copies_rotated=n_copies, launch="graph"),
+               roofline=dict(bound="hbm", achieved=nbytes / (us * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                             frac=nbytes / (us * 1e-6) / PEAK_BYTES, traffic=None,
+                             kernel="rms_norm_kernel + gemv_rows_kernel<Q6_K> (last norm + output matrix)", launch_us=us,
+                             bytes_per_launch=nbytes),
+               parity=dict(err_row=err, err_floor1pct=err, rows=f"{n_rows} logits in runs of 256 (first, last, middle, random), max |got - want| / max |want| per run, vs the CPU oracle"))
+    if with_cpu:
+        res["cpu_baseline"] = dict(value=n_rows * rb / cpu_s / 1e9, unit="GB/s", cores=1, kind="port", sample=f"{n_rows} of {n_vocab} rows, {cpu_s:.1f} s")
+    del ws
+    torch.cuda.empty_cache()
+    return res
+
+
 def run(torch, kernels, name, steps, warmup, with_cpu):
     kind = WORKLOADS[name][1]
-    fn = {"decode_layer": run_decode_layer, "prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "copy": run_copy, "read": run_read, "patterns": run_patterns, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
+    fn = {"decode_layer": run_decode_layer, "prefill": run_prefill, "decode": run_decode, "decode_store": run_decode, "decode_rope_store": run_decode, "logits": run_logits, "copy": run_copy, "read": run_read, "patterns": run_patterns, "handoff": run_handoff, "timeline": run_timeline, "cutoffs": run_cutoffs, "kv_store": run_kv_store,
           "kv_shift": run_kv_shift, "rope": run_rope}[kind]
     return fn(torch, kernels, name, steps, warmup, with_cpu)
 

@@ -30,7 +30,7 @@ def test_decode_bytes_counts_k_and_v_once_plus_q_and_out():
 def test_workload_table_is_consistent():
     assert bench.WORKLOADS["qwen1.5b-prefill512"][3] == [(0, 512), (3584, 512)]   # the configuration the metric is quoted on
     for name, (shape, kind, n_ctx, spec) in bench.WORKLOADS.items():
-        assert kind in ("prefill", "decode", "decode_store", "decode_rope_store", "copy", "read", "patterns", "handoff", "timeline", "cutoffs", "kv_store", "kv_shift", "rope", "decode_layer"), name
+        assert kind in ("prefill", "decode", "decode_store", "decode_rope_store", "copy", "read", "patterns", "logits", "handoff", "timeline", "cutoffs", "kv_store", "kv_shift", "rope", "decode_layer"), name
         if kind == "prefill":
             assert all(P + B <= n_ctx for P, B in spec), name
         if kind in ("decode", "decode_store"):
