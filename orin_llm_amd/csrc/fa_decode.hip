@@ -170,6 +170,21 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         cs_given = *reinterpret_cast<const float2*>(anp);
         ff_given = *ffp;
     }
+    // (store, rotate + store) The new row, in as few loads as will do, by every wave: only the one whose tiles
+    // include the row's uses it (at its last tile), but which wave that is depends on the position, which is
+    // still on its way, and a load issued later, while the CU's tiles stream in, holds its wave up for a few
+    // hundred cycles each (three of them: 0.5 us between the query's arrival and its conversion).  Here they
+    // are small loads ahead of the flood, hits in the cache for all but the first wave to ask.  K: elements
+    // 4*lane .. 4*lane+3 (the lanes hand each other the pieces they hold of a K row through LDS then); V: piece
+    // lane % (D/8), which is what the lane holds of a V row.
+    float4 k_raw = float4{0.f, 0.f, 0.f, 0.f}, v_raw[2] = {k_raw, k_raw};
+    if constexpr (STORE) {
+        const float* kp4 = a.k_new + (size_t)kvh * D + (lane % (D / 4)) * 4;
+        const float* vp8 = a.v_new + (size_t)kvh * D + (lane % G::kChunksPerRow) * 8;
+        k_raw = *reinterpret_cast<const float4*>(kp4);
+        v_raw[0] = *reinterpret_cast<const float4*>(vp8);
+        v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
+    }
     __builtin_amdgcn_sched_barrier(0); // the small loads first: they return first, and nothing that needs them waits for a tile
 
     // The query loads above are used only behind the early return below, and left alone the
@@ -251,7 +266,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         qf[kk][4] = x1.x; qf[kk][5] = x1.y; qf[kk][6] = x1.z; qf[kk][7] = x1.w;
     }
     // (rotate + store) the rotation of this lane's 8 elements of every k-step, by the wave's table
-    __shared__ float sh_cs_all[ROPE ? kWaves : 1][D / 2][2];
+    __shared__ __attribute__((aligned(16))) float sh_cs_all[ROPE ? kWaves : 1][D / 2][2];
     __shared__ __attribute__((aligned(16))) float sh_krow_all[STORE ? kWaves : 1][D];
     float (*const sh_cs)[2] = sh_cs_all[ROPE ? wave : 0];
     // x0, x1: this lane's elements of k-steps kk and kk + kSteps/2 (head_dim indices kk*32 + grp*8 + e
@@ -264,11 +279,28 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
                 rope_rotate(x0[e], x1[e], sh_cs[i][0], sh_cs[i][1]);
             }
         } else {      // elements 2i and 2i + 1, below n_rot
+            // No branch per pair: el0 differs from lane to lane, and a branch around each pair's table
+            // read makes the wave wait out sixteen LDS round trips one after the other (1.7 us of a
+            // Llama-3-8B launch).  Every lane reads an entry (its own, or the table's last), all reads
+            // go out together, and a pair past n_rot keeps its values by a select.
+            const int last = a.n_rot / 2 - 1;
+            float2 cs0[4], cs1[4];
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
                 const int el0 = kk * 32 + grp * 8 + e, el1 = el0 + D / 2;
-                if (el0 < a.n_rot) rope_rotate(x0[e], x0[e + 1], sh_cs[el0 / 2][0], sh_cs[el0 / 2][1]);
-                if (el1 < a.n_rot) rope_rotate(x1[e], x1[e + 1], sh_cs[el1 / 2][0], sh_cs[el1 / 2][1]);
+                cs0[e / 2] = *reinterpret_cast<const float2*>(sh_cs[min(el0 / 2, last)]);
+                cs1[e / 2] = *reinterpret_cast<const float2*>(sh_cs[min(el1 / 2, last)]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const int el0 = kk * 32 + grp * 8 + e, el1 = el0 + D / 2;
+                float a0 = x0[e], a1 = x0[e + 1], b0 = x1[e], b1 = x1[e + 1];
+                rope_rotate(a0, a1, cs0[e / 2].x, cs0[e / 2].y);
+                rope_rotate(b0, b1, cs1[e / 2].x, cs1[e / 2].y);
+                x0[e] = el0 < a.n_rot ? a0 : x0[e];
+                x0[e + 1] = el0 < a.n_rot ? a1 : x0[e + 1];
+                x1[e] = el1 < a.n_rot ? b0 : x1[e];
+                x1[e + 1] = el1 < a.n_rot ? b1 : x1[e + 1];
             }
         }
     };
@@ -310,24 +342,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         }
     }
 
-    __builtin_amdgcn_sched_barrier(0);
-    // The new row, requested by the one wave whose tiles include the row's (its last one, so the
-    // row has long arrived when it is wanted) in as few loads as will do -- and only now, behind
-    // the query's conversion: while a CU's tiles stream in, every further load a wave issues
-    // holds it up for a few hundred cycles, which the conversion can do without.  K: elements 4*lane ..
-    // 4*lane+3 (the lanes hand each other the pieces they hold of a K row through LDS then); V:
-    // piece lane % (D/8), which is what the lane holds of a V row.  The other waves make the same
-    // loads from the query, which their cache holds: no branch, so no wait where one would end.
-    float4 k_raw = float4{0.f, 0.f, 0.f, 0.f}, v_raw[2] = {k_raw, k_raw};
-    if constexpr (STORE) {
-        const int pt = pos / kTile;
-        const bool owner = store && pt >= tile_first && (pt - tile_first) % tile_step == 0;
-        const float* kp4 = (owner ? a.k_new + (size_t)kvh * D : q) + (lane % (D / 4)) * 4;
-        const float* vp8 = (owner ? a.v_new + (size_t)kvh * D : q) + (lane % G::kChunksPerRow) * 8;
-        k_raw = *reinterpret_cast<const float4*>(kp4);
-        v_raw[0] = *reinterpret_cast<const float4*>(vp8);
-        v_raw[1] = *reinterpret_cast<const float4*>(vp8 + 4);
-    }
     __builtin_amdgcn_sched_barrier(0);
     FA_STAMP(2);
     // m_ref: reference maximum of the raw scores (before the scale); l_run: this lane's share of
