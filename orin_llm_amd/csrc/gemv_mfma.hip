@@ -26,6 +26,11 @@
 //     10 % slower) and moved to the matrix instruction's lanes by one lane permutation per register.
 //   * The four waves of a workgroup take every fourth 256-element block of the same 16 rows and meet
 //     in LDS at the end; blocks are requested one iteration ahead, across row tiles.
+//   * Q4_K, Q5_K and Q6_K matrices made of whole 16-row tiles -- every matrix of a model -- take a second
+//     kernel with the same arithmetic and another way to the bytes (gemv_rows_kernel, further down): rows
+//     read in lane-linear runs of two blocks with streaming loads and laid out for the matrix instruction
+//     through a wave's own LDS buffer, which this machine's memory path serves a quarter faster.  The
+//     kernel described above remains for Q8_0 and for matrices with a ragged last tile.
 #include "layer_common.hpp"
 
 #include <stdlib.h>
