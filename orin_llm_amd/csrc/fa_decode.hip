@@ -220,13 +220,46 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     const int tile_step = wu * n_splits;
     int tile = tile_first;
     float* const qs = reinterpret_cast<float*>(smem + G::kQOff);
+    __shared__ __attribute__((aligned(16))) float sh_cs_all[ROPE ? kWaves : 1][D / 2][2];
+    __shared__ __attribute__((aligned(16))) float sh_krow_all[STORE ? kWaves : 1][D];
+    float (*const sh_cs)[2] = sh_cs_all[ROPE ? wave : 0];
+    const bool rot_early = ROPE && !a.neox && a.rope_angles != nullptr; // (the query is rotated piece by piece before it is parked)
     if (id * wu < n_tiles) {
         // The query pieces meet in LDS: each wave parks the piece it fetched, then a barrier that
         // waits for LDS only.  Ahead of the tile requests, where the eight waves are still in
         // step (the position and the pieces arrive together); behind them the waves are microseconds
         // apart -- the load unit takes a CU's 128 KB of requests as fast as memory answers them --
         // and a barrier there holds every wave's products until the last has all its requests out.
-        *reinterpret_cast<float4*>(qs + col * G::kQStride + (q_piece >> 1) * 32 + grp * 8 + (q_piece & 1) * 4) = q_share;
+        float4 q_park = q_share;
+        if constexpr (ROPE) {
+            // "Normal" pairs are neighbours, so the piece a wave fetched holds two whole pairs: with the caller's
+            // table of angles at hand the wave rotates just those before it parks the piece, and nobody has to
+            // rotate the whole query behind the barrier (eight waves each used to: sixteen table reads and as
+            // many rotations a lane between the query's arrival and its conversion; 0.4 us of a Llama-3-8B
+            // launch pair).  Without a table the angles are a power, a sine and a cosine away, which must not
+            // sit ahead of the tile requests.  ("neox" pairs sit half a head apart, in another wave's piece:
+            // fetching that piece as well and rotating early was built and gained nothing.)
+            if (rot_early) {
+                if (lane < a.n_rot / 2) {
+                    sh_cs[lane][0] = cs_given.x;
+                    sh_cs[lane][1] = cs_given.y;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const int e0 = (q_piece >> 1) * 32 + grp * 8 + (q_piece & 1) * 4, last = max(a.n_rot / 2 - 1, 0);
+                const float2 c0 = *reinterpret_cast<const float2*>(sh_cs[min(e0 / 2, last)]);
+                const float2 c1 = *reinterpret_cast<const float2*>(sh_cs[min(e0 / 2 + 1, last)]);
+                float x0 = q_park.x, x1 = q_park.y, y0 = q_park.z, y1 = q_park.w;
+                rope_rotate(x0, x1, c0.x, c0.y);
+                rope_rotate(y0, y1, c1.x, c1.y);
+                q_park.x = e0 < a.n_rot ? x0 : q_park.x;
+                q_park.y = e0 < a.n_rot ? x1 : q_park.y;
+                q_park.z = e0 + 2 < a.n_rot ? y0 : q_park.z;
+                q_park.w = e0 + 2 < a.n_rot ? y1 : q_park.w;
+            }
+        }
+        *reinterpret_cast<float4*>(qs + col * G::kQStride + (q_piece >> 1) * 32 + grp * 8 + (q_piece & 1) * 4) = q_park;
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         fetch_k(tile);
         fetch_v(tile);
@@ -266,9 +299,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         qf[kk][4] = x1.x; qf[kk][5] = x1.y; qf[kk][6] = x1.z; qf[kk][7] = x1.w;
     }
     // (rotate + store) the rotation of this lane's 8 elements of every k-step, by the wave's table
-    __shared__ __attribute__((aligned(16))) float sh_cs_all[ROPE ? kWaves : 1][D / 2][2];
-    __shared__ __attribute__((aligned(16))) float sh_krow_all[STORE ? kWaves : 1][D];
-    float (*const sh_cs)[2] = sh_cs_all[ROPE ? wave : 0];
     // x0, x1: this lane's elements of k-steps kk and kk + kSteps/2 (head_dim indices kk*32 + grp*8 + e
     // and the same + head_dim/2)
     auto rotate2 = [&](float (&x0)[8], float (&x1)[8], int kk) {
@@ -283,7 +313,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
             // read makes the wave wait out sixteen LDS round trips one after the other (1.7 us of a
             // Llama-3-8B launch).  Every lane reads an entry (its own, or the table's last), all reads
             // go out together, and a pair past n_rot keeps its values by a select.
-            const int last = a.n_rot / 2 - 1;
+            const int last = max(a.n_rot / 2 - 1, 0); // (n_rot = 0: nothing is rotated, entry 0 is read and not used)
             float2 cs0[4], cs1[4];
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
@@ -312,7 +342,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         // are the same wave's, and a wave's LDS operations complete in order.
         static_assert(D / 2 <= 64, "one lane per pair");
         const int half = a.n_rot / 2;
-        if (lane < half) {
+        if (!rot_early && lane < half) {
             if (!a.rope_angles) {
                 float freq = rope_freq_base(lane, a.n_rot, a.theta);
                 if (a.freq_factors) freq /= ff_given;
@@ -326,8 +356,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (!rot_early) {
 #pragma unroll
-        for (int kk = 0; kk < G::kSteps / 2; ++kk) rotate2(qf[kk], qf[kk + G::kSteps / 2], kk);
+            for (int kk = 0; kk < G::kSteps / 2; ++kk) rotate2(qf[kk], qf[kk + G::kSteps / 2], kk);
+        }
     }
     // ---- query heads -> B operands, fp16 hi + lo ----
     h8 qhi[G::kSteps], qlo[G::kSteps];
