@@ -550,7 +550,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_mfma_kernel(const GemvArgs a
 // together as well.  Barriers wait for LDS only, row sums leave through stores and atomic adds without a return
 // value, a tile's bias values travel with its items: nothing in the loop waits for anything but the oldest item.
 // Requires whole 16-row tiles.  (Deeper request queues, three and four items a wave, were slower in both kernels,
-// and so were four-block items: what bounds the kernels after the loads is the vector ALU, about 85 instructions
+// and so were four-block items: what bounds the kernels after the loads is the vector ALU, about 74 instructions
 // per block and wave for the nibbles, the six-bit pairs and the digit sums.)
 constexpr int kRowsMaxCb = 2; // blocks of a row in an item, at most
 constexpr int kRowsRedBytes = 2 * kMaxWaves * 2 * 16 * 4 + 64; // two sets of partial row sums (tiles alternate: one barrier a tile), the waves' sums of squares
@@ -739,8 +739,11 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
 #pragma unroll
         for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(transit + loff[i]) = r[i];
         const int cb = min(CB, nb - cs_c * CB);
+        // (unrolled over CB with a test per block, not a loop over cb: every LDS offset is a constant of its instruction)
         float v = 0.0f;
-        for (int j = 0; j < cb; ++j) v += F::from_lds(transit + (c.n * R + j * P) * 16, c, addr, cs_c * CB + j);
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+            if (j < cb) v += F::from_lds(transit + (c.n * R + j * P) * 16, c, addr, cs_c * CB + j);
         rowacc[m] += v;
         if (m == M - 1) {
             cs_c += kWaves;
