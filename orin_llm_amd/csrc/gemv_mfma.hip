@@ -153,8 +153,29 @@ __device__ __forceinline__ float half_of(unsigned bits) { return (float)__builti
 __device__ __forceinline__ unsigned from_lane(int src_lane4, unsigned v) {
     return (unsigned)__builtin_amdgcn_ds_bpermute(src_lane4, (int)v);
 }
+// (the upper two digits' sums are put together as integers: below 2^30 for every block type, and rounded once on
+// conversion where the fused multiply-add of the converted parts would round, to the same value)
 __device__ __forceinline__ float digits_sum(const i32x4& acc) {
-    return ((float)acc[0] * 256.0f + (float)acc[1]) * 256.0f + (float)acc[2];
+    return (float)(acc[0] * 256 + acc[1]) * 256.0f + (float)acc[2];
+}
+// Every byte's low nibble from a, its high nibble from b, in one instruction (spelled out, since the compiler, which
+// knows which bits of b can be set, narrows the mask and then needs an AND and an AND-OR).
+__device__ __forceinline__ unsigned low_nibbles_of(unsigned a, unsigned b) {
+    unsigned r;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(r) : "v"(0x0f0f0f0fu), "v"(a), "v"(b));
+    return r;
+}
+// LDS byte offset of a lane's A operand: base + x for a lane that holds digits (step 1), base (the zero bytes) for
+// one whose rows are zero (step 0); x is the same in every lane.  One 24-bit multiply-add.
+__device__ __forceinline__ int operand_at(int base, int step, int x) {
+    return (int)(__umul24((unsigned)x, (unsigned)step) + (unsigned)base);
+}
+// (the step as a value the compiler knows nothing of: told that it is 0 or 1, it replaces the multiply-add by a
+// move, a select and an add)
+__device__ __forceinline__ int opaque_step(bool on) {
+    int step = on ? 1 : 0;
+    asm volatile("" : "+v"(step));
+    return step;
 }
 
 // What a lane needs to know of itself: as a loader (row ln of the tile, 16-byte piece lg), as a lane of
@@ -183,7 +204,7 @@ struct MFK45 {
         u32x4 qh;          // (Q5_K) the 16 bytes of fifth bits that cover this lane's elements
     };
     struct Addr {
-        int lo_base, hi_base, lo_step, hi_step; // LDS byte offsets of this lane's A operands; a lane whose row is zero reads the 16 zero bytes, stride 0
+        int lo_base, hi_base, lo_step, hi_step; // LDS byte offsets of this lane's A operands and whether they move with the block (1); a lane whose row is zero reads the 16 zero bytes (0)
     };
     static __device__ __forceinline__ void load(const unsigned char* blk, int lg, Raw& r) {
         r.hdr = load16_aligned(blk);
@@ -196,7 +217,7 @@ struct MFK45 {
         const bool live = ad < 3 && (ap >> 1) == (g >> 1);
         const int elem = 64 * (g >> 1) + 16 * (g & 1);
         const bool lo = live && (ap & 1) == 0, hi = live && (ap & 1) == 1;
-        return Addr{lo ? ad * c.n_in + elem : c.zero_off, hi ? ad * c.n_in + elem + 32 : c.zero_off, lo ? 256 : 0, hi ? 256 : 0};
+        return Addr{lo ? ad * c.n_in + elem : c.zero_off, hi ? ad * c.n_in + elem + 32 : c.zero_off, opaque_step(lo), opaque_step(hi)};
     }
     static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
         // (the loading lane holds piece lg of its row, and lane (n, g) wants piece g of row n: the bytes of
@@ -211,7 +232,11 @@ struct MFK45 {
             q1[i] = from_lane(c.src_lane4, r.q1[i]);
             q2[i] = from_lane(c.src_lane4, r.q2[i]);
         }
-        return math(dd, bb, q1, q2, fifth, c, ad, b);
+        const unsigned b0 = bb & 0xffu, b1 = (bb >> 8) & 0xffu, b2 = (bb >> 16) & 0xffu;
+        // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
+        const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
+        const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
+        return math(dd, sc, mn, q1, q2, fifth, c, ad, b);
     }
     // A block laid out in LDS piece after piece (the kernel that reads rows in long runs): piece k is the block's
     // bytes 16 k ...
@@ -224,24 +249,23 @@ struct MFK45 {
         const u32x4 q2 = *reinterpret_cast<const u32x4*>(blk + kQs + 64 + 16 * c.g);
         u32x4 fifth = {0u, 0u, 0u, 0u};
         if constexpr (FIVE) fifth = *reinterpret_cast<const u32x4*>(blk + 16 + 16 * (c.g & 1)) >> (unsigned)(2 * (c.g >> 1));
-        const unsigned bb = ((hdr.y >> (8 * c.g)) & 0xffu) | (((hdr.z >> (8 * c.g)) & 0xffu) << 8) | (((hdr.w >> (8 * c.g)) & 0xffu) << 16);
-        return math(hdr.x, bb, q1, q2, fifth, c, ad, b);
+        // the six-bit pairs straight out of the three words (bit fields at 8 g: no byte is put together first)
+        const unsigned s8 = 8 * c.g;
+        const float sc[2] = {(float)__builtin_amdgcn_ubfe(hdr.y, s8, 6), (float)(__builtin_amdgcn_ubfe(hdr.w, s8, 4) | ((hdr.y >> (s8 + 2)) & 0x30u))};
+        const float mn[2] = {(float)__builtin_amdgcn_ubfe(hdr.z, s8, 6), (float)(__builtin_amdgcn_ubfe(hdr.w, s8 + 4, 4) | ((hdr.z >> (s8 + 2)) & 0x30u))};
+        return math(hdr.x, sc, mn, q1, q2, fifth, c, ad, b);
     }
-    // In lane (n, g): dd = the block's two fp16 scales, bb = bytes g of the three words of packed six-bit pairs,
-    // q1 / q2 = piece g of each half of the nibbles, fifth = the fifth bits of this lane's elements shifted down
-    // to bit 0 (Q5_K).
-    static __device__ __forceinline__ float math(unsigned dd, unsigned bb, const u32x4& q1, const u32x4& q2, const u32x4& fifth,
-                                                 const LaneCtx& c, const Addr& ad, int b) {
+    // In lane (n, g): dd = the block's two fp16 scales, sc / mn = the six-bit scales and minima of sub-blocks g (first
+    // half of the block) and 4 + g (second half), q1 / q2 = piece g of each half of the nibbles, fifth = the fifth
+    // bits of this lane's elements shifted down to bit 0 (Q5_K).
+    static __device__ __forceinline__ float math(unsigned dd, const float (&sc)[2], const float (&mn)[2], const u32x4& q1, const u32x4& q2,
+                                                 const u32x4& fifth, const LaneCtx& c, const Addr& ad, int b) {
         const float d = half_of(dd & 0xffffu), dmin = half_of(dd >> 16);
-        const unsigned b0 = bb & 0xffu, b1 = (bb >> 8) & 0xffu, b2 = (bb >> 16) & 0xffu;
-        // pairs g (first half of the block) and 4 + g (second half) of the twelve packed bytes
-        const float sc[2] = {(float)(b0 & 63u), (float)((b2 & 0x0fu) | ((b0 >> 6) << 4))};
-        const float mn[2] = {(float)(b1 & 63u), (float)((b2 >> 4) | ((b1 >> 6) << 4))};
-        float out = 0.0f;
+        float scaled[2], offset[2]; // sum of sc * q * x and of mn * x over a sub-block pair; the block's two scales come last
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + ad.lo_base + b * ad.lo_step + (ad.lo_step ? 128 * h : 0));
-            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + ad.hi_base + b * ad.hi_step + (ad.hi_step ? 128 * h : 0));
+            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.lo_base, ad.lo_step, 256 * b + 128 * h));
+            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.hi_base, ad.hi_step, 256 * b + 128 * h));
             const XPair xp = c.pairs[8 * b + 4 * h + c.g];
             const u32x4 qs = h ? q2 : q1;
             i32x4 lo, hi;
@@ -260,9 +284,10 @@ struct MFK45 {
             i32x4 acc = {0, 0, 0, 0};
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, lo, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, hi, acc, 0, 0, 0);
-            out += (d * sc[h]) * (digits_sum(acc) * xp.scale) - (dmin * mn[h]) * xp.sum;
+            scaled[h] = sc[h] * (digits_sum(acc) * xp.scale);
+            offset[h] = mn[h] * xp.sum;
         }
-        return out;
+        return d * (scaled[0] + scaled[1]) - dmin * (offset[0] + offset[1]);
     }
 };
 template <>
@@ -300,14 +325,14 @@ struct MF<kQ8_0> {
         const bool live = ad < 3 && (ap & 1) == (g >> 1);
         const int elem = 32 * ap + 16 * (g & 1);
         const bool r0 = live && (ap >> 1) == 0, r1 = live && (ap >> 1) == 1;
-        return Addr{r0 ? ad * c.n_in + elem : c.zero_off, r1 ? ad * c.n_in + elem : c.zero_off, r0 ? 256 : 0, r1 ? 256 : 0};
+        return Addr{r0 ? ad * c.n_in + elem : c.zero_off, r1 ? ad * c.n_in + elem : c.zero_off, opaque_step(r0), opaque_step(r1)};
     }
     static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
-        float out = 0.0f;
+        float out[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const i32x4 a0 = *reinterpret_cast<const i32x4*>(c.smem + ad.lo_base + b * ad.lo_step + (ad.lo_step ? 128 * h : 0));
-            const i32x4 a1 = *reinterpret_cast<const i32x4*>(c.smem + ad.hi_base + b * ad.hi_step + (ad.hi_step ? 128 * h : 0));
+            const i32x4 a0 = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.lo_base, ad.lo_step, 256 * b + 128 * h));
+            const i32x4 a1 = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.hi_base, ad.hi_step, 256 * b + 128 * h));
             const XPair xp = c.pairs[8 * b + 4 * h + c.g];
             const float d = half_of(from_lane(c.src_lane4, r.d[h]));
             i32x4 w0, w1;
@@ -319,9 +344,9 @@ struct MF<kQ8_0> {
             i32x4 acc = {0, 0, 0, 0};
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, w0, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, w1, acc, 0, 0, 0);
-            out += d * (digits_sum(acc) * xp.scale);
+            out[h] = d * (digits_sum(acc) * xp.scale);
         }
-        return out;
+        return out[0] + out[1];
     }
 };
 
@@ -356,7 +381,7 @@ struct MF<kQ6_K> {
     static __device__ __forceinline__ Addr addr(const LaneCtx& c) {
         const int ap = c.am >> 2, ad = c.am & 3;
         const bool live = ad < 3 && ap == c.g;
-        return Addr{live ? ad * c.n_in + 16 * c.g : c.zero_off, live ? 1 : 0};
+        return Addr{live ? ad * c.n_in + 16 * c.g : c.zero_off, opaque_step(live)};
     }
     static __device__ __forceinline__ float block(const Raw& r, const LaneCtx& c, const Addr& ad, int b) {
         // scales 8 h + g and 8 h + 4 + g of both halves: byte lg of each of the loading lane's four words
@@ -400,28 +425,28 @@ struct MF<kQ6_K> {
                                                  const Addr& ad, int b) {
         const float d = half_of(dd & 0xffffu);
         const int s1 = 2 * (c.g >> 1);
-        float out = 0.0f;
+        float out[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int off = ad.step ? 256 * b + 128 * h : 0;
-            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + ad.base + off);
-            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + ad.base + off + (ad.step ? 64 : 0));
+            const i32x4 alo = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.base, ad.step, 256 * b + 128 * h));
+            const i32x4 ahi = *reinterpret_cast<const i32x4*>(c.smem + operand_at(ad.base, ad.step, 256 * b + 128 * h + 64));
             const XPair xlo = c.pairs[16 * b + 8 * h + c.g], xhi = c.pairs[16 * b + 8 * h + 4 + c.g];
             i32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const unsigned l = ql[h][i], u = qh[h][i] >> s1;
-                lo[i] = (int)((l & 0x0f0f0f0fu) | ((u & 0x03030303u) << 4));
-                hi[i] = (int)(((l >> 4) & 0x0f0f0f0fu) | (((u >> 4) & 0x03030303u) << 4));
+                // u: this lane's two bit pairs of every byte at bits 0, 1 and 4, 5, nothing else; each lands in the
+                // high nibble of its element by one bit-field insert
+                const unsigned l = ql[h][i], u = (qh[h][i] >> s1) & 0x33333333u;
+                lo[i] = (int)low_nibbles_of(l, u << 4);
+                hi[i] = (int)low_nibbles_of(l >> 4, u);
             }
             const i32x4 zero = {0, 0, 0, 0};
             const i32x4 acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, lo, zero, 0, 0, 0);
             const i32x4 acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, hi, zero, 0, 0, 0);
             const float sc_lo = (float)((int)(ss << (24 - 16 * h)) >> 24), sc_hi = (float)((int)(ss << (16 - 16 * h)) >> 24);
-            out += (d * sc_lo) * (digits_sum(acc_lo) * xlo.scale - 32.0f * xlo.sum) +
-                   (d * sc_hi) * (digits_sum(acc_hi) * xhi.scale - 32.0f * xhi.sum);
+            out[h] = sc_lo * (digits_sum(acc_lo) * xlo.scale - 32.0f * xlo.sum) + sc_hi * (digits_sum(acc_hi) * xhi.scale - 32.0f * xhi.sum);
         }
-        return out;
+        return d * (out[0] + out[1]);
     }
 };
 
@@ -740,9 +765,9 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(transit + loff[i]) = r[i];
         const int cb = min(CB, nb - cs_c * CB);
         // (unrolled over CB with a test per block, not a loop over cb: every LDS offset is a constant of its instruction)
-        float v = 0.0f;
+        float v = F::from_lds(transit + c.n * R * 16, c, addr, cs_c * CB);
 #pragma unroll
-        for (int j = 0; j < CB; ++j)
+        for (int j = 1; j < CB; ++j)
             if (j < cb) v += F::from_lds(transit + (c.n * R + j * P) * 16, c, addr, cs_c * CB + j);
         rowacc[m] += v;
         if (m == M - 1) {
