@@ -687,7 +687,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         // digits (stamps in a development build: first digits 1.4 us after the requests, the second chunk's 2.1 us
         // later, the first item 0.5 us after that).
         constexpr int kPre = kWaves == 8 ? 2 : 4; // (eight-wave workgroups: fewer chunks a wave, and registers for four waves a SIMD)
-        float xs[kPre][kPasses][8] = {}, gs[kPre][kPasses][8] = {};
+        float xs[kPre][kPasses][8], gs[kPre][kPasses][8]; // (read under the conditions they are loaded under)
 #pragma unroll
         for (int i = 0; i < kPre; ++i) {
             const int ch = wave + i * kWaves, end = min((ch + 1) * CB * 256, n_in);
