@@ -599,8 +599,9 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     using G = RowsGeom<T, CB>;
     constexpr int M = DUAL ? 2 : 1, P = G::P, R = G::R, NL = G::NL;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const int nb_row = a.n_in >> 8;
-    const int b0 = (int)blockIdx.z * nb_row / (int)gridDim.z, nb = ((int)blockIdx.z + 1) * nb_row / (int)gridDim.z - b0;
+    // (this share's blocks of a row, from what the launcher divided: no division ahead of the first requests)
+    const int b0 = (int)blockIdx.z * a.share_blocks + min((int)blockIdx.z, a.share_extra);
+    const int nb = a.share_blocks + ((int)blockIdx.z < a.share_extra ? 1 : 0);
     const int n_in = nb << 8;
     float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
     const GemvSeg seg = a.seg[blockIdx.y];
@@ -620,7 +621,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
                                            static_cast<const unsigned char*>(DUAL ? a.w_up : seg.w)};
     const int n_chunks = (nb + CB - 1) / CB;
     const int my_chunks = wave < n_chunks ? (n_chunks - wave + kWaves - 1) / kWaves : 0;
-    const int n_mine = (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int n_mine = n_tiles <= (int)gridDim.x ? 1 : (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
     const int total = n_mine * my_chunks * M;
     // slot 64 i + lane of an item: (row, piece), row-major
     unsigned goff[NL];
@@ -858,7 +859,10 @@ template <int T, bool DUAL, int kWaves, int CB>
 bool launch_rows_as(const GemvArgs& a, dim3 grid, int n_in_wg, hipStream_t stream) {
     const size_t lds = RowsGeom<T, CB>::lds_bytes(n_in_wg, kWaves);
     if (lds > kMfmaLdsMax) return false;
-    hipLaunchKernelGGL((gemv_rows_kernel<T, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, a);
+    GemvArgs b = a;
+    b.share_blocks = (a.n_in / 256) / (int)grid.z;
+    b.share_extra = (a.n_in / 256) % (int)grid.z;
+    hipLaunchKernelGGL((gemv_rows_kernel<T, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, b);
     return true;
 }
 
@@ -960,6 +964,8 @@ hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) 
     a.n_seg_types = 1;
     bool rows = rows_enabled();
     for (int i = 0; i < a.n_seg; ++i) rows = rows && a.seg[i].n_out % 16 == 0 && a.seg[i].type != kQ8_0;
+    a.share_blocks = a.n_in / 256; // (one share: whole rows)
+    a.share_extra = 0;
     if (rows) {
         const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu), nb = a.n_in / 256;
         const dim3 gr(min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16), a.n_seg);

@@ -33,6 +33,7 @@ struct GemvArgs {
     // filled in by the launcher
     size_t row_bytes;
     int team_waves, wgs_per_cu, mfma_wgs_per_cu, n_seg_types, k_split_override;
+    int share_blocks, share_extra; // blocks of a row per share of it (gridDim.z shares), and how many shares take one more
 };
 
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
