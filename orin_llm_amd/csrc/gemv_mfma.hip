@@ -599,12 +599,19 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     using G = RowsGeom<T, CB>;
     constexpr int M = DUAL ? 2 : 1, P = G::P, R = G::R, NL = G::NL;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const GemvSeg seg = a.seg[blockIdx.y];
+    {
+        // Every argument word the kernel reads, asked for here in one batch: left to the compiler the scalar loads
+        // sit ahead of their uses, four dependent trips to the argument block before the first weight request.
+        const int grid_x = gridDim.x;
+        asm volatile("" ::"s"(seg.w), "s"(seg.bias), "s"(seg.y), "s"(seg.n_out), "s"(seg.row_bytes), "s"(a.w_up), "s"(a.x), "s"(a.norm_w),
+                     "s"(a.eps), "s"(a.accumulate), "s"(a.row_bytes), "s"(a.n_seg_types), "s"(a.share_blocks), "s"(a.share_extra), "s"(grid_x));
+    }
     // (this share's blocks of a row, from what the launcher divided: no division ahead of the first requests)
     const int b0 = (int)blockIdx.z * a.share_blocks + min((int)blockIdx.z, a.share_extra);
     const int nb = a.share_blocks + ((int)blockIdx.z < a.share_extra ? 1 : 0);
     const int n_in = nb << 8;
     float* const red = reinterpret_cast<float*>(smem + L::red_off(n_in));
-    const GemvSeg seg = a.seg[blockIdx.y];
     const unsigned row_bytes = (unsigned)(a.n_seg_types ? seg.row_bytes : a.row_bytes);
     const int n_tiles = seg.n_out >> 4;
     if ((int)blockIdx.x >= n_tiles) return; // (whole workgroup: a shorter matrix of a shared launch)
