@@ -103,6 +103,10 @@ WORKLOADS = {
     "llama8b-decode-8k-cutoffs": ("llama8b", "cutoffs", 8192, 8192),   # (shapes where a wave has one tile: the cut-off kernel leaves after its first)
     "qwen1.5b-decode-32k-timeline": ("qwen1.5b", "timeline", 32768, ("decode", 32768, 1)),
     "qwen7b-decode-32k-timeline": ("qwen7b", "timeline", 32768, ("decode", 32767, 1)),
+    # ... and of the matrix-vector kernel that reads rows in long runs, on the two big products of a Llama-3-8B layer
+    # (Q4_K gate/up pair with the norm folded in; Q6_K down projection adding into the residual stream): (what, n_in, n_out)
+    "llama8b-gateup-timeline": ("llama8b", "timeline", 0, ("gateup", 4096, 14336)),
+    "llama8b-down-timeline": ("llama8b", "timeline", 0, ("down", 14336, 4096)),
 }
 # HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
 # WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy: recorded
@@ -123,7 +127,7 @@ TRAFFIC, TRAFFIC_COMMIT = _load_traffic()
 ALSO = ["llama8b-rope-512", "llama8b-kv-store-512", "qwen1.5b-kv-shift-32k", "qwen1.5b-decode-store-32k",
         "qwen1.5b-decode-rope-store-32k", "qwen1.5b-prefill512-d32256", "llama8b-decode-8k",
         "llama8b-prefill512-d4096-timeline", "llama8b-prefill512-d4096-cutoffs", "qwen1.5b-decode-32k-timeline",
-        "qwen1.5b-decode-32k-cutoffs", "weights-read-patterns", "llama8b-logits", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
+        "qwen1.5b-decode-32k-cutoffs", "weights-read-patterns", "llama8b-gateup-timeline", "llama8b-logits", "qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock",
         "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 TARGETS = ["qwen1.5b-decode-layer-32k", "llama8b-decode-layer-8k", "decode-handoff-mock", "hbm-read-32MiB", "hbm-read-64MiB", "llama8b-prefill512-d4096", "qwen1.5b-decode-32k", "qwen7b-decode-32k"]
 ALSO_CPU = {"qwen1.5b-decode-32k"}  # the decode half of the metric gets its CPU baseline in the default run too
@@ -845,6 +849,9 @@ def run_patterns(torch, kernels, name, steps, warmup, with_cpu):
 PREFILL_STAGES = [(0, "entry"), (9, "queries and first K tile requested"), (10, "first V tile and second K tile requested"),
                   (1, "queries in registers"), (2, "first two score tiles"), (3, "first weights"), (4, "main loop done"),
                   (5, "last products done, accumulators in LDS"), (7, "barrier passed"), (8, "output stored")]
+GEMV_STAGES = [(0, "entry"), (1, "first two items of weights requested"), (2, "digits of the wave's part of the activation done"),
+               (3, "item 0 in LDS"), (4, "item 1 in LDS"), (5, "item 2 in LDS"), (6, "item 3 in LDS"), (7, "item 4 in LDS"),
+               (10, "item 7 in LDS"), (13, "tile's sums out"), (14, "exit")]
 DECODE_STAGES = [(0, "entry"), (1, "position known, query pieces met, tile requests issued"), (2, "query converted"),
                  (3, "K arrived, scores of the last tile done"), (4, "V arrived, last products done"), (5, "partials in LDS"),
                  (6, "barrier passed"), (7, "partial written")]
@@ -857,6 +864,8 @@ def run_timeline(torch, kernels, name, steps, warmup, with_cpu):
     import ctypes
 
     shape, _, n_ctx, (what, a, batch) = WORKLOADS[name]
+    if what in ("gateup", "down"):
+        return run_gemv_timeline(torch, kernels, name, steps)
     sh = SHAPES[shape]
     H, G, d = sh["H"], sh["G"], sh["d"]
     L = kernels.stamps_lib()
@@ -916,6 +925,78 @@ def run_timeline(torch, kernels, name, steps, warmup, with_cpu):
                 roofline=dict(bound=bound, achieved=work / (span * 1e-6) / scale_u, peak=peak / scale_u, unit=unit,
                               frac=work / (span * 1e-6) / peak, traffic=None, kernel=kern, launch_us=span,
                               note="launch_us: first wave's entry to last wave's last mark in the timeline build, stamps included"),
+                parity=None, timeline_us=timeline)
+
+
+def run_gemv_timeline(torch, kernels, name, steps):
+    """run_timeline for the matrix-vector kernel: one big product of a decode layer over cold copies of its matrices
+    (random block bytes with sane scales: the kernel's time does not depend on the values)."""
+    import ctypes
+
+    _, _, _, (what, n_in, n_out) = WORKLOADS[name]
+    L = kernels.stamps_lib()
+    rc = L.orin_fa_init(0)
+    assert rc == 0, rc
+    L.orin_fa_set_stream(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    wtype, blk, d_at = (12, 144, 0) if what == "gateup" else (14, 210, 208)   # Q4_K / Q6_K: where a block keeps its fp16 scale
+    n_mat = 2 if what == "gateup" else 1
+    row = n_in // 256 * blk
+    per = n_mat * n_out * row
+    copies = max(3, int(600e6 // per))  # more than the memory-side cache holds
+    g = torch.Generator(device="cuda").manual_seed(77)
+    W = torch.randint(0, 255, (copies, n_mat, n_out * row), dtype=torch.uint8, device="cuda", generator=g)
+    Wb = W.view(copies, n_mat, -1, blk)
+    Wb[..., d_at] = 0x00
+    Wb[..., d_at + 1] = 0x2c
+    if what == "gateup":
+        Wb[..., 2] = 0x00
+        Wb[..., 3] = 0x2c
+    x = torch.randn(n_in, device="cuda", generator=g)
+    nw = torch.ones(n_in, device="cuda")
+    y = torch.zeros(n_out, device="cuda")
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    L.orin_gemv_norm_gate_up_swiglu.argtypes = [ci, vp, vp, vp, vp, ctypes.c_float, vp, ci, ci]
+    L.orin_gemv_multi.argtypes = [ci, ci, vp, vp, vp, vp, vp, vp, ctypes.c_float, ci, ci]
+
+    def launch(c):
+        if what == "gateup":
+            rc = L.orin_gemv_norm_gate_up_swiglu(wtype, W[c, 0].data_ptr(), W[c, 1].data_ptr(), x.data_ptr(), nw.data_ptr(), 1e-5,
+                                                 y.data_ptr(), n_in, n_out)
+        else:
+            ws, ys, ns = (vp * 1)(W[c, 0].data_ptr()), (vp * 1)(y.data_ptr()), (ci * 1)(n_out)
+            rc = L.orin_gemv_multi(wtype, 1, ws, None, ys, ns, x.data_ptr(), None, 0.0, n_in, 1)
+        assert rc == 0, rc
+
+    stages = GEMV_STAGES
+    rows = []
+    host = np.zeros(1024 * 4 * 16, np.int64)
+    for rep_ in range(1 + max(1, min(steps, 5))):
+        n_run = copies - rep_ % 2
+        for c in range(n_run):            # (the earlier ones push the last launch's matrices out of every cache)
+            launch(c)
+            torch.cuda.synchronize()      # (every launch starts on an idle chip: behind another it shares the memory with its tail)
+        rc = L.orin_fa_bench_stamps(2, host.ctypes.data, host.size)
+        assert rc == 0, rc
+        t = host.reshape(1024, 4, 16)[:, :, [slot for slot, _ in stages]].astype(np.float64) * 0.01  # 100 MHz -> us
+        passed = t > 0                    # (a wave with fewer items leaves the later item marks at zero)
+        passed &= passed[:, :, -1:]
+        t0 = t[:, :, 0][passed[:, :, 0]].min()
+        if rep_ > 0:
+            rows.append([(float(np.median(t[:, :, j][passed[:, :, j]] - t0)), float((t[:, :, j][passed[:, :, j]] - t0).min()),
+                          float((t[:, :, j][passed[:, :, j]] - t0).max())) if passed[:, :, j].any() else (0.0, 0.0, 0.0)
+                         for j in range(len(stages))])
+    med = np.median(np.array(rows), axis=0)
+    timeline = {label: dict(median=round(float(m[0]), 2), earliest=round(float(m[1]), 2), latest=round(float(m[2]), 2))
+                for (_, label), m in zip(stages, med) if m[2] > 0}
+    span = float(med[-1][2])
+    del W, Wb
+    torch.cuda.empty_cache()
+    return dict(value=per / (span * 1e-6) / 1e9, unit="GB/s", ms_per_step=span * 1e-3,
+                config=dict(workload=name, what=what, n_in=n_in, n_out=n_out, weights="Q4_K" if wtype == 12 else "Q6_K", bytes=per),
+                roofline=dict(bound="hbm", achieved=per / (span * 1e-6) / 1e9, peak=PEAK_BYTES / 1e9, unit="GB/s",
+                              frac=per / (span * 1e-6) / PEAK_BYTES, traffic=None, kernel="gemv_rows_kernel (timeline build)", launch_us=span,
+                              note="launch_us: first wave's entry to last wave's last mark in the timeline build, stamps included; "
+                                   "one launch on an idle chip, its matrices cold"),
                 parity=None, timeline_us=timeline)
 
 

@@ -57,10 +57,11 @@ int orin_fa_bench_tiny_launch(void);
  * wrong by design and only bench.py's cut-off workloads load them.) */
 
 /* Timeline build only (liborin_fa_stamps.so: the same sources compiled with -DORIN_FA_STAMPS, in which
- * lane 0 of every wave of the prefill kernel and of the decode split kernel stores the 100 MHz wall
- * clock at the end of each stage).  Copies the table of the kernel's last launch to host memory:
- * which = 0 prefill, n <= 1024 workgroups x 4 waves x 16 slots; which = 1 decode split kernel,
- * n <= 1024 x 8 x 16; entry [workgroup][wave][slot], workgroups numbered x + gridDim.x * (y +
+ * lane 0 of every wave of the prefill kernel, of the decode split kernel and of the matrix-vector kernel that
+ * reads rows in long runs stores the 100 MHz wall clock at the end of each stage).  Copies the table of the
+ * kernel's last launch to host memory: which = 0 prefill, n <= 1024 workgroups x 4 waves x 16 slots; which = 1
+ * decode split kernel, n <= 1024 x 8 x 16; which = 2 matrix-vector kernel, n <= 1024 x 4 x 16 (waves 0-3 of a
+ * workgroup); entry [workgroup][wave][slot], workgroups numbered x + gridDim.x * (y +
  * gridDim.y * z); a mark a wave did not pass reads 0.  Clears the table afterwards.  Synchronous.  The ordinary library returns a HIP "not supported" error. */
 int orin_fa_bench_stamps(int which, long long* host, size_t n);
 

@@ -5,10 +5,10 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "liborin_fa.so")
-# The timeline build: the same sources, the two attention kernels compiled with -DORIN_FA_STAMPS so that their
+# The timeline build: the same sources, the two attention kernels and the matrix-vector kernel compiled with -DORIN_FA_STAMPS so that their
 # stage marks store the wall clock.  A measurement aid for bench.py's timeline workloads; never the library that is timed.
 STAMPS_LIB = os.path.join(HERE, "liborin_fa_stamps.so")
-STAMPED = ("fa_prefill.hip", "fa_decode.hip")
+STAMPED = ("fa_prefill.hip", "fa_decode.hip", "gemv_mfma.hip")
 # The cut-off builds: the decode split kernel with parts taken out (-DORIN_FA_DECODE_PROBE=flags, see fa_decode.hip;
 # results wrong by design), one library per flag set, for bench.py's cut-off workload.  Measurement aids.
 PROBE_FLAGS = (1, 3, 7, 15, 31)
@@ -64,7 +64,7 @@ def build(verbose=False):
     objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in SOURCES]
     cmds = [[HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(s), []) + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
     stamped = {s: os.path.join(OBJ_DIR, os.path.basename(s) + ".stamps.o") for s in SOURCES if os.path.basename(s) in STAMPED}
-    cmds += [[HIPCC] + FLAGS + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
+    cmds += [[HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(s), []) + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
     dec = next(s for s in SOURCES if os.path.basename(s) == "fa_decode.hip")
     probes = {f: os.path.join(OBJ_DIR, f"fa_decode.hip.probe{f}.o") for f in PROBE_FLAGS}
     cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_DECODE_PROBE={f}", "-c", dec, "-o", o] for f, o in probes.items()]

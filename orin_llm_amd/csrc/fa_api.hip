@@ -409,8 +409,8 @@ size_t orin_fa_bench_handoff_stream_bytes(void) { return kHandoffStreamBytes; }
 
 int orin_fa_bench_stamps(int which, long long* host, size_t n) {
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
-    if (!host || n == 0 || (which != 0 && which != 1)) return ORIN_FA_E_INVALID;
-    return hip_code(which == 0 ? prefill_stamps(host, n) : decode_stamps(host, n));
+    if (!host || n == 0 || which < 0 || which > 2) return ORIN_FA_E_INVALID;
+    return hip_code(which == 0 ? prefill_stamps(host, n) : which == 1 ? decode_stamps(host, n) : gemv_stamps(host, n));
 }
 
 int orin_fa_bench_tiny_launch(void) {

@@ -108,10 +108,12 @@ constexpr int kStampWgs = 1024, kStampSlots = 16;
         __builtin_amdgcn_sched_barrier(0);                                                                     \
     } while (0)
 #endif
-// Copies a kernel's table to the host (which: 0 prefill, 4 waves a workgroup; 1 decode split, 8 waves);
+// Copies a kernel's table to the host (which: 0 prefill, 4 waves a workgroup; 1 decode split, 8 waves; 2 the
+// matrix-vector kernel, 4 waves);
 // hipErrorNotSupported in the ordinary library.
 hipError_t prefill_stamps(long long* host, size_t n);
 hipError_t decode_stamps(long long* host, size_t n);
+hipError_t gemv_stamps(long long* host, size_t n); // the matrix-vector kernel that reads rows in long runs: waves 0-3 of a workgroup
 constexpr size_t kHandoffScratchBytes = 1u << 20; // partials of both levels and the arrival counters
 constexpr size_t kHandoffStreamBytes = (size_t)256 * 512 * 16 * 16; // 32 MiB read per launch
 hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out, hipStream_t stream);

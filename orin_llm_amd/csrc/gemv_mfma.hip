@@ -32,6 +32,35 @@
 //     through a wave's own LDS buffer, which this machine's memory path serves a quarter faster.  The
 //     kernel described above remains for Q8_0 and for matrices with a ragged last tile.
 #include "layer_common.hpp"
+#include "fa_common.hpp"
+
+// Stage marks of the kernel that reads rows in long runs: wall-clock stamps in the timeline build (waves 0-3 of a
+// workgroup), nothing otherwise (fa_common.hpp).  ROWS_ITEM_STAMP marks an item's arrival in LDS and waits for the
+// LDS writes first, in that build only.
+#ifdef ORIN_FA_STAMPS
+namespace orin_fa {
+__device__ long long g_gemv_stamps[kStampWgs * 4 * kStampSlots];
+}
+// (its own store, all conditions in one test: wrapped around the attention kernels' macro the marks cost this kernel a
+// quarter of its time)
+#define ROWS_STAMP(i)                                                                                                      \
+    do {                                                                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                                 \
+        const unsigned wg_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);                               \
+        if ((threadIdx.x & 63) == 0 && threadIdx.x < 256 && wg_ < (unsigned)orin_fa::kStampWgs && (i) < orin_fa::kStampSlots) \
+            orin_fa::g_gemv_stamps[(wg_ * 4 + (threadIdx.x >> 6)) * orin_fa::kStampSlots + (i)] =                          \
+                (long long)__builtin_amdgcn_s_memrealtime();                                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    } while (0)
+#define ROWS_ITEM_STAMP(i)                                  \
+    do {                                                    \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); \
+        ROWS_STAMP(i);                                      \
+    } while (0)
+#else
+#define ROWS_STAMP(i)
+#define ROWS_ITEM_STAMP(i)
+#endif
 
 #include <stdlib.h>
 
@@ -599,6 +628,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     using G = RowsGeom<T, CB>;
     constexpr int M = DUAL ? 2 : 1, P = G::P, R = G::R, NL = G::NL;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    ROWS_STAMP(0);
     const GemvSeg seg = a.seg[blockIdx.y];
     {
         // Every argument word the kernel reads, asked for here in one batch: left to the compiler the scalar loads
@@ -692,7 +722,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         constexpr int kPasses = (CB * 256 + 511) / 512; // 512 elements a pass
         // The wave's first kPre chunks are fetched ahead of the weight requests: loads return in order, so fetched
         // behind them a chunk's few floats wait for two items of weights, and the wave's first item for all its
-        // digits (stamps in a development build: first digits 1.4 us after the requests, the second chunk's 2.1 us
+        // digits (the stage marks below, read in the timeline build: first digits 1.4 us after the requests, the second chunk's 2.1 us
         // later, the first item 0.5 us after that).
         constexpr int kPre = kWaves == 8 ? 2 : 4; // (eight-wave workgroups: fewer chunks a wave, and registers for four waves a SIMD)
         float xs[kPre][kPasses][8], gs[kPre][kPasses][8]; // (read under the conditions they are loaded under)
@@ -713,6 +743,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         for (int j = 0; j < kRing; ++j)
             if (j < total) request(buf[j], bias_v[j], j % M);
         __builtin_amdgcn_sched_barrier(0);
+        ROWS_STAMP(1);
 #pragma unroll
         for (int i = 0; i < kPre; ++i) {
             const int ch = wave + i * kWaves, end = min((ch + 1) * CB * 256, n_in);
@@ -735,6 +766,8 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         ss = wave_sum(ss);
         if (lane == 0) wave_ss[wave] = ss;
     }
+    ROWS_STAMP(2);
+    [[maybe_unused]] int n_consumed = 0;
     const bool has_norm = a.norm_w != nullptr;
     const float norm_n = (float)n_in, norm_eps = a.eps;
 
@@ -772,6 +805,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
             if (gridDim.z > 1 || a.accumulate) atomicAdd(seg.y + r, y); // (one writer a row and share: with one share the sum is the plain one)
             else seg.y[r] = y;
         }
+        ROWS_STAMP(13);
     };
     if (my_chunks == 0) { // (fewer chunks than waves: this wave only keeps the barriers' count)
         const float zero[M] = {};
@@ -783,6 +817,8 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     auto consume = [&](const u32x4 (&r)[NL], float bias, int m) {
 #pragma unroll
         for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(transit + loff[i]) = r[i];
+        ROWS_ITEM_STAMP(3 + n_consumed);
+        ++n_consumed;
         const int cb = min(CB, nb - cs_c * CB);
         // (unrolled over CB with a test per block, not a loop over cb: every LDS offset is a constant of its instruction)
         float v = F::from_lds(transit + c.n * R * 16, c, addr, cs_c * CB);
@@ -816,6 +852,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     if (k + 2 < total) request(buf[0], bias_v[0], 0);
     if (k + 1 < total) consume(buf[1], bias_v[1], M - 1);
     if (k + 2 < total) consume(buf[0], bias_v[0], 0);
+    ROWS_STAMP(14);
 }
 
 template <int T, bool DUAL, int kWaves, int CB>
@@ -1040,6 +1077,20 @@ hipError_t gemv_mfma_allow_lds() {
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax)) != hipSuccess) return e;
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_mixed_kernel<4>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+}
+
+hipError_t gemv_stamps(long long* host, size_t n) {
+#ifdef ORIN_FA_STAMPS
+    if (n > (size_t)kStampWgs * 4 * kStampSlots) return hipErrorInvalidValue;
+    hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(g_gemv_stamps), n * sizeof(long long)); // (synchronises with the device)
+    void* dev = nullptr;
+    if (e == hipSuccess) e = hipGetSymbolAddress(&dev, HIP_SYMBOL(g_gemv_stamps));
+    if (e == hipSuccess) e = hipMemset(dev, 0, sizeof(g_gemv_stamps)); // the next launch starts from an empty table
+    return e;
+#else
+    (void)host; (void)n;
+    return hipErrorNotSupported;
+#endif
 }
 
 } // namespace orin_fa
