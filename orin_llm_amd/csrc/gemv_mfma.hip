@@ -621,7 +621,7 @@ struct RowsGeom {
     }
 };
 
-template <int T, bool DUAL, int kWaves, int CB>
+template <int T, bool DUAL, int kWaves, int CB, bool kShortPrologue = false>
 __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     using F = MF<T>;
     using L = Lds<F::kGroup>;
@@ -726,6 +726,33 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
         // later, the first item 0.5 us after that).
         constexpr int kPre = kWaves == 8 ? 2 : 4; // (eight-wave workgroups: fewer chunks a wave, and registers for four waves a SIMD)
         float xs[kPre][kPasses][8], gs[kPre][kPasses][8]; // (read under the conditions they are loaded under)
+        if (kShortPrologue && kPasses == 1 && total >= kRing && my_chunks <= 2) {
+            // One or two chunks and at least two items: nothing between the loads and their uses is under a
+            // condition (a second chunk the wave does not have is fetched from the row's end and dropped), so the
+            // compiler's waits are exact: the digits wait for the activation, not for the weights behind it, and
+            // the first item is used as soon as it is there.  Only in the kernel for launches that leave resident places empty
+            // (Qwen2.5-1.5B's gate/up 8.1 -> 7.4 us, its down projection 7.25 -> 6.9): a launch that fills the chip
+            // runs 1.5 us longer this way, its second round of requests getting in the way of the first.  Not in
+            // the kernels of eight waves and of mixed types either.
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int e = min((wave + i * kWaves) * CB * 256 + lane * 8, n_in - 8);
+                fetch(ax, e, xs[i][0]);
+                fetch(aw ? aw : ax, e, gs[i][0]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < kRing; ++j) request(buf[j], bias_v[j], j % M);
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                const int e = wave * CB * 256 + lane * 8;
+                if (e < min((wave + 1) * CB * 256, n_in)) digits(xs[0][0], gs[0][0], e);
+            }
+            if (my_chunks == 2) {
+                const int e = (wave + kWaves) * CB * 256 + lane * 8;
+                if (e < min((wave + kWaves + 1) * CB * 256, n_in)) digits(xs[1][0], gs[1][0], e);
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < kPre; ++i) {
             const int ch = wave + i * kWaves, end = min((ch + 1) * CB * 256, n_in);
@@ -761,6 +788,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
                 if (aw) fetch(aw, e, g);
                 digits(x, g, e);
             }
+        }
         }
         if (lane < 4) reinterpret_cast<unsigned*>(smem + L::zero_off(n_in))[lane] = 0u; // (every wave writes the same zeros)
         ss = wave_sum(ss);
@@ -855,9 +883,11 @@ __device__ __forceinline__ void gemv_rows_body(const GemvArgs& a) {
     ROWS_STAMP(14);
 }
 
-template <int T, bool DUAL, int kWaves, int CB>
+// kShortPrologue: the kernel for launches that leave resident places empty (see the body's prologue): a kernel of
+// its own, because the second path's code alone costs the launches that do not take it a microsecond.
+template <int T, bool DUAL, int kWaves, int CB, bool kShortPrologue = false>
 __global__ __launch_bounds__(kWaves * 64) void gemv_rows_kernel(const GemvArgs a) {
-    gemv_rows_body<T, DUAL, kWaves, CB>(a);
+    gemv_rows_body<T, DUAL, kWaves, CB, kShortPrologue>(a);
 }
 
 // Matrices of different block types in one launch (the q, k, v projections of a file that keeps attn_v in
@@ -899,6 +929,8 @@ int rows_wgs_per_cu(int given) {
     return env ? given : 3;
 }
 
+int g_rows_resident = 768; // workgroups of four waves the chip holds at once (three a CU; set by the launcher)
+
 template <int T, bool DUAL, int kWaves, int CB>
 bool launch_rows_as(const GemvArgs& a, dim3 grid, int n_in_wg, hipStream_t stream) {
     const size_t lds = RowsGeom<T, CB>::lds_bytes(n_in_wg, kWaves);
@@ -906,6 +938,14 @@ bool launch_rows_as(const GemvArgs& a, dim3 grid, int n_in_wg, hipStream_t strea
     GemvArgs b = a;
     b.share_blocks = (a.n_in / 256) / (int)grid.z;
     b.share_extra = (a.n_in / 256) % (int)grid.z;
+    // (... and gives a wave one or two chunks: the other kernel's prologue serves more)
+    b.few_workgroups = kWaves == 4 && (int)(grid.x * grid.y * grid.z) <= g_rows_resident * 3 / 4 && (n_in_wg / 256 + CB - 1) / CB <= 2 * kWaves;
+    if constexpr (kWaves == 4) {
+        if (b.few_workgroups) {
+            hipLaunchKernelGGL((gemv_rows_kernel<T, DUAL, kWaves, CB, true>), grid, dim3(kWaves * 64), lds, stream, b);
+            return true;
+        }
+    }
     hipLaunchKernelGGL((gemv_rows_kernel<T, DUAL, kWaves, CB>), grid, dim3(kWaves * 64), lds, stream, b);
     return true;
 }
@@ -948,6 +988,7 @@ hipError_t launch(const GemvArgs& a, int cu_count, hipStream_t stream) {
     const bool wide = ks == 1 && nb_row >= 16 && !a.w_up && (int)grid.x == (max_out + 15) / 16;
     if constexpr (T == kQ4_K || T == kQ5_K || T == kQ6_K) {
         const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu);
+        g_rows_resident = cu_count * 3;
         dim3 gr = g3;
         gr.x = min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16);
         // (its LDS buffers let three workgroups of four waves share a CU: no more shares of a row than are resident at once)
@@ -982,6 +1023,11 @@ hipError_t allow() {
 
 template <int T, bool DUAL, int kWaves, int CB>
 hipError_t allow_rows() {
+    if constexpr (kWaves == 4) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_kernel<T, DUAL, kWaves, CB, true>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
+        if (e != hipSuccess) return e;
+    }
     return hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_rows_kernel<T, DUAL, kWaves, CB>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaLdsMax);
 }
@@ -1010,6 +1056,7 @@ hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) 
     for (int i = 0; i < a.n_seg; ++i) rows = rows && a.seg[i].n_out % 16 == 0 && a.seg[i].type != kQ8_0;
     a.share_blocks = a.n_in / 256; // (one share: whole rows)
     a.share_extra = 0;
+    a.few_workgroups = 0;
     if (rows) {
         const int per_cu = rows_wgs_per_cu(a.mfma_wgs_per_cu), nb = a.n_in / 256;
         const dim3 gr(min((max_out + 15) / 16, per_cu > 0 ? cu_count * per_cu : (max_out + 15) / 16), a.n_seg);

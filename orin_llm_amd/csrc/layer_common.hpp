@@ -34,6 +34,7 @@ struct GemvArgs {
     size_t row_bytes;
     int team_waves, wgs_per_cu, mfma_wgs_per_cu, n_seg_types, k_split_override;
     int share_blocks, share_extra; // blocks of a row per share of it (gridDim.z shares), and how many shares take one more
+    int few_workgroups;            // not 0: the launch leaves resident places empty (see gemv_rows_body's prologue)
 };
 
 size_t weight_row_bytes(int type, int n); // 0: unknown type or n not a whole number of blocks
