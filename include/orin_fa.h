@@ -180,6 +180,11 @@ int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx);
 int orin_fa_cu_count(void);
 
+/* What llm::cuda::device_info prints (reference: src/kernels.h:9, src/kernels.cu:1739-1744): the name of a
+ * device (NUL-terminated, cut to name_bytes), its compute units and its memory in bytes.  Any of the three
+ * outputs may be NULL.  Needs no orin_fa_init. */
+int orin_fa_device_info(int device, char* name, size_t name_bytes, int* cu_count, size_t* total_mem);
+
 /* Human-readable name of a return code. */
 const char* orin_fa_error_string(int code);
 

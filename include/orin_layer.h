@@ -12,7 +12,9 @@
  * 14 Q6_K), a matrix is n_out rows of n_in elements, rows packed back to back.
  * Limits: n_in a multiple of 32 (256 for the K types), at most 24576; matrices of type F32, F16,
  * Q4_K, Q5_K 16-byte aligned (2 bytes for Q8_0 and Q6_K, whose blocks are 34 and 210 bytes);
- * activations and outputs 16-byte aligned.  ORIN_FA_E_INVALID otherwise.
+ * activations and norm weights 16-byte aligned; outputs and biases plain float arrays (4-byte aligned).
+ * ORIN_FA_E_INVALID otherwise.  orin_decode_layer checks all seven of its matrices against these limits
+ * before its first launch.
  *
  * Arithmetic: the reference's GPU operators round the activation to int8 in blocks of 32 before a
  * product (quantize_activation + dp4a).  These keep it at fp32 precision (as fp32, or as three int8
@@ -44,16 +46,20 @@ int orin_rms_norm_rows(const float* x, const float* w, int rows, int cols, float
 
 /* Replaces llm::cuda::quantize_activation (reference: src/kernels.h:15, src/kernels.cu:136-157, 1778-1784).
  * The reference stores an int8 copy of x for the *_q8 products that follow; this stores an fp32
- * copy (n_in <= 32768) in the library's own device memory, so that those products see x as it
- * was at this call, as they do in the reference. */
+ * copy (n_in <= 32768; the products themselves take rows of at most 24576) in the library's own device
+ * memory, so that those products see x as it was at this call, as they do in the reference. */
 int orin_quantize_activation(const float* x, int n_in);
 
 /* Replace llm::cuda::gemv_q8 / gemv_q8_bias / gemv_q8_add (reference: src/kernels.h:21-27,
  * src/kernels.cu:1786-1806, 1825-1836): y = W xs, y = W xs + bias, y += W xs, with xs the activation of the
- * last orin_quantize_activation call (whose n_in must equal this n_in).  The accumulating form may add a row's sum
- * to y in several shares with atomic adds (long rows of a matrix with few rows): y must be written by nothing else
- * while the launch runs, and the order in which a row's shares are added is not fixed (the last bits of y may
- * differ from run to run; with one share the result is the plain sum). */
+ * last orin_quantize_activation call, of which a product over n_in elements reads the first n_in (as the
+ * reference's do: its decode_layer stages n_embd elements of the attention output and multiplies by wo, whose
+ * rows have n_head * head_dim, src/model_gpu.cu:284-285); a product longer than what was staged is refused.
+ * The accumulating form may add a row's sum to y in several shares with atomic adds (long rows of a matrix with
+ * few rows): y must be written by nothing else while the launch runs, and the order in which a row's shares are
+ * added is not fixed, so the last bits of y may differ from run to run and between replays of one graph (the
+ * reference's gemv_q8_add is a plain sum, src/kernels.cu:350-374).  orin_gemv_row_shares(1) switches the shares
+ * off: y is then bit for bit the same on every run. */
 int orin_gemv_q8(int type, const void* W, float* y, int n_in, int n_out);
 int orin_gemv_q8_bias(int type, const void* W, const float* bias, float* y, int n_in, int n_out);
 int orin_gemv_q8_add(int type, const void* W, float* y, int n_in, int n_out);
@@ -80,6 +86,14 @@ int orin_swiglu(float* act, const float* gate, const float* up, int n);
  * blocks' scales applied in fp32) and on the vector ALU otherwise, as F16 and F32 always do.  on = 0 keeps
  * everything on the vector ALU: for comparisons and tests; the results agree to the order of an fp32 sum. */
 void orin_gemv_use_matrix_cores(int on);
+
+/* How many shares an accumulating projection (y += W x: orin_gemv_q8_add, orin_gemv_multi with accumulate,
+ * the output and down projections of orin_decode_layer) may cut a row into: 0 (default) = the launcher
+ * chooses 1, 2 or 4 by shape, which is fastest and leaves the order of a row's adds open (see orin_gemv_q8_add);
+ * 1 = never cut, every result bit for bit reproducible, at 1-2 us more per projection on small models; 2, 4 = forced
+ * (tuning).  Takes effect with the next launch; graphs captured earlier keep the launches they recorded.
+ * ORIN_GEMV_KSPLIT in the environment sets the initial value. */
+void orin_gemv_row_shares(int shares);
 
 /* ---- forms with no counterpart in the reference: fewer launches per layer ---- */
 
@@ -108,6 +122,9 @@ int orin_gemv_norm_gate_up_swiglu(int type, const void* Wg, const void* Wu, cons
  * not take (NeoX pairing with n_rot < head_dim) goes through the separate rope and store calls.
  * x is updated in place; q, k, v, attn, act (and up_tmp, needed only when ffn_gate and ffn_up
  * differ in type) are scratch the caller provides; k and v leave un-rotated / as projected.
+ * The two projections that add into x may cut their rows into shares that meet by atomic adds, so x can differ
+ * in its last bits between runs and between replays of a captured layer unless orin_gemv_row_shares(1) was
+ * called before the launches (or the capture).
  * A descriptor with a missing pointer or a non-positive size returns ORIN_FA_E_INVALID before
  * anything is launched; shapes a kernel cannot take are refused by the launch that meets them. */
 typedef struct orin_decode_layer_desc {

@@ -1,6 +1,6 @@
 // The decode layer's slice of the orin_llm operator API -- attention, KV cache, rotary embedding, and the norms
 // and quantised matrix-vector products around them -- with the reference's own signatures (reference:
-// src/kernels.h:8-10, :15-47, :55-62, :66-73 and :77-81), implemented for MI355X by liborin_fa.so.  An engine
+// src/kernels.h:8-12, :15-47, :55-62, :66-73 and :77-81), implemented for MI355X by liborin_fa.so.  An engine
 // built against the reference header links these symbols unchanged; each forwards to the C ABI in
 // include/orin_fa.h and include/orin_layer.h and, like the reference's CUDA_CHECK (src/common.h:14-22), prints
 // and abort()s on failure.
@@ -34,7 +34,14 @@ namespace llm::cuda {
 // build the shim with -DORIN_FA_SHIM_NO_PLUMBING and call orin_fa_init /
 // orin_fa_set_stream from the engine's init / set_stream.
 int init();
+void device_info();
 void set_stream(void* stream);
+// The engine carves one block of device memory for the operator layer out of its activation allocation
+// (reference: src/model_gpu.cu:175, 208).  Here that block holds the partial results of the attention
+// kernels' KV splits (orin_fa_workspace_bytes(), whatever max_in and max_batch are); the staged activation
+// of quantize_activation lives in the library's own device data.
+size_t scratch_size(int max_in, int max_batch);
+void scratch_assign(void* base, int max_in, int max_batch);
 #endif
 
 void quantize_activation(const float* x, int n_in);

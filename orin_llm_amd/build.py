@@ -1,4 +1,5 @@
-"""Builds liborin_fa.so (HIP kernels + C ABI + llm::cuda shim) for gfx950, in-tree."""
+"""Builds liborin_fa.so (HIP kernels + C ABI + llm::cuda shim) for gfx950, in-tree, and beside it the two
+measurement-aid libraries that bench.py and one GPU test load (liborin_fa_stamps.so, liborin_fa_bench.so)."""
 import os
 import subprocess
 from concurrent.futures import ThreadPoolExecutor
@@ -8,9 +9,13 @@ LIB = os.path.join(HERE, "liborin_fa.so")
 # The timeline build: the same sources, the two attention kernels and the matrix-vector kernel compiled with -DORIN_FA_STAMPS so that their
 # stage marks store the wall clock.  A measurement aid for bench.py's timeline workloads; never the library that is timed.
 STAMPS_LIB = os.path.join(HERE, "liborin_fa_stamps.so")
-STAMPED = ("fa_prefill.hip", "fa_decode.hip", "gemv_mfma.hip")
+STAMPED = ("fa_prefill.hip", "fa_decode.hip", "gemv_mfma.hip", "fa_api.hip")
+# Read-only stand-ins and a do-nothing kernel (csrc/bench_aids.hip), a library of their own: the product exports none of them.
+BENCH_LIB = os.path.join(HERE, "liborin_fa_bench.so")
+BENCH_SOURCE = os.path.join(HERE, "csrc", "bench_aids.hip")
 # The cut-off builds: the decode split kernel with parts taken out (-DORIN_FA_DECODE_PROBE=flags, see fa_decode.hip;
-# results wrong by design), one library per flag set, for bench.py's cut-off workload.  Measurement aids.
+# results wrong by design), one library per flag set, for bench.py's cut-off workloads.  Measurement aids, built
+# only on request: build(probes=True), `python -m orin_llm_amd.build --probes`, or the cut-off workloads themselves.
 PROBE_FLAGS = (1, 3, 7, 15, 31)
 PROBE_LIB = os.path.join(HERE, "liborin_fa_probe_{}.so")
 # ... and of the prefill kernel (-DORIN_FA_PREFILL_PROBE=flags, see fa_prefill.hip)
@@ -18,7 +23,7 @@ PPROBE_FLAGS = (1, 2, 4, 7, 8, 16)
 PPROBE_LIB = os.path.join(HERE, "liborin_fa_pprobe_{}.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)
-           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "bench_aids.hip", "gemv.hip", "gemv_mfma.hip", "layer_ops.hip",
+           for n in ("fa_prefill.hip", "fa_decode.hip", "kv_cache.hip", "rope.hip", "gemv.hip", "gemv_mfma.hip", "layer_ops.hip",
                      "layer_api.hip", "fa_api.hip", "llm_cuda_shim.cpp")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -57,25 +62,30 @@ def _run(cmd):
     return " ".join(cmd)
 
 
-def build(verbose=False):
-    """Compiles every source (in parallel) and links the shared library.  Always recompiles."""
+def build(verbose=False, probes=False):
+    """Compiles every source (in parallel) and links the shared library and its timeline build.  Always recompiles.
+    probes=True also builds the eleven cut-off libraries (measurement aids whose results are wrong by design)."""
     check_toolchain()
     os.makedirs(OBJ_DIR, exist_ok=True)
     objs = [os.path.join(OBJ_DIR, os.path.basename(s) + ".o") for s in SOURCES]
     cmds = [[HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(s), []) + ["-c", s, "-o", o] for s, o in zip(SOURCES, objs)]
     stamped = {s: os.path.join(OBJ_DIR, os.path.basename(s) + ".stamps.o") for s in SOURCES if os.path.basename(s) in STAMPED}
     cmds += [[HIPCC] + FLAGS + EXTRA_FLAGS.get(os.path.basename(s), []) + ["-DORIN_FA_STAMPS", "-c", s, "-o", o] for s, o in stamped.items()]
+    bench_obj = os.path.join(OBJ_DIR, "bench_aids.hip.o")
+    cmds.append([HIPCC] + FLAGS + ["-c", BENCH_SOURCE, "-o", bench_obj])
     dec = next(s for s in SOURCES if os.path.basename(s) == "fa_decode.hip")
-    probes = {f: os.path.join(OBJ_DIR, f"fa_decode.hip.probe{f}.o") for f in PROBE_FLAGS}
+    want_probes = bool(probes)
+    probes = {f: os.path.join(OBJ_DIR, f"fa_decode.hip.probe{f}.o") for f in (PROBE_FLAGS if want_probes else ())}
     cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_DECODE_PROBE={f}", "-c", dec, "-o", o] for f, o in probes.items()]
     pre = next(s for s in SOURCES if os.path.basename(s) == "fa_prefill.hip")
-    pprobes = {f: os.path.join(OBJ_DIR, f"fa_prefill.hip.probe{f}.o") for f in PPROBE_FLAGS}
+    pprobes = {f: os.path.join(OBJ_DIR, f"fa_prefill.hip.probe{f}.o") for f in (PPROBE_FLAGS if want_probes else ())}
     cmds += [[HIPCC] + FLAGS + [f"-DORIN_FA_PREFILL_PROBE={f}", "-c", pre, "-o", o] for f, o in pprobes.items()]
     with ThreadPoolExecutor(max_workers=8) as pool:
         lines = list(pool.map(_run, cmds))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB]))
     lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [stamped.get(s, o) for s, o in zip(SOURCES, objs)]
                       + ["-o", STAMPS_LIB]))
+    lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", bench_obj, "-o", BENCH_LIB]))
     for f, o in probes.items():
         lines.append(_run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [o if s == dec else x for s, x in zip(SOURCES, objs)]
                           + ["-o", PROBE_LIB.format(f)]))
@@ -87,5 +97,11 @@ def build(verbose=False):
     return LIB
 
 
+def probes_built():
+    return all(os.path.exists(PROBE_LIB.format(f)) for f in PROBE_FLAGS) and all(os.path.exists(PPROBE_LIB.format(f)) for f in PPROBE_FLAGS)
+
+
 if __name__ == "__main__":
-    print(build(verbose=True))
+    import sys
+
+    print(build(verbose=True, probes="--probes" in sys.argv[1:]))

@@ -1,9 +1,15 @@
-// Measurement aids of liborin_fa.so: kernels that are not part of the attention path but give
-// the yardsticks its figures are read against.  Declared in include/orin_fa_bench.h.
+// Measurement aids, built into a library of their own (liborin_fa_bench.so, independent of liborin_fa.so):
+// kernels that are not part of the attention path but give the yardsticks its figures are read against.
+// C ABI in include/orin_fa_bench.h; every call names its stream and its buffers.
 #include "fa_common.hpp"
+
+#include "../../include/orin_fa_bench.h"
 
 namespace orin_fa {
 namespace {
+
+constexpr size_t kHandoffScratchBytes = 1u << 20; // partials of both levels and the arrival counters
+constexpr size_t kHandoffStreamBytes = (size_t)256 * 512 * 16 * 16; // 32 MiB read per launch
 
 // Plain streaming read: every thread issues PER 16-byte loads with the streaming hint (the
 // decode kernel's kind of load), a grid stride apart, and folds them into a word that is
@@ -186,8 +192,6 @@ __global__ __launch_bounds__(256) void read_pattern_kernel(const unsigned char* 
     if (acc == 0x9E3779B9u) *sink = acc;
 }
 
-} // namespace
-
 hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream) {
     const size_t n16 = bytes / 16;
     const int per = loads_per_thread <= 2 ? 2 : loads_per_thread <= 4 ? 4 : loads_per_thread <= 8 ? 8 : 16;
@@ -251,4 +255,37 @@ hipError_t read_pattern_launch(const void* w, size_t mat_bytes, int n_rows, int 
     return hipGetLastError();
 }
 
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
 } // namespace orin_fa
+
+using namespace orin_fa;
+
+extern "C" {
+
+int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, void* stream) {
+    if (!src || !sink || !aligned16(src)) return -1;
+    return -(int)hbm_read_launch(src, bytes, loads_per_thread, sink, static_cast<hipStream_t>(stream));
+}
+
+int orin_fa_bench_read_pattern(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups,
+                               unsigned* sink, void* stream) {
+    if (!w || !sink || !aligned16(w) || mat_bytes < (size_t)n_rows * n_blocks * 144 || (mat_bytes & 15u)) return -1;
+    return -(int)read_pattern_launch(w, mat_bytes, n_rows, n_blocks, pattern, workgroups, sink, static_cast<hipStream_t>(stream));
+}
+
+int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out, void* stream) {
+    if (!src || !scratch || !out || !aligned16(src) || !aligned16(scratch) || !aligned16(out)) return -1;
+    return -(int)handoff_launch(src, fused, scratch, out, static_cast<hipStream_t>(stream));
+}
+
+size_t orin_fa_bench_handoff_scratch_bytes(void) { return kHandoffScratchBytes; }
+size_t orin_fa_bench_handoff_stream_bytes(void) { return kHandoffStreamBytes; }
+
+int orin_fa_bench_tiny_launch(const unsigned* src, unsigned* sink, void* stream) {
+    if (!src || !sink) return -1;
+    return -(int)tiny_launch(src, sink, static_cast<hipStream_t>(stream));
+}
+
+} // extern "C"

@@ -10,7 +10,9 @@
 #include <stdio.h>
 
 #include "../../include/orin_fa.h"
+#ifdef ORIN_FA_STAMPS
 #include "../../include/orin_fa_bench.h"
+#endif
 
 namespace orin_fa {
 namespace {
@@ -202,13 +204,13 @@ struct RopeArgs {
 };
 // partials: null = the active workspace; else a block of kStaticScratchBytes (the static scratch)
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
-                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
+                int head_dim, int n_ctx, const int* d_pos, float scale,
                 const float* k_new, const float* v_new, const RopeArgs* rope = nullptr, void* partials = nullptr);
 }
 
 int orin_fa_decode_ind(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                        int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
-    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr);
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr);
 }
 
 int orin_fa_decode_ind_static(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
@@ -216,7 +218,7 @@ int orin_fa_decode_ind_static(const float* q, const uint16_t* kc, const uint16_t
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
     void* const block = g_state.static_ws[g_state.device]; // looked up in orin_fa_init; never the array's name
     if (!block) return ORIN_FA_E_NOT_INIT;
-    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr, nullptr, block);
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, nullptr, nullptr, block);
 }
 
 size_t orin_fa_static_scratch_bytes(void) { return kStaticScratchBytes; }
@@ -225,7 +227,7 @@ int orin_fa_decode_store_ind(const float* q, const float* k_new, const float* v_
                              float* out, int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale) {
     if (!k_new || !v_new) return ORIN_FA_E_INVALID;
     if (((reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15u) != 0) return ORIN_FA_E_INVALID;
-    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, k_new, v_new);
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, k_new, v_new);
 }
 
 int orin_fa_rope_angles_ind(float* angles, int n_rot, float theta, const float* freq_factors, const int* d_pos) {
@@ -246,34 +248,13 @@ int orin_fa_decode_rope_store_ind(const float* q, const float* k_new, const floa
     // "neox" when the rotation spans the whole head
     if (neox && n_rot != 0 && n_rot != head_dim) return ORIN_FA_E_INVALID;
     const RopeArgs rope{n_rot, theta, freq_factors, neox != 0, angles};
-    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, nullptr, k_new, v_new,
+    return decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, k_new, v_new,
                        n_rot > 0 ? &rope : nullptr);
-}
-
-int orin_fa_decode_ind_timed(const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
-                             int n_head, int n_kv, int head_dim, int n_ctx, const int* d_pos, float scale,
-                             float* us_split, float* us_combine) {
-    static hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
-    hipError_t e = hipSuccess;
-    for (int i = 0; i < 3 && e == hipSuccess; ++i)
-        if (!ev[i]) e = hipEventCreate(&ev[i]);
-    if (e != hipSuccess) return hip_code(e);
-    if ((e = hipEventRecord(ev[0], g_state.stream)) != hipSuccess) return hip_code(e);
-    const int rc = decode_impl(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale, ev[1], nullptr, nullptr);
-    if (rc != ORIN_FA_OK) return rc;
-    if ((e = hipEventRecord(ev[2], g_state.stream)) != hipSuccess) return hip_code(e);
-    if ((e = hipEventSynchronize(ev[2])) != hipSuccess) return hip_code(e);
-    float ms_split = 0.0f, ms_combine = 0.0f;
-    if ((e = hipEventElapsedTime(&ms_split, ev[0], ev[1])) != hipSuccess) return hip_code(e);
-    if ((e = hipEventElapsedTime(&ms_combine, ev[1], ev[2])) != hipSuccess) return hip_code(e);
-    if (us_split) *us_split = ms_split * 1e3f;
-    if (us_combine) *us_combine = ms_combine * 1e3f;
-    return ORIN_FA_OK;
 }
 
 namespace {
 int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int n_head, int n_kv,
-                int head_dim, int n_ctx, const int* d_pos, float scale, hipEvent_t mid,
+                int head_dim, int n_ctx, const int* d_pos, float scale,
                 const float* k_new, const float* v_new, const RopeArgs* rope, void* partials) {
     int rc = check_common(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx);
     if (rc != ORIN_FA_OK) return rc;
@@ -305,7 +286,7 @@ int decode_impl(const float* q, const uint16_t* kc, const uint16_t* vc, float* o
         a.part_ml = a.part_o + (size_t)a.n_splits * n_head * head_dim;
     }
     set_scale(a, scale);
-    return hip_code(decode_launch(a, head_dim, g_state.stream, mid));
+    return hip_code(decode_launch(a, head_dim, g_state.stream));
 }
 } // namespace
 
@@ -380,45 +361,14 @@ int orin_fa_rope_store_batch(float* q, float* k, const float* v, uint16_t* kc, u
     return hip_code(kv_store_launch(kc, vc, k, v, n_kv, head_dim, n_ctx, n_past, batch, nullptr, g_state.stream));
 }
 
-// ---- measurement aids (include/orin_fa_bench.h) ----
-int orin_fa_bench_hbm_read(const void* src, size_t bytes, int loads_per_thread) {
-    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
-    if (!src || (reinterpret_cast<uintptr_t>(src) & 15u)) return ORIN_FA_E_INVALID;
-    // (the word that is never written lives in the library's own workspace block)
-    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
-    return hip_code(hbm_read_launch(src, bytes, loads_per_thread, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
-}
-
-int orin_fa_bench_read_pattern(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups) {
-    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
-    if (!w || (reinterpret_cast<uintptr_t>(w) & 15u) || mat_bytes < (size_t)n_rows * n_blocks * 144 || (mat_bytes & 15u)) return ORIN_FA_E_INVALID;
-    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
-    return hip_code(read_pattern_launch(w, mat_bytes, n_rows, n_blocks, pattern, workgroups, static_cast<unsigned*>(g_state.own_ws), g_state.stream));
-}
-
-int orin_fa_bench_handoff(const void* src, int fused, void* scratch, float* out) {
-    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
-    if (!src || !scratch || !out) return ORIN_FA_E_INVALID;
-    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(scratch) | reinterpret_cast<uintptr_t>(out)) & 15u)
-        return ORIN_FA_E_INVALID;
-    return hip_code(handoff_launch(src, fused, scratch, out, g_state.stream));
-}
-
-size_t orin_fa_bench_handoff_scratch_bytes(void) { return kHandoffScratchBytes; }
-size_t orin_fa_bench_handoff_stream_bytes(void) { return kHandoffStreamBytes; }
-
+#ifdef ORIN_FA_STAMPS
+// Timeline build only (include/orin_fa_bench.h): the stage-mark tables of the kernels' last launches.
 int orin_fa_bench_stamps(int which, long long* host, size_t n) {
     if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
     if (!host || n == 0 || which < 0 || which > 2) return ORIN_FA_E_INVALID;
     return hip_code(which == 0 ? prefill_stamps(host, n) : which == 1 ? decode_stamps(host, n) : gemv_stamps(host, n));
 }
-
-int orin_fa_bench_tiny_launch(void) {
-    if (!g_state.ready) return ORIN_FA_E_NOT_INIT;
-    if (!g_state.own_ws) return ORIN_FA_E_WORKSPACE;
-    unsigned* const w = static_cast<unsigned*>(g_state.own_ws);
-    return hip_code(tiny_launch(w, w + 64, g_state.stream));
-}
+#endif
 
 int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
     if (n_head <= 0 || n_kv <= 0 || n_ctx <= 0 || n_head % n_kv != 0) return 0;
@@ -427,6 +377,16 @@ int orin_fa_decode_splits(int n_head, int n_kv, int head_dim, int n_ctx) {
 }
 
 int orin_fa_cu_count(void) { return g_state.cu_count; }
+
+int orin_fa_device_info(int device, char* name, size_t name_bytes, int* cu_count, size_t* total_mem) {
+    hipDeviceProp_t prop;
+    const hipError_t e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_code(e);
+    if (name && name_bytes > 0) snprintf(name, name_bytes, "%s", prop.name);
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (total_mem) *total_mem = prop.totalGlobalMem;
+    return ORIN_FA_OK;
+}
 
 const char* orin_fa_error_string(int code) {
     switch (code) {

@@ -59,12 +59,17 @@ struct FaArgs {
     float qsign;       // sign of scale, folded into Q
 };
 
+// hipGetLastError() returns, and clears, the last error of any HIP call this host thread has made, the host
+// application's own included.  Every launcher below starts by dropping what is pending, so that the code it
+// returns after its launch is the launch's own and an unrelated stale error is not blamed on (and, through the
+// llm::cuda shim, does not abort) an operator that worked.
+inline void drop_stale_error() { (void)hipGetLastError(); }
+
 // Launchers (defined next to their kernels).  All return hipError_t of the launch.
 hipError_t prefill_launch(const FaArgs& args, int head_dim, int cu_count, hipStream_t stream, void* workspace,
                           size_t workspace_bytes);
 hipError_t prefill_allow_lds();
-// mid, when not null, is recorded between the split kernel and the combine kernel (timing only).
-hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream, hipEvent_t mid = nullptr);
+hipError_t decode_launch(const FaArgs& args, int head_dim, hipStream_t stream);
 hipError_t decode_allow_lds();
 
 // KV-cache mutators (kv_cache.hip).  d_pos not null selects the single-token form that reads
@@ -84,12 +89,6 @@ hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, u
                              bool neox, hipStream_t stream);
 hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
                               hipStream_t stream);
-
-// Measurement aids (bench_aids.hip).
-hipError_t hbm_read_launch(const void* src, size_t bytes, int loads_per_thread, unsigned* sink, hipStream_t stream);
-hipError_t read_pattern_launch(const void* w, size_t mat_bytes, int n_rows, int n_blocks, int pattern, int workgroups, unsigned* sink,
-                               hipStream_t stream);
-hipError_t tiny_launch(const unsigned* src, unsigned* sink, hipStream_t stream);
 
 // ---- timeline build (-DORIN_FA_STAMPS, liborin_fa_stamps.so; a measurement aid) ----
 // The attention kernels carry FA_STAMP(i) marks at the ends of their stages.  In the ordinary
@@ -114,9 +113,6 @@ constexpr int kStampWgs = 1024, kStampSlots = 16;
 hipError_t prefill_stamps(long long* host, size_t n);
 hipError_t decode_stamps(long long* host, size_t n);
 hipError_t gemv_stamps(long long* host, size_t n); // the matrix-vector kernel that reads rows in long runs: waves 0-3 of a workgroup
-constexpr size_t kHandoffScratchBytes = 1u << 20; // partials of both levels and the arrival counters
-constexpr size_t kHandoffStreamBytes = (size_t)256 * 512 * 16 * 16; // 32 MiB read per launch
-hipError_t handoff_launch(const void* src, int fused, void* scratch, float* out, hipStream_t stream);
 
 template <int N>
 struct IntC {

@@ -662,7 +662,7 @@ __global__ __launch_bounds__(512) void fa_decode_combine_kernel(const float* __r
 }
 
 template <int D>
-hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
+hipError_t launch(const FaArgs& a, hipStream_t stream) {
     if (a.n_splits > 0xffff || a.r > 0xffff || a.n_hgroups > 0xffff) return hipErrorInvalidValue;
     constexpr int lds = DGeom<D>::kLdsB;
     const dim3 g(a.n_kv, a.n_hgroups, a.n_splits), b(kDecodeWaves * 64);
@@ -673,8 +673,7 @@ hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
     else if (a.k_new) hipLaunchKernelGGL((fa_decode_split_kernel<D, 1>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
     else hipLaunchKernelGGL((fa_decode_split_kernel<D, 0>), g, b, lds, stream, ORIN_FA_SPLIT_ARGS);
 #undef ORIN_FA_SPLIT_ARGS
-    hipError_t e = hipGetLastError();
-    if (e == hipSuccess && mid) e = hipEventRecord(mid, stream);
+    const hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.n_splits == 1 || kProbeNoCombine) return e;
     const dim3 cgrid(a.n_head * (D / 64));
 #define ORIN_FA_COMBINE_ARGS a.part_o, a.part_ml, a.out, a.n_splits, a.n_head
@@ -688,8 +687,9 @@ hipError_t launch(const FaArgs& a, hipStream_t stream, hipEvent_t mid) {
 
 } // namespace
 
-hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream, hipEvent_t mid) {
-    return head_dim == 128 ? launch<128>(a, stream, mid) : launch<64>(a, stream, mid);
+hipError_t decode_launch(const FaArgs& a, int head_dim, hipStream_t stream) {
+    drop_stale_error();
+    return head_dim == 128 ? launch<128>(a, stream) : launch<64>(a, stream);
 }
 
 // The split kernel uses more than 64 KB of dynamic LDS; the opt-in is set once at init so

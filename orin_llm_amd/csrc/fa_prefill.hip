@@ -1104,6 +1104,7 @@ hipError_t launch(FaArgs a, int cu_count, hipStream_t stream, void* workspace, s
 
 hipError_t prefill_launch(const FaArgs& a, int head_dim, int cu_count, hipStream_t stream, void* workspace,
                           size_t workspace_bytes) {
+    drop_stale_error();
     return head_dim == 128 ? launch<128>(a, cu_count, stream, workspace, workspace_bytes)
                            : launch<64>(a, cu_count, stream, workspace, workspace_bytes);
 }

@@ -480,6 +480,20 @@ bool gemv_use_mfma() {
 }
 void gemv_set_use_mfma(bool on) { g_use_mfma = on ? 1 : 0; }
 
+// Shares of a row that an accumulating projection may be cut into (0: the launcher chooses 1, 2 or 4 by shape;
+// 1: never cut, which makes `y += W x` a plain sum with a fixed order; orin_gemv_row_shares(), or ORIN_GEMV_KSPLIT in
+// the environment as the initial value).
+static int g_row_shares = -1;
+int gemv_row_shares() {
+    if (g_row_shares < 0) {
+        const char* e = getenv("ORIN_GEMV_KSPLIT");
+        const int n = e ? atoi(e) : 0;
+        g_row_shares = n >= 0 && n <= 4 ? n : 0;
+    }
+    return g_row_shares;
+}
+void gemv_set_row_shares(int n) { g_row_shares = n >= 0 && n <= 4 ? n : 0; }
+
 size_t weight_row_bytes(int type, int n) {
     switch (type) {
     case kF32: return (size_t)n * 4;
@@ -495,14 +509,12 @@ size_t weight_row_bytes(int type, int n) {
 int weight_align(int type) { return type == kQ6_K || type == kQ8_0 ? 2 : 16; }
 
 hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
+    drop_stale_error();
     a.row_bytes = weight_row_bytes(type, a.n_in);
     if (a.row_bytes == 0 || a.n_in % 32 != 0 || a.n_seg < 1 || a.n_seg > 3) return hipErrorInvalidValue;
     if (a.wgs_per_cu < 1) a.wgs_per_cu = gemv_wgs_per_cu();
     a.mfma_wgs_per_cu = gemv_mfma_wgs_per_cu();
-    {
-        static const int ks = [] { const char* e = getenv("ORIN_GEMV_KSPLIT"); return e ? atoi(e) : 0; }();
-        a.k_split_override = ks;
-    }
+    a.k_split_override = gemv_row_shares();
     if (gemv_use_mfma() && gemv_mfma_ok(type, a)) return gemv_mfma_launch(type, a, cu_count, stream);
     switch (type) {
     case kF32: return launch_type<kF32>(a, cu_count, stream);
@@ -518,6 +530,7 @@ hipError_t gemv_launch(int type, GemvArgs a, int cu_count, hipStream_t stream) {
 // Matrices of different types over one activation: one launch when every one of them is Q4_K or Q6_K and the
 // matrix-core kernel takes the shape; hipErrorNotSupported otherwise (the caller then launches them one by one).
 hipError_t gemv_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) {
+    drop_stale_error();
     if (!gemv_use_mfma() || a.w_up || a.n_seg < 1 || a.n_seg > 3) return hipErrorNotSupported;
     for (int i = 0; i < a.n_seg; ++i) {
         if (!gemv_mfma_ok(a.seg[i].type, a)) return hipErrorNotSupported;

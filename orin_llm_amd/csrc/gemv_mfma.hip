@@ -100,7 +100,10 @@ __device__ __forceinline__ void digits8(const float (&x)[8], int e, int n_in, un
         mx = fmaxf(mx, dpp_xor_step(mx, 1));
         sum += dpp_xor_step(sum, 1);
     }
-    const float scale = mx > 0.0f ? mx / kDigitRange : 1.0f;
+    // A group that holds an infinity or a NaN gets a NaN scale, so that every row sum it enters is NaN, as the
+    // products of the vector-ALU kernel are (fmaxf above drops a NaN and (int)rintf would turn it into 0; the sum
+    // does not lose it: a sum of floats is finite only if every term is).
+    const float scale = sum - sum == 0.0f ? (mx > 0.0f ? mx / kDigitRange : 1.0f) : __builtin_nanf("");
     const float inv = 1.0f / scale;
     // X + 0x808080 carries 128 into each of the three byte positions, so its bytes are the signed
     // digits plus 128 (byte k of X + 0x808080 is ((X >> 8 k) + 128) & 255 with the lower digits'
@@ -1047,6 +1050,7 @@ hipError_t allow_rows_all() {
 
 // Every matrix of a block type (Q4_K, Q5_K, Q6_K, Q8_0), each its own type (GemvSeg::type, row_bytes filled in by the caller).
 hipError_t gemv_mfma_mixed_launch(GemvArgs a, int cu_count, hipStream_t stream) {
+    drop_stale_error();
     int max_out = 0;
     for (int i = 0; i < a.n_seg; ++i) max_out = max(max_out, a.seg[i].n_out);
     const int cap = a.mfma_wgs_per_cu > 0 ? cu_count * a.mfma_wgs_per_cu : (max_out + 15) / 16;
@@ -1093,6 +1097,7 @@ bool gemv_mfma_ok(int type, const GemvArgs& a) {
 }
 
 hipError_t gemv_mfma_launch(int type, const GemvArgs& a, int cu_count, hipStream_t stream) {
+    drop_stale_error();
     switch (type) {
     case kQ4_K: return launch<kQ4_K>(a, cu_count, stream);
     case kQ5_K: return launch<kQ5_K>(a, cu_count, stream);

@@ -96,6 +96,7 @@ __global__ __launch_bounds__(256) void kv_shift_kernel(uint16_t* kc, uint16_t* v
 
 hipError_t kv_store_launch(uint16_t* kc, uint16_t* vc, const float* k, const float* v, int heads, int head_dim,
                            int n_ctx, int pos_base, int batch, const int* d_pos, hipStream_t stream) {
+    drop_stale_error();
     const bool vec = head_dim % 8 == 0 &&
                      ((reinterpret_cast<uintptr_t>(kc) | reinterpret_cast<uintptr_t>(vc) |
                        reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) & 15u) == 0;
@@ -114,6 +115,7 @@ hipError_t kv_store_launch(uint16_t* kc, uint16_t* vc, const float* k, const flo
 
 hipError_t kv_shift_launch(uint16_t* kc, uint16_t* vc, int n_layer, int n_kv, int head_dim, int n_ctx, int n_keep,
                            int shift, hipStream_t stream) {
+    drop_stale_error();
     const int row_bytes = head_dim * 2;
     const bool vec = row_bytes % 16 == 0 &&
                      ((reinterpret_cast<uintptr_t>(kc) | reinterpret_cast<uintptr_t>(vc)) & 15u) == 0;

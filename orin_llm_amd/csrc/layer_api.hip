@@ -35,7 +35,7 @@ int gemv_call(int type, int n_mat, const void* const* w, const float* const* bia
     for (int i = 0; i < n_mat; ++i) {
         const int rc = check_matrix(type, w[i], n_in, n_out[i]);
         if (rc != ORIN_FA_OK) return rc;
-        if (!y[i]) return ORIN_FA_E_INVALID;
+        if (!y[i] || !aligned(y[i], 4) || (bias && bias[i] && !aligned(bias[i], 4))) return ORIN_FA_E_INVALID;
         a.seg[i] = GemvSeg{w[i], bias ? bias[i] : nullptr, y[i], n_out[i], type, 0};
     }
     if (w_up) {
@@ -64,7 +64,7 @@ int gemv_call_mixed(const int* types, int n_mat, const void* const* w, const flo
     for (int i = 0; i < n_mat; ++i) {
         const int rc = check_matrix(types[i], w[i], n_in, n_out[i]);
         if (rc != ORIN_FA_OK) return rc;
-        if (!y[i]) return ORIN_FA_E_INVALID;
+        if (!y[i] || !aligned(y[i], 4) || (bias && bias[i] && !aligned(bias[i], 4))) return ORIN_FA_E_INVALID;
         a.seg[i] = GemvSeg{w[i], bias ? bias[i] : nullptr, y[i], n_out[i], types[i], 0};
     }
     a.n_seg = n_mat;
@@ -81,9 +81,15 @@ int gemv_one(int type, const void* w, const float* bias, float* y, int n_out, co
     return gemv_call(type, 1, &w, &bias, &y, &n_out, w_up, x, norm_w, eps, n_in, accumulate);
 }
 
+// The staged activation for a product over n_in elements: the first n_in of what the last
+// orin_quantize_activation staged.  The reference's products read the first n_in elements of its g_q8 block
+// whatever length was quantised (src/kernels.cu:1786-1836), and its decode_layer relies on that: it stages
+// n_embd elements of d_attn_ and multiplies by wo, whose rows have n_head * head_dim (src/model_gpu.cu:284-285),
+// which is shorter in models whose heads do not add up to n_embd.  A product longer than what was staged would
+// read elements nobody staged: refused.
 int staged(int n_in, const float** x) {
     if (!lib_ready()) return ORIN_FA_E_NOT_INIT;
-    if (!lib_stage() || g_staged_n != n_in) return ORIN_FA_E_INVALID; // no orin_quantize_activation of this length came before
+    if (!lib_stage() || g_staged_n < n_in) return ORIN_FA_E_INVALID;
     *x = lib_stage();
     return ORIN_FA_OK;
 }
@@ -96,6 +102,8 @@ using namespace orin_fa;
 extern "C" {
 
 void orin_gemv_use_matrix_cores(int on) { gemv_set_use_mfma(on != 0); }
+
+void orin_gemv_row_shares(int shares) { gemv_set_row_shares(shares); }
 
 size_t orin_row_bytes(int type, int n) { return n < 0 ? 0 : weight_row_bytes(type, n); }
 
@@ -195,6 +203,16 @@ int orin_decode_layer(const orin_decode_layer_desc* L) {
     if (L->gate_type != L->up_type && !L->up_tmp) return ORIN_FA_E_INVALID; // (checked here so that nothing has run when it fails)
     const int nq = L->n_head * L->head_dim, nkv = L->n_kv * L->head_dim;
     int rc;
+    // Every product's row length against the kernels' limit, before the first launch: a layer refused half way
+    // would leave x updated by its first half.
+    {
+        const int n_in[7] = {L->n_embd, L->n_embd, L->n_embd, nq, L->n_embd, L->n_embd, L->n_ff};
+        const int n_out[7] = {nq, nkv, nkv, L->n_embd, L->n_ff, L->n_ff, L->n_embd};
+        const int t[7] = {L->wq_type, L->wk_type, L->wv_type, L->wo_type, L->gate_type, L->up_type, L->down_type};
+        const void* w[7] = {L->wq, L->wk, L->wv, L->wo, L->ffn_gate, L->ffn_up, L->ffn_down};
+        for (int i = 0; i < 7; ++i)
+            if ((rc = check_matrix(t[i], w[i], n_in[i], n_out[i])) != ORIN_FA_OK) return rc;
+    }
     // ---- attn_norm + q, k, v projections: matrices of one type share a launch ----
     {
         const void* w[3] = {L->wq, L->wk, L->wv};

@@ -50,6 +50,8 @@ hipError_t gemv_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
 hipError_t gemv_mfma_mixed_launch(GemvArgs args, int cu_count, hipStream_t stream);
 bool gemv_use_mfma();
 void gemv_set_use_mfma(bool on);
+int gemv_row_shares();          // 0: chosen by shape; 1: accumulating projections never cut a row into shares
+void gemv_set_row_shares(int n);
 
 hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream);
 hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream);

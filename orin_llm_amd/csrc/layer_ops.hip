@@ -107,6 +107,7 @@ __global__ __launch_bounds__(256) void dequant_row_kernel(int type, const unsign
 } // namespace
 
 hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, float eps, float* y, hipStream_t stream) {
+    drop_stale_error();
     if (cols <= 256)
         hipLaunchKernelGGL((rms_norm_kernel<64>), dim3(rows), dim3(64), 0, stream, x, w, cols, eps, y);
     else
@@ -115,16 +116,19 @@ hipError_t rms_norm_launch(const float* x, const float* w, int rows, int cols, f
 }
 
 hipError_t stage_launch(const float* x, float* stage, int n, hipStream_t stream) {
+    drop_stale_error();
     hipLaunchKernelGGL(stage_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, x, stage, n);
     return hipGetLastError();
 }
 
 hipError_t swiglu_launch(float* act, const float* gate, const float* up, int n, hipStream_t stream) {
+    drop_stale_error();
     hipLaunchKernelGGL(swiglu_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, act, gate, up, n);
     return hipGetLastError();
 }
 
 hipError_t dequant_row_launch(int type, const void* src, float* y, int n, hipStream_t stream) {
+    drop_stale_error();
     hipLaunchKernelGGL(dequant_row_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, type,
                        static_cast<const unsigned char*>(src), y, n);
     return hipGetLastError();

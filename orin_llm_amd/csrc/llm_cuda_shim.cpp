@@ -1,5 +1,5 @@
 // llm::cuda::* entry points with the reference's signatures (reference:
-// src/kernels.h:8-10,15-47,55-62,66-73,77-81; definitions src/kernels.cu:1728-1737,1778-1836,1944-2044,2059-2093),
+// src/kernels.h:8-12,15-47,55-62,66-73,77-81; definitions src/kernels.cu:1728-1776,1778-1836,1944-2044,2059-2093),
 // forwarding to the C ABI.  Plain C++: no HIP headers, no device code.
 #include "../../include/orin_llm_amd/kernels.h"
 
@@ -33,6 +33,27 @@ int init() {
 }
 
 void set_stream(void* stream) { orin_fa_set_stream(stream); }
+
+// The reference prints the name, compute capability and memory of device 0 (src/kernels.cu:1739-1744).
+void device_info() {
+    char name[256];
+    int cus = 0;
+    size_t mem = 0;
+    const int rc = orin_fa_device_info(0, name, sizeof name, &cus, &mem);
+    if (rc != ORIN_FA_OK) die("device_info", rc);
+    printf("[hip] device: %s (%d CUs, %.1f GB)\n", name, cus, (double)mem / (double)(1u << 30));
+}
+
+// The reference sizes and carves its int8 staging buffers and the batched GEMM's scratch here
+// (src/kernels.cu:1753-1776).  This library needs one block: the attention kernels' split-KV partial results.
+// 256 bytes more than that, so that scratch_assign can align whatever base it is given.
+size_t scratch_size(int, int) { return orin_fa_workspace_bytes() + 256; }
+
+void scratch_assign(void* base, int, int) {
+    void* const aligned = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(base) + 255u) & ~(uintptr_t)255u);
+    const int rc = orin_fa_set_workspace(aligned, orin_fa_workspace_bytes());
+    if (rc != ORIN_FA_OK) die("scratch_assign", rc);
+}
 #endif
 
 void quantize_activation(const float* x, int n_in) {

@@ -249,6 +249,7 @@ __global__ __launch_bounds__(64) void rope_angles_kernel(float* angles, int n_ro
 
 hipError_t rope_angles_launch(float* angles, int n_rot, float theta, const int* d_pos, const float* freq_factors,
                               hipStream_t stream) {
+    drop_stale_error();
     const unsigned grid = (unsigned)((n_rot / 2 + 63) / 64);
     if (grid == 0) return hipSuccess;
     hipLaunchKernelGGL(rope_angles_kernel, dim3(grid), dim3(64), 0, stream, angles, n_rot, theta, d_pos, freq_factors);
@@ -265,6 +266,7 @@ bool rope_store_fused_ok(const float* q, const float* k, const float* v, const u
 hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, uint16_t* vc, int tokens, int n_head,
                              int n_kv, int head_dim, int n_ctx, int n_past, float theta, const float* freq_factors,
                              bool neox, hipStream_t stream) {
+    drop_stale_error();
     const int quads = head_dim / 8;
     auto blocks = [](long long threads) { return (unsigned)((threads + 255) / 256); };
     const unsigned nbq = blocks((long long)tokens * ((n_head + kHeadsPerThread4 - 1) / kHeadsPerThread4) * quads);
@@ -282,6 +284,7 @@ hipError_t rope_store_launch(float* q, float* k, const float* v, uint16_t* kc, u
 
 hipError_t rope_launch(float* x, int rows, int head_dim, int n_rot, float theta, int n_past, int heads,
                        const int* d_pos, const float* freq_factors, bool neox, hipStream_t stream) {
+    drop_stale_error();
     // batch form: rows = tokens * heads; single-token form: every row belongs to the one token
     const int tokens = d_pos ? 1 : rows / heads;
     const int heads_per_token = d_pos ? rows : heads;

@@ -15,9 +15,12 @@ _int = ctypes.c_int
 _flt = ctypes.c_float
 
 STAMPS_LIB_PATH = os.path.join(_HERE, "liborin_fa_stamps.so")
+BENCH_LIB_PATH = os.path.join(_HERE, "liborin_fa_bench.so")
 
 _lib = None
 _stamps_lib = None
+_bench_lib = None
+_stream = None  # what set_stream was last given: the measurement aids launch on it too
 
 
 class OrinFaError(RuntimeError):
@@ -69,21 +72,6 @@ def lib():
         L.orin_fa_kv_store_ind.restype = _int
         L.orin_fa_kv_shift.argtypes = [_vp, _vp, _int, _int, _int, _int, _int, _int]
         L.orin_fa_kv_shift.restype = _int
-        L.orin_fa_decode_ind_timed.argtypes = [_vp, _vp, _vp, _vp, _int, _int, _int, _int, _vp, _flt,
-                                               ctypes.POINTER(_flt), ctypes.POINTER(_flt)]
-        L.orin_fa_decode_ind_timed.restype = _int
-        L.orin_fa_bench_hbm_read.argtypes = [_vp, ctypes.c_size_t, _int]
-        L.orin_fa_bench_hbm_read.restype = _int
-        L.orin_fa_bench_read_pattern.argtypes = [_vp, ctypes.c_size_t, _int, _int, _int, _int]
-        L.orin_fa_bench_read_pattern.restype = _int
-        L.orin_fa_bench_handoff.argtypes = [_vp, _int, _vp, _vp]
-        L.orin_fa_bench_handoff.restype = _int
-        L.orin_fa_bench_handoff_scratch_bytes.argtypes = []
-        L.orin_fa_bench_handoff_scratch_bytes.restype = ctypes.c_size_t
-        L.orin_fa_bench_handoff_stream_bytes.argtypes = []
-        L.orin_fa_bench_handoff_stream_bytes.restype = ctypes.c_size_t
-        L.orin_fa_bench_tiny_launch.argtypes = []
-        L.orin_fa_bench_tiny_launch.restype = _int
         L.orin_fa_decode_splits.argtypes = [_int, _int, _int, _int]
         L.orin_fa_decode_splits.restype = _int
         L.orin_fa_cu_count.argtypes = []
@@ -115,7 +103,9 @@ def init(device=0):
 
 def set_stream(stream):
     """stream: a hipStream_t address (e.g. torch.cuda.Stream.cuda_stream), or None/0 for the null stream."""
-    lib().orin_fa_set_stream(_ptr(stream) or None)
+    global _stream
+    _stream = _ptr(stream) or None
+    lib().orin_fa_set_stream(_stream)
 
 
 def workspace_bytes():
@@ -234,17 +224,6 @@ def kv_shift(kc, vc, n_layer, n_kv, head_dim, n_ctx, n_keep, shift):
         raise OrinFaError("kv_shift", rc)
 
 
-def flash_attention_decode_ind_timed(q, kc, vc, out, n_head, n_kv, head_dim, n_ctx, d_pos, scale):
-    """Measurement aid: the same launch with HIP events around its two kernels; synchronises and
-    returns (microseconds of the split kernel, microseconds of the combine kernel)."""
-    us_split, us_combine = _flt(0.0), _flt(0.0)
-    rc = lib().orin_fa_decode_ind_timed(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), n_head, n_kv, head_dim, n_ctx,
-                                        _ptr(d_pos), scale, ctypes.byref(us_split), ctypes.byref(us_combine))
-    if rc != 0:
-        raise OrinFaError("flash_attention_decode_ind_timed", rc)
-    return us_split.value, us_combine.value
-
-
 def decode_splits(n_head, n_kv, head_dim, n_ctx):
     return int(lib().orin_fa_decode_splits(n_head, n_kv, head_dim, n_ctx))
 
@@ -253,33 +232,53 @@ def cu_count():
     return int(lib().orin_fa_cu_count())
 
 
-def bench_hbm_read(src, nbytes, loads_per_thread=16):
-    """Measurement aid: one launch of a plain streaming read of nbytes at src."""
-    rc = lib().orin_fa_bench_hbm_read(_ptr(src), int(nbytes), int(loads_per_thread))
+def bench_lib():
+    """The measurement aids' own library (include/orin_fa_bench.h): read-only stand-ins and a do-nothing kernel."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with __graft_entry__.build()")
+        L = ctypes.CDLL(BENCH_LIB_PATH)
+        L.orin_fa_bench_hbm_read.argtypes = [_vp, ctypes.c_size_t, _int, _vp, _vp]
+        L.orin_fa_bench_read_pattern.argtypes = [_vp, ctypes.c_size_t, _int, _int, _int, _int, _vp, _vp]
+        L.orin_fa_bench_handoff.argtypes = [_vp, _int, _vp, _vp, _vp]
+        L.orin_fa_bench_tiny_launch.argtypes = [_vp, _vp, _vp]
+        for n in ("orin_fa_bench_hbm_read", "orin_fa_bench_read_pattern", "orin_fa_bench_handoff", "orin_fa_bench_tiny_launch"):
+            getattr(L, n).restype = _int
+        L.orin_fa_bench_handoff_scratch_bytes.argtypes = []
+        L.orin_fa_bench_handoff_scratch_bytes.restype = ctypes.c_size_t
+        L.orin_fa_bench_handoff_stream_bytes.argtypes = []
+        L.orin_fa_bench_handoff_stream_bytes.restype = ctypes.c_size_t
+        _bench_lib = L
+    return _bench_lib
+
+
+def _bench_check(what, rc):
     if rc != 0:
-        raise OrinFaError("bench_hbm_read", rc)
+        raise RuntimeError(f"{what}: measurement aid returned {rc}")
 
 
-def bench_read_pattern(w, mat_bytes, n_rows, n_blocks, pattern, workgroups):
+def bench_hbm_read(src, nbytes, sink, loads_per_thread=16):
+    """Measurement aid: one launch (on the stream of set_stream) of a plain streaming read of nbytes at src;
+    sink: a device word."""
+    _bench_check("bench_hbm_read", bench_lib().orin_fa_bench_hbm_read(_ptr(src), int(nbytes), int(loads_per_thread), _ptr(sink), _stream))
+
+
+def bench_read_pattern(w, mat_bytes, n_rows, n_blocks, pattern, workgroups, sink):
     """Measurement aid: one launch of a read-only stand-in for a matrix-vector kernel's loads over a pair of Q4_K-shaped matrices."""
-    rc = lib().orin_fa_bench_read_pattern(_ptr(w), int(mat_bytes), int(n_rows), int(n_blocks), int(pattern), int(workgroups))
-    if rc != 0:
-        raise OrinFaError("bench_read_pattern", rc)
+    _bench_check("bench_read_pattern", bench_lib().orin_fa_bench_read_pattern(_ptr(w), int(mat_bytes), int(n_rows), int(n_blocks),
+                                                                              int(pattern), int(workgroups), _ptr(sink), _stream))
 
 
-def bench_tiny_launch():
-    """Measurement aid: one launch of a one-wave kernel."""
-    rc = lib().orin_fa_bench_tiny_launch()
-    if rc != 0:
-        raise OrinFaError("bench_tiny_launch", rc)
+def bench_tiny_launch(src, sink):
+    """Measurement aid: one launch of a one-wave kernel that reads the word at src."""
+    _bench_check("bench_tiny_launch", bench_lib().orin_fa_bench_tiny_launch(_ptr(src), _ptr(sink), _stream))
 
 
 def bench_handoff(src, fused, scratch, out):
     """Measurement aid: a stand-in for a split-KV decode step, partial results merged by a second
     kernel (fused=False) or inside the launch (fused=True)."""
-    rc = lib().orin_fa_bench_handoff(_ptr(src), int(fused), _ptr(scratch), _ptr(out))
-    if rc != 0:
-        raise OrinFaError("bench_handoff", rc)
+    _bench_check("bench_handoff", bench_lib().orin_fa_bench_handoff(_ptr(src), int(fused), _ptr(scratch), _ptr(out), _stream))
 
 
 def probe_lib(flags, prefill=False):
@@ -288,7 +287,7 @@ def probe_lib(flags, prefill=False):
     fa_prefill.hip) as an independent ctypes handle.  A measurement aid of bench.py."""
     path = os.path.join(_HERE, f"liborin_fa_{'pprobe' if prefill else 'probe'}_{int(flags)}.so")
     if not os.path.exists(path):
-        raise ImportError(f"{path} is missing: build it with __graft_entry__.build()")
+        raise ImportError(f"{path} is missing: build the cut-off libraries with `python -m orin_llm_amd.build --probes`")
     L = ctypes.CDLL(path)
     L.orin_fa_init.argtypes = [_int]
     L.orin_fa_init.restype = _int
@@ -327,4 +326,4 @@ def stamps_lib():
 
 
 def bench_handoff_sizes():
-    return int(lib().orin_fa_bench_handoff_stream_bytes()), int(lib().orin_fa_bench_handoff_scratch_bytes())
+    return int(bench_lib().orin_fa_bench_handoff_stream_bytes()), int(bench_lib().orin_fa_bench_handoff_scratch_bytes())

@@ -30,6 +30,8 @@ def _lib():
     if not _ready:
         L.orin_gemv_use_matrix_cores.argtypes = [_int]
         L.orin_gemv_use_matrix_cores.restype = None
+        L.orin_gemv_row_shares.argtypes = [_int]
+        L.orin_gemv_row_shares.restype = None
         L.orin_row_bytes.argtypes = [_int, _int]
         L.orin_row_bytes.restype = ctypes.c_size_t
         L.orin_rms_norm.argtypes = [_vp, _vp, _int, _flt, _vp]
@@ -67,6 +69,12 @@ def _check(what, rc):
 def use_matrix_cores(on):
     """Block types on the matrix cores (default) or on the vector ALU (for comparisons and tests)."""
     _lib().orin_gemv_use_matrix_cores(1 if on else 0)
+
+
+def gemv_row_shares(shares):
+    """Shares an accumulating projection may cut a row into: 0 = chosen by shape (default), 1 = never cut (every
+    result bit for bit reproducible)."""
+    _lib().orin_gemv_row_shares(int(shares))
 
 
 def row_bytes(wtype, n):
@@ -192,7 +200,7 @@ def _decode_layer_calls(o, ka, hp, L, bufs, kc, vc, d_pos, n_ctx):
     rope_ind(k, nkv, hd, hp["n_rot"], hp["rope_theta"], d_pos, hp.get("freq_factors_dev"))
     ka.kv_store_ind(kc, vc, k, v, nkv, hd, n_ctx, d_pos)
     ka.flash_attention_decode_ind(q, kc, vc, attn, nh, nkv, hd, n_ctx, d_pos, scale)
-    quantize_activation(attn, nh * hd)
+    quantize_activation(attn, ne)  # (as the reference: n_embd elements staged, the product reads the first n_head * head_dim)
     gemv_q8_add(L["wo"][0], L["wo"][1], x, nh * hd, ne)
     rms_norm(x, L["ffn_norm"], ne, eps, xn2)
     quantize_activation(xn2, ne)

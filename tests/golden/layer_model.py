@@ -97,6 +97,14 @@ VARIANTS = {
                    embd=Q6_K, output=None,
                    types=[dict(wq=Q5_K, wk=Q5_K, wv=Q5_K, wo=Q6_K, ffn_gate=Q8_0, ffn_up=Q8_0, ffn_down=Q4_K),
                           dict(wq=Q4_K, wk=Q6_K, wv=Q6_K, wo=Q8_0, ffn_gate=Q6_K, ffn_up=Q6_K, ffn_down=Q5_K)]),
+    # heads that do not add up to n_embd (n_head * head_dim = 512 < n_embd = 768), with per-head q/k norms: the
+    # output projection's rows are shorter than what the reference's decode_layer stages ahead of it
+    # (src/model_gpu.cu:284-285)
+    "narrow": dict(arch="qwen3", seed=505, n_embd=768, n_head=4, n_kv=2, head_dim=128, n_ff=1024, n_layer=2,
+                   n_vocab=88, n_rot=128, theta=1.0e6, eps=1.0e-6, bias=False, qk_norm=True, factors=False,
+                   embd=Q4_K, output=Q6_K,
+                   types=[dict(wq=Q4_K, wk=Q4_K, wv=Q6_K, wo=Q4_K, ffn_gate=Q4_K, ffn_up=Q4_K, ffn_down=Q6_K),
+                          dict(wq=Q8_0, wk=Q5_K, wv=F16, wo=Q6_K, ffn_gate=Q5_K, ffn_up=Q4_K, ffn_down=Q8_0)]),
 }
 N_TOKENS = 12
 

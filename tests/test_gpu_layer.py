@@ -119,10 +119,90 @@ def test_staged_products_bias_add_and_snapshot(ly, wtype):
     assert vec_err(yb.cpu().numpy()[:n_out], (base + bias).astype(np.float64)) < TOL_OP
     assert vec_err(ya.cpu().numpy()[:n_out], (y0 + base).astype(np.float64)) < TOL_OP
     assert (ya.cpu().numpy()[n_out:] == 12345.0).all() and (yb.cpu().numpy()[n_out:] == 12345.0).all()
-    # a product of another length than the staged one is refused
+    # a shorter product reads the first elements of what was staged, as the reference's do (its decode_layer stages
+    # n_embd elements ahead of the output projection, whose rows have n_head * head_dim: src/model_gpu.cu:284-285) ...
+    n_short = n_in // 2 if wtype == lm.F16 else 1280
+    rb, rb_short = ref.row_bytes(wtype, n_in), ref.row_bytes(wtype, n_short)
+    t_short = np.concatenate([t[1][r * rb:r * rb + rb_short] for r in range(n_out)])
+    ys = out_buf(n_out)
+    ly.gemv_q8(wtype, dev_bytes(t_short), ys, n_short, n_out)
+    torch.cuda.synchronize()
+    assert vec_err(ys.cpu().numpy()[:n_out], ref.gemv(wtype, t_short, x[:n_short], n_short, n_out).astype(np.float64)) < TOL_OP
+    # ... and a longer one, which would read what nobody staged, is refused
     from orin_llm_amd.kernels import OrinFaError
+    ly.quantize_activation(dx, n_short)
     with pytest.raises(OrinFaError):
-        ly.gemv_q8(wtype, w, y, n_in // 2 if wtype == lm.F16 else 1280, n_out)
+        ly.gemv_q8(wtype, w, y, n_in, n_out)
+
+
+@pytest.mark.parametrize("wtype,n_in,n_out", [(lm.Q4_K, 4096, 1536), (lm.Q6_K, 8960, 1536), (lm.Q6_K, 14336, 4096)])
+def test_accumulating_projection_is_bit_stable_with_one_share(ly, wtype, n_in, n_out):
+    """y += W x over long rows of a matrix with few rows (the output and down projections): by default a row is cut
+    into shares that meet by atomic adds in no fixed order, so repeated runs agree to the order of an fp32 sum only;
+    with orin_gemv_row_shares(1) every run gives the same bits (the reference's gemv_q8_add is a plain sum,
+    src/kernels.cu:350-374)."""
+    import torch
+
+    rs = lm.Stream(7000 + wtype + n_in)
+    t = lm.make_tensor(rs, wtype, n_in, n_out)
+    x, y0 = rs.sym(n_in, 1.0), rs.sym(n_out, 2.0)
+    want = (y0 + ref.gemv(wtype, t[1], x, n_in, n_out)).astype(np.float64)
+    w, dx = dev_bytes(t[1], offset=2 if wtype == lm.Q6_K else 0), _dev(x)
+
+    def runs(n):
+        out = []
+        for _ in range(n):
+            y = _dev(y0)
+            ly.gemv_multi(wtype, [w], None, [y], [n_out], dx, None, 0.0, n_in, True)
+            torch.cuda.synchronize()
+            out.append(y.cpu().numpy())
+        return out
+
+    try:
+        ly.gemv_row_shares(0)
+        shared = runs(20)
+        ly.gemv_row_shares(1)
+        single = runs(20)
+    finally:
+        ly.gemv_row_shares(0)
+    for y in shared + single:
+        assert vec_err(y, want) < TOL_OP
+    assert all(np.array_equal(single[0].view(np.uint32), y.view(np.uint32)) for y in single[1:])
+    spread = max(float(np.abs(y.astype(np.float64) - shared[0]).max() / np.abs(want).max()) for y in shared[1:])
+    print(f"type {wtype} {n_in} x {n_out}: spread over 20 runs with shares {spread:.1e}", flush=True)
+    assert spread < 1e-6   # (a few units in the last place of the largest element)
+
+
+@pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q6_K, lm.Q8_0])
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
+def test_a_non_finite_activation_is_not_laundered(ly, wtype, bad):
+    """An infinity or a NaN in the activation makes every row's sum non-finite on the matrix cores as on the vector
+    ALU (the int8 digits of the matrix-core path cannot carry it: its sub-block's scale does)."""
+    import torch
+
+    n_in, n_out = 1536, 48
+    rs = lm.Stream(8100 + wtype)
+    t = lm.make_tensor(rs, wtype, n_in, n_out)
+    x = rs.sym(n_in, 1.0)
+    x[777] = bad
+    w = dev_bytes(t[1], offset=2 if wtype in (lm.Q6_K, lm.Q8_0) else 0)
+    got = {}
+    for unit in (1, 0):
+        ly.use_matrix_cores(unit)
+        try:
+            y = out_buf(n_out)
+            ly.gemv(wtype, w, _dev(x), y, n_in, n_out)
+            torch.cuda.synchronize()
+            got[unit] = y.cpu().numpy()[:n_out]
+        finally:
+            ly.use_matrix_cores(1)
+    assert not np.isfinite(got[1]).any() and not np.isfinite(got[0]).any()
+    # the same rows over a finite activation stay finite (the flag is per sub-block and per launch)
+    x[777] = 0.5
+    y = out_buf(n_out)
+    ly.gemv(wtype, w, _dev(x), y, n_in, n_out)
+    torch.cuda.synchronize()
+    assert vec_err(y.cpu().numpy()[:n_out], ref.gemv(wtype, t[1], x, n_in, n_out).astype(np.float64)) < TOL_OP
 
 
 def test_q8_0_rows_that_are_not_whole_256s_stay_on_the_vector_alu(ly):
@@ -299,6 +379,8 @@ def test_dequant_row_bit_exact(ly, wtype):
 
 
 def test_rejects_bad_arguments(ly):
+    import torch
+
     from orin_llm_amd.kernels import OrinFaError
 
     w = dev_bytes(np.zeros(144 * 8, np.uint8))
@@ -307,6 +389,7 @@ def test_rejects_bad_arguments(ly):
                  lambda: ly.gemv(7, w, x, y, 256, 2),                  # unknown type
                  lambda: ly.gemv(lm.Q4_K, w[4:], x, y, 256, 2),        # misaligned matrix
                  lambda: ly.gemv(lm.Q4_K, w, x[1:], y, 256, 2),        # misaligned activation
+                 lambda: ly.gemv(lm.Q4_K, w, x, y.view(torch.uint8)[2:10].view(torch.int16), 256, 2),  # output not on a float boundary
                  lambda: ly.gemv(lm.F16, w, x, y, 32768, 1),           # longer than a workgroup covers
                  lambda: ly.gemv(lm.Q4_K, None, x, y, 256, 2),
                  lambda: ly.quantize_activation(x, 40000)):
@@ -370,7 +453,8 @@ def make_bufs(hp):
 
     z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")  # noqa: E731
     nq, nkv = hp["n_head"] * hp["head_dim"], hp["n_kv"] * hp["head_dim"]
-    return dict(x=z(hp["n_embd"]), xn=z(hp["n_embd"]), xn2=z(hp["n_embd"]), q=z(nq), k=z(nkv), v=z(nkv), attn=z(nq),
+    # (attn as large as the reference's: its decode_layer stages n_embd elements of it, src/model_gpu.cu:284)
+    return dict(x=z(hp["n_embd"]), xn=z(hp["n_embd"]), xn2=z(hp["n_embd"]), q=z(nq), k=z(nkv), v=z(nkv), attn=z(max(nq, hp["n_embd"])),
                 act=z(hp["n_ff"]), up_tmp=z(hp["n_ff"]), logits=z(hp["n_vocab"]))
 
 

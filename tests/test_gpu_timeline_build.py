@@ -69,11 +69,8 @@ def test_timeline_build_gives_the_same_results_and_ordered_marks():
 
 
 def test_ordinary_library_has_no_stamps():
-    torch = pytest.importorskip("torch")
+    """The stage marks and their reader exist in the timeline build only: the product library does not export them."""
     from orin_llm_amd import kernels
 
-    kernels.init(0)
-    lib = kernels.lib()
-    lib.orin_fa_bench_stamps.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t]
-    host = np.zeros(64, np.int64)
-    assert lib.orin_fa_bench_stamps(0, host.ctypes.data, host.size) != 0
+    assert not hasattr(kernels.lib(), "orin_fa_bench_stamps")
+    assert hasattr(kernels.stamps_lib(), "orin_fa_bench_stamps")

@@ -178,7 +178,7 @@ LAYER_SHIM = {  # the rest of what decode_layer calls (reference: src/model_gpu.
 }
 
 
-@pytest.mark.parametrize("name", ["qwen2", "llama", "qwen2p"])
+@pytest.mark.parametrize("name", ["qwen2", "llama", "qwen2p", "narrow"])
 def test_whole_decode_step_through_the_shim_replayed_from_a_graph(shim, name):
     """The reference's forward_capture (src/model_gpu.cu:295-316) over a small quantised model: embedding
     row, every layer call for call, last norm, output matrix -- through the llm::cuda symbols, captured once

@@ -5,15 +5,17 @@ import numpy as np
 #   TOL            err_row < 2e-3, everywhere.
 #   FLOOR_DECODE   err_floor1pct < 2e-3 for decode (fp16 hi + lo operands: fp32-accurate), wherever
 #                  both sides read the same cache values.
-#   FLOOR_PREFILL  err_floor1pct < 5e-2 for prefill: its weights P are single fp16 values (the
+#   FLOOR_PREFILL  err_floor1pct < 4e-2 for prefill: its weights P are single fp16 values (the
 #                  reference GPU kernel's choice too), whose rounding alone costs about
-#                  100 x err_row on this figure; the bound keeps that figure from drifting.
+#                  100 x err_row on this figure; the bound keeps that figure from drifting
+#                  (largest value any test measures: 3.8e-2, test_prefill_row_equals_decode_and_chunk_split;
+#                  the benchmark's stacks: 2.6e-2).
 #   FLOOR_FP32_KV  err_floor1pct < 1e-1 where the reference side kept K/V in fp32 and the GPU
 #                  reads the fp16 cache (config 1, faithful variant): the cache format alone
 #                  scores 4.9e-2 (tests/test_oracle.py::test_fp16_cache_format_error).
 TOL = 2e-3
 FLOOR_DECODE = 2e-3
-FLOOR_PREFILL = 5e-2
+FLOOR_PREFILL = 4e-2
 FLOOR_FP32_KV = 1e-1
 
 
