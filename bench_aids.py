@@ -66,7 +66,8 @@ def run_patterns(torch, kernels, name, steps, warmup, with_cpu):
 
 
 # Stage marks of the kernels (slot, what has happened by then), in the order a wave passes them.
-PREFILL_STAGES = [(0, "entry"), (9, "queries and first K tile requested"), (10, "first V tile and second K tile requested"),
+PREFILL_STAGES = [(0, "entry"), (9, "queries and first K tile requested"), (11, "output accumulators cleared"), (12, "first V buffer cleared"),
+                  (13, "first V tile requested"), (10, "second K tile requested"),
                   (1, "queries in registers"), (2, "first two score tiles"), (3, "first weights"), (4, "main loop done"),
                   (5, "last products done, accumulators in LDS"), (7, "barrier passed"), (8, "output stored")]
 GEMV_STAGES = [(0, "entry"), (1, "first two items of weights requested"), (2, "digits of the wave's part of the activation done"),

@@ -384,69 +384,95 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fa_decode_split_kernel(
     for (int db = 0; db < G::kDBlk; ++db) o[db] = f4{0.f, 0.f, 0.f, 0.f};
     const int v_rd = (grp * 4 + (col >> 2)) * G::kRowBV + (col & 3) * 8; // + h*16 rows, + db*32 bytes
 
+    // (store, rotate + store) The new row is made ready here, while the tiles travel, by the one wave whose tiles
+    // include the row's (the last visible tile: the wave's own last): converted -- and the K row rotated -- as the
+    // store kernel and the rotary kernel would, the pieces this lane is to substitute and to write kept in
+    // registers.  At that tile only the substitution and the two cache writes are left.  (Made ready at the tile
+    // itself, as it used to be, the LDS round trips and the rotation sat between the arrival of the launch's last
+    // tile and its products: 0.7 us of a Qwen2.5-1.5B launch pair at 32k.)  The row's loads went out ahead of the
+    // tile requests, so waiting for them waits for no tile.
+    const int own_tile = n_tiles - 1;
+    [[maybe_unused]] bool owner = false;
+    [[maybe_unused]] u32x4 k_new16[G::kSteps], v_new16 = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (STORE) {
+#pragma unroll
+        for (int kk = 0; kk < G::kSteps; ++kk) k_new16[kk] = u32x4{0u, 0u, 0u, 0u};
+        owner = store && tile_first <= own_tile && (own_tile - tile_first) % tile_step == 0;
+        if (owner) {
+            // (Nothing below may be started ahead of this branch: the compiler would otherwise
+            // convert the new row in every wave.)
+            auto here = [](float x) { // a copy the compiler cannot make anywhere else
+                float y;
+                asm volatile("v_mov_b32 %0, %1" : "=v"(y) : "v"(x));
+                return y;
+            };
+            const float4 k_own = float4{here(k_raw.x), here(k_raw.y), here(k_raw.z), here(k_raw.w)};
+            const float4 v_own[2] = {float4{here(v_raw[0].x), here(v_raw[0].y), here(v_raw[0].z), here(v_raw[0].w)},
+                                     float4{here(v_raw[1].x), here(v_raw[1].y), here(v_raw[1].z), here(v_raw[1].w)}};
+            {
+                // The new K row is rotated (rotate + store) and converted by the one wave
+                // that needs it.  It has waited in four registers a lane; the lanes now hand
+                // each other the pieces they hold of a K row through the wave's LDS row.
+                float* const krow = sh_krow_all[wave];
+                if (lane < D / 4) *reinterpret_cast<float4*>(krow + lane * 4) = k_own;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int kk = 0; kk < G::kSteps / 2; ++kk) { // two k-steps at a time: the pair of a "neox" rotation
+                    float x[2][8];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const float* src = krow + (kk + u * (G::kSteps / 2)) * 32 + grp * 8;
+                        const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+                        x[u][0] = lo.x; x[u][1] = lo.y; x[u][2] = lo.z; x[u][3] = lo.w;
+                        x[u][4] = hi.x; x[u][5] = hi.y; x[u][6] = hi.z; x[u][7] = hi.w;
+                    }
+                    if constexpr (ROPE) rotate2(x[0], x[1], kk);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        h8 h;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) h[e] = (_Float16)x[u][e];
+                        k_new16[kk + u * (G::kSteps / 2)] = __builtin_bit_cast(u32x4, h);
+                    }
+                }
+            }
+            h8 vh;
+            vh[0] = (_Float16)v_own[0].x; vh[1] = (_Float16)v_own[0].y; vh[2] = (_Float16)v_own[0].z; vh[3] = (_Float16)v_own[0].w;
+            vh[4] = (_Float16)v_own[1].x; vh[5] = (_Float16)v_own[1].y; vh[6] = (_Float16)v_own[1].z; vh[7] = (_Float16)v_own[1].w;
+            v_new16 = __builtin_bit_cast(u32x4, vh);
+            // The cache gets the row now (one head group's wave writes it): whatever the tile request that is under
+            // way brings back for this row is replaced from the registers above, and no other wave reads it, so the
+            // order of the two does not matter, and stores issued here are long done when the kernel ends.
+            if (hg == 0) {
+                const int row = pos % kTile;
+                const size_t row_off = ((size_t)kvh * n_ctx + pos) * D;
+                if (col == row % 16) {
+#pragma unroll
+                    for (int kk = 0; kk < G::kSteps; ++kk)
+                        *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(kc) + row_off + (kk * 4 + grp) * 8) = k_new16[kk];
+                }
+                if (lane < G::kChunksPerRow) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(vc) + row_off + lane * 8) = v_new16;
+            }
+        }
+    }
+
     for (; tile < n_tiles; tile += tile_step) {
         const bool more = tile + tile_step < n_tiles;
         if constexpr (STORE) {
-            if (store && tile == pos / kTile) { // the tile of the new row (the last visible one)
+            if (owner && tile == own_tile) { // the tile of the new row: into the operand registers
                 const int row = pos % kTile;
-                const size_t row_off = ((size_t)kvh * n_ctx + pos) * D;
-                // (Nothing below may be started ahead of this branch: the compiler would otherwise
-                // convert the new row before the loop, in every wave, and wait there for the row's
-                // loads -- the last ones issued, so for the whole first tile.)
-                auto here = [](float x) { // a copy the compiler cannot make anywhere else
-                    float y;
-                    asm volatile("v_mov_b32 %0, %1" : "=v"(y) : "v"(x));
-                    return y;
-                };
-                const float4 k_own = float4{here(k_raw.x), here(k_raw.y), here(k_raw.z), here(k_raw.w)};
-                const float4 v_own[2] = {float4{here(v_raw[0].x), here(v_raw[0].y), here(v_raw[0].z), here(v_raw[0].w)},
-                                         float4{here(v_raw[1].x), here(v_raw[1].y), here(v_raw[1].z), here(v_raw[1].w)}};
-                auto put_k = [&](int kk, u32x4 piece) { // into the operand registers and (one head group's wave) the cache
-                    if (col == row % 16) {
-                        kreg[(row / 16) * G::kSteps + kk] = piece;
-                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(kc) + row_off + (kk * 4 + grp) * 8) = piece;
-                    }
-                };
-                {
-                    // The new K row is rotated (rotate + store) and converted here, by the one wave
-                    // that needs it.  It has waited in four registers a lane; the lanes now hand
-                    // each other the pieces they hold of a K row through the wave's LDS row.
-                    float* const krow = sh_krow_all[wave];
-                    if (lane < D / 4) *reinterpret_cast<float4*>(krow + lane * 4) = k_own;
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                if (col == row % 16) {
 #pragma unroll
-                    for (int kk = 0; kk < G::kSteps / 2; ++kk) { // two k-steps at a time: the pair of a "neox" rotation
-                        float x[2][8];
+                    for (int kk = 0; kk < G::kSteps; ++kk)
 #pragma unroll
-                        for (int u = 0; u < 2; ++u) {
-                            const float* src = krow + (kk + u * (G::kSteps / 2)) * 32 + grp * 8;
-                            const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
-                            x[u][0] = lo.x; x[u][1] = lo.y; x[u][2] = lo.z; x[u][3] = lo.w;
-                            x[u][4] = hi.x; x[u][5] = hi.y; x[u][6] = hi.z; x[u][7] = hi.w;
-                        }
-                        if constexpr (ROPE) rotate2(x[0], x[1], kk);
-#pragma unroll
-                        for (int u = 0; u < 2; ++u) {
-                            h8 h;
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) h[e] = (_Float16)x[u][e];
-                            put_k(kk + u * (G::kSteps / 2), __builtin_bit_cast(u32x4, h));
-                        }
-                    }
+                        for (int t = 0; t < 2; ++t) // (constant register indices: a computed one sends the array to scratch memory)
+                            if (row / 16 == t) kreg[t * G::kSteps + kk] = k_new16[kk];
                 }
-                h8 vh;
-                vh[0] = (_Float16)v_own[0].x; vh[1] = (_Float16)v_own[0].y; vh[2] = (_Float16)v_own[0].z; vh[3] = (_Float16)v_own[0].w;
-                vh[4] = (_Float16)v_own[1].x; vh[5] = (_Float16)v_own[1].y; vh[6] = (_Float16)v_own[1].z; vh[7] = (_Float16)v_own[1].w;
-                const u32x4 v_new16 = __builtin_bit_cast(u32x4, vh);
 #pragma unroll
-                for (int i = 0; i < G::kLoads; ++i) {
-                    if ((i * 64 + lane) / G::kChunksPerRow == row) {
-                        vreg[i] = v_new16;
-                        if (hg == 0) *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(vc) + row_off + (lane % G::kChunksPerRow) * 8) = v_new16;
-                    }
-                }
+                for (int i = 0; i < G::kLoads; ++i)
+                    if ((i * 64 + lane) / G::kChunksPerRow == row) vreg[i] = v_new16;
             }
         }
         // ---- S^T = K Q^T : rows = KV row (sub-tile t, row col), columns = query head ----
