@@ -10,7 +10,7 @@
  * Weight matrices are GGUF tensors as the reference maps them (reference: src/common.h:47-77,
  * src/quant.h:14-45): `type` is the ggml type number (0 F32, 1 F16, 8 Q8_0, 12 Q4_K, 13 Q5_K,
  * 14 Q6_K), a matrix is n_out rows of n_in elements, rows packed back to back.
- * Limits: n_in a multiple of 32 (256 for the K types), at most 24576; matrices of type F32, F16,
+ * Limits: n_in a multiple of 32 (256 for the K types), at most 32768; matrices of type F32, F16,
  * Q4_K, Q5_K 16-byte aligned (2 bytes for Q8_0 and Q6_K, whose blocks are 34 and 210 bytes);
  * activations and norm weights 16-byte aligned; outputs and biases plain float arrays (4-byte aligned).
  * ORIN_FA_E_INVALID otherwise.  orin_decode_layer checks all seven of its matrices against these limits
@@ -46,7 +46,7 @@ int orin_rms_norm_rows(const float* x, const float* w, int rows, int cols, float
 
 /* Replaces llm::cuda::quantize_activation (reference: src/kernels.h:15, src/kernels.cu:136-157, 1778-1784).
  * The reference stores an int8 copy of x for the *_q8 products that follow; this stores an fp32
- * copy (n_in <= 32768; the products themselves take rows of at most 24576) in the library's own device
+ * copy (n_in <= 32768, the longest row the products take) in the library's own device
  * memory, so that those products see x as it was at this call, as they do in the reference. */
 int orin_quantize_activation(const float* x, int n_in);
 

@@ -425,11 +425,12 @@ hipError_t launch_slots(const GemvArgs& a, dim3 grid, hipStream_t stream) {
 template <int T>
 hipError_t launch_type(GemvArgs& a, int cu_count, hipStream_t stream) {
     const int n_slots = a.n_in / 32;
-    // Fewest waves per row that keep a lane at three slots or fewer (96 activations in registers).
+    // Fewest waves per row that keep a lane at three slots or fewer (96 activations in registers); rows past
+    // what four waves cover that way (24576 elements) take a fourth slot.
     int kw = 1;
     while (kw < kGemvWaves && n_slots > kw * 64 * 3) kw *= 2;
     const int slots = (n_slots + kw * 64 - 1) / (kw * 64);
-    if (slots > 3) return hipErrorInvalidValue;
+    if (slots > 4) return hipErrorInvalidValue;
     a.team_waves = kw;
     const int per_group = (kGemvWaves / kw) * (slots == 1 ? 2 : 1);
     int max_out = 0;
@@ -442,7 +443,8 @@ hipError_t launch_type(GemvArgs& a, int cu_count, hipStream_t stream) {
     switch (slots) {
     case 1: return launch_slots<T, 1>(a, grid, stream);
     case 2: return launch_slots<T, 2>(a, grid, stream);
-    default: return launch_slots<T, 3>(a, grid, stream);
+    case 3: return launch_slots<T, 3>(a, grid, stream);
+    default: return launch_slots<T, 4>(a, grid, stream);
     }
 }
 

@@ -9,7 +9,7 @@ namespace orin_fa {
 // Weight types, numbered as the reference numbers them (reference: src/common.h:47-54).
 enum : int { kF32 = 0, kF16 = 1, kQ8_0 = 8, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14 };
 
-constexpr int kMaxGemvIn = 24576;   // elements per weight row, at most (4 waves x 64 lanes x 3 slots x 32)
+constexpr int kMaxGemvIn = 32768;   // elements per weight row, at most (4 waves x 64 lanes x 4 slots x 32; the staged activation's size)
 constexpr int kStageFloats = 32768; // the staged activation of the *_q8 entry points
 
 struct GemvSeg {

@@ -56,7 +56,8 @@ def out_buf(n, fill=12345.0, pad=4):
 
 # rows that exercise every team shape of the vector-ALU kernel: (n_in, waves per row, slots per lane); on the
 # matrix cores the same lengths are 1 ... 74 blocks per row, shared among four waves
-SHAPES = [(256, 1, 1), (1536, 1, 1), (2048, 1, 1), (4096, 1, 2), (6144, 1, 3), (8960, 2, 3), (14336, 4, 2), (18944, 4, 3)]
+SHAPES = [(256, 1, 1), (1536, 1, 1), (2048, 1, 1), (4096, 1, 2), (6144, 1, 3), (8960, 2, 3), (14336, 4, 2), (18944, 4, 3),
+          (28672, 4, 4), (32768, 4, 4)]
 
 
 @pytest.fixture(params=["matrix cores", "vector ALU"])
@@ -92,6 +93,43 @@ def test_gemv_against_the_oracle(ly, wtype, where, n_in, kw, slots):
     ly.use_matrix_cores(True)
     print(f"gemv {lm.TYPE_NAME[wtype]} n_in {n_in} on the {unit}: err {e:.2e}", flush=True)
     assert e < TOL_OP
+
+
+@pytest.mark.parametrize("where", ["matrix cores", "vector ALU"])
+@pytest.mark.parametrize("wtype,n_in", [(lm.Q4_K, 28672), (lm.Q6_K, 29696), (lm.Q5_K, 32768), (lm.Q8_0, 32768)])
+def test_rows_past_24576_elements(ly, wtype, n_in, where):
+    """Rows longer than four waves cover at three slots a lane (the feed-forward width of a 70B-class model is
+    28672), up to the staged activation's 32768: the accumulating down projection and the gate/up pair
+    with the norm folded in, on either unit, and the next multiple of 256 refused."""
+    import torch
+    from orin_llm_amd.kernels import OrinFaError
+
+    n_out = 48
+    rs = lm.Stream(8800 + wtype + n_in)
+    t, tu = lm.make_tensor(rs, wtype, n_in, n_out), lm.make_tensor(rs, wtype, n_in, n_out)
+    x, y0 = rs.sym(n_in, 1.0), rs.sym(n_out, 2.0)
+    nw = (1.0 + rs.sym(n_in, 0.3)).astype(np.float32)
+    off = 2 if wtype in (lm.Q8_0, lm.Q6_K) else 0
+    w, wu, dx = dev_bytes(t[1], offset=off), dev_bytes(tu[1], offset=off), _dev(x)
+    ly.use_matrix_cores(where == "matrix cores")
+    try:
+        y = _dev(y0)
+        ly.gemv_multi(wtype, [w], None, [y], [n_out], dx, None, 0.0, n_in, True)
+        act = out_buf(n_out)
+        ly.gemv_norm_gate_up_swiglu(wtype, w, wu, dx, _dev(nw), 1e-6, act, n_in, n_out)
+        torch.cuda.synchronize()
+        e_add = vec_err(y.cpu().numpy(), (y0 + ref.gemv(wtype, t[1], x, n_in, n_out)).astype(np.float64))
+        xn = ref.rms_norm(x, nw, 1e-6)
+        want = ref.swiglu(ref.gemv(wtype, t[1], xn, n_in, n_out), ref.gemv(wtype, tu[1], xn, n_in, n_out)).astype(np.float64)
+        got = act.cpu().numpy()
+        e_ffn = vec_err(got[:n_out], want)
+        print(f"type {lm.TYPE_NAME[wtype]} n_in {n_in} on the {where}: += {e_add:.2e}, norm + gate/up {e_ffn:.2e}", flush=True)
+        assert (got[n_out:] == 12345.0).all()
+        assert e_add < TOL_OP and e_ffn < TOL_OP
+        with pytest.raises(OrinFaError):
+            ly.gemv(wtype, w, dx, out_buf(n_out), 32768 + 256, n_out)
+    finally:
+        ly.use_matrix_cores(True)
 
 
 @pytest.mark.parametrize("wtype", [lm.Q4_K, lm.Q6_K, lm.F16])
