@@ -428,7 +428,7 @@ def test_rejects_bad_arguments(ly):
                  lambda: ly.gemv(lm.Q4_K, w[4:], x, y, 256, 2),        # misaligned matrix
                  lambda: ly.gemv(lm.Q4_K, w, x[1:], y, 256, 2),        # misaligned activation
                  lambda: ly.gemv(lm.Q4_K, w, x, y.view(torch.uint8)[2:10].view(torch.int16), 256, 2),  # output not on a float boundary
-                 lambda: ly.gemv(lm.F16, w, x, y, 32768, 1),           # longer than a workgroup covers
+                 lambda: ly.gemv(lm.F16, w, x, y, 32768 + 32, 1),      # longer than a workgroup covers
                  lambda: ly.gemv(lm.Q4_K, None, x, y, 256, 2),
                  lambda: ly.quantize_activation(x, 40000)):
         with pytest.raises(OrinFaError):
