@@ -111,6 +111,9 @@ WORKLOADS = {
     # (Q4_K gate/up pair with the norm folded in; Q6_K down projection adding into the residual stream): (what, n_in, n_out)
     "llama8b-gateup-timeline": ("llama8b", "timeline", 0, ("gateup", 4096, 14336)),
     "llama8b-down-timeline": ("llama8b", "timeline", 0, ("down", 14336, 4096)),
+    # ... and of a Qwen2.5-1.5B layer, whose launches leave resident places empty
+    "qwen1.5b-gateup-timeline": ("qwen1.5b", "timeline", 0, ("gateup", 1536, 8960)),
+    "qwen1.5b-down-timeline": ("qwen1.5b", "timeline", 0, ("down", 8960, 1536)),
 }
 # HBM bytes per launch of the dominant kernel (decode: per layer, both kernels), from the FETCH_SIZE and
 # WRITE_SIZE counter passes of rocprofv3 scaled by the same counters on a plain 256 MiB copy: recorded
