@@ -1,6 +1,8 @@
 """orin_decode_layer at the benchmark's model shapes, against the CPU oracle's operators in the reference's order
-(src/model_gpu.cu:251-293): one Llama-3-8B-shaped layer at cache length 8192 and one Qwen2.5-1.5B-shaped layer (with
-q/k/v biases) at 32768, weights in the mix of a Q4_K_M file (Q4_K; attn_v and ffn_down Q6_K).  These are the shapes
+(src/model_gpu.cu:251-293): one Llama-3-8B-shaped layer at cache length 8192, one Qwen2.5-1.5B-shaped and one
+Qwen2.5-7B-shaped layer (with q/k/v biases; seven query heads per KV head in the latter) at 32768, and one
+Llama-3.2-1B-shaped layer (head_dim 64, rotary frequencies divided by per-pair factors) at 8192, weights in the mix
+of a Q4_K_M file (Q4_K; attn_v and ffn_down Q6_K).  These are the shapes
 at which the layer's launches take the forms the small whole-model fixtures never reach: q, k, v of two types in one
 launch with eight waves a workgroup, accumulating projections whose rows are shared among workgroups, the kernel for
 launches that leave resident places empty, 32-128 KV splits.
@@ -29,6 +31,10 @@ MODELS = {
                     eps=1.0e-5),
     "qwen1.5b": dict(n_embd=1536, n_head=12, n_kv=2, head_dim=128, n_ff=8960, n_ctx=32768, L=32768, bias=True, neox=1, theta=1.0e6,
                      eps=1.0e-6),
+    "qwen7b": dict(n_embd=3584, n_head=28, n_kv=4, head_dim=128, n_ff=18944, n_ctx=32768, L=32767, bias=True, neox=1, theta=1.0e6,
+                   eps=1.0e-6),
+    "llama1b": dict(n_embd=2048, n_head=32, n_kv=8, head_dim=64, n_ff=8192, n_ctx=8192, L=8192, bias=False, neox=0, theta=5.0e5,
+                    eps=1.0e-5, freq_factors=True),
 }
 TYPES = dict(wq=lm.Q4_K, wk=lm.Q4_K, wv=lm.Q6_K, wo=lm.Q4_K, ffn_gate=lm.Q4_K, ffn_up=lm.Q4_K, ffn_down=lm.Q6_K)
 
@@ -43,6 +49,8 @@ def make_layer(name):
     L["ffn_norm"] = (1.0 + rs.sym(ne, 0.2)).astype(np.float32)
     if c["bias"]:
         L["bq"], L["bk"], L["bv"] = rs.sym(nq, 0.3), rs.sym(nkv, 0.3), rs.sym(nkv, 0.3)
+    if c.get("freq_factors"):   # (the long-context scaling of the Llama-3 family: low frequencies slowed down)
+        L["freq_factors"] = np.linspace(1.0, 8.0, c["head_dim"] // 2).astype(np.float32)
     x0 = rs.sym(ne, 1.0)
     rng = np.random.default_rng(77)
     kc = rng.standard_normal((c["n_kv"], c["n_ctx"], c["head_dim"]), dtype=np.float32).astype(np.float16).view(np.uint16)
@@ -58,8 +66,8 @@ def oracle_layer(c, L, dims, x0, kc, vc):
     q, k, v = mv("wq", xn), mv("wk", xn), mv("wv", xn)
     if c["bias"]:
         q, k, v = q + L["bq"], k + L["bk"], v + L["bv"]
-    q = ref.rope_batch(q.reshape(H, d), d, d, c["theta"], pos, H, None, bool(c["neox"]))
-    k = ref.rope_batch(k.reshape(G, d), d, d, c["theta"], pos, G, None, bool(c["neox"]))
+    q = ref.rope_batch(q.reshape(H, d), d, d, c["theta"], pos, H, L.get("freq_factors"), bool(c["neox"]))
+    k = ref.rope_batch(k.reshape(G, d), d, d, c["theta"], pos, G, L.get("freq_factors"), bool(c["neox"]))
     kc, vc = kc.copy(), vc.copy()
     ref.kv_store_f16(kc, vc, k.reshape(1, G, d), v.reshape(1, G, d), G, d, c["n_ctx"], pos, 1)
     attn = ref.flash_attention_decode_ind(q, kc, vc, H, G, d, c["n_ctx"], pos, float(1.0 / np.sqrt(d))).reshape(-1)
@@ -82,9 +90,9 @@ def test_decode_layer_at_model_shape(fa, ly, case, how):
 
     name, c, L, x0, kc, vc, want, kc_want, vc_want = case
     H, G, d, ne, nff, n_ctx = c["n_head"], c["n_kv"], c["head_dim"], c["n_embd"], c["n_ff"], c["n_ctx"]
-    hp = dict(n_embd=ne, n_head=H, n_kv=G, head_dim=d, n_ff=nff, n_rot=d, neox=c["neox"], rms_eps=c["eps"], rope_theta=c["theta"],
-              freq_factors_dev=None)
     D = {k: ((v[0], dev_bytes(v[1], offset=2 if v[0] == lm.Q6_K else 0)) if isinstance(v, tuple) else _dev(v)) for k, v in L.items()}
+    hp = dict(n_embd=ne, n_head=H, n_kv=G, head_dim=d, n_ff=nff, n_rot=d, neox=c["neox"], rms_eps=c["eps"], rope_theta=c["theta"],
+              freq_factors_dev=D.get("freq_factors"))
     z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")  # noqa: E731
     bufs = dict(x=z(ne), xn=z(ne), xn2=z(ne), q=z(H * d), k=z(G * d), v=z(G * d), attn=z(max(H * d, ne)), act=z(nff), up_tmp=z(nff))
     dkc, dvc = torch.from_numpy(kc.view(np.int16)).cuda(), torch.from_numpy(vc.view(np.int16)).cuda()
@@ -96,7 +104,7 @@ def test_decode_layer_at_model_shape(fa, ly, case, how):
         if how == "calls":
             ly.decode_layer_calls(hp, D, bufs, dkc, dvc, d_pos, n_ctx)
         else:
-            fa.rope_angles_ind(angles, d, c["theta"], d_pos)
+            fa.rope_angles_ind(angles, d, c["theta"], d_pos, D.get("freq_factors"))
             ly.decode_layer(desc)
 
     bufs["x"].copy_(_dev(x0))
@@ -142,9 +150,9 @@ def test_decode_layer_replays_bit_for_bit_with_one_share(fa, ly, case):
 
     name, c, L, x0, kc, vc, want, _, _ = case
     H, G, d, ne, nff, n_ctx = c["n_head"], c["n_kv"], c["head_dim"], c["n_embd"], c["n_ff"], c["n_ctx"]
-    hp = dict(n_embd=ne, n_head=H, n_kv=G, head_dim=d, n_ff=nff, n_rot=d, neox=c["neox"], rms_eps=c["eps"], rope_theta=c["theta"],
-              freq_factors_dev=None)
     D = {k: ((v[0], dev_bytes(v[1], offset=2 if v[0] == lm.Q6_K else 0)) if isinstance(v, tuple) else _dev(v)) for k, v in L.items()}
+    hp = dict(n_embd=ne, n_head=H, n_kv=G, head_dim=d, n_ff=nff, n_rot=d, neox=c["neox"], rms_eps=c["eps"], rope_theta=c["theta"],
+              freq_factors_dev=D.get("freq_factors"))
     z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")  # noqa: E731
     bufs = dict(x=z(ne), q=z(H * d), k=z(G * d), v=z(G * d), attn=z(max(H * d, ne)), act=z(nff), up_tmp=z(nff))
     dkc, dvc = torch.from_numpy(kc.view(np.int16)).cuda(), torch.from_numpy(vc.view(np.int16)).cuda()
