@@ -229,7 +229,9 @@ CUTOFFS = [(None, "whole layer (split + combine kernels)"), (1, "split kernel al
 PREFILL_CUTOFFS = [(None, "whole kernel"), (16, "leaving once the accumulators are handed over (no barrier, merge, store)"),
                    (8, "leaving behind the main loop (no last products either)"),
                    (1, "whole, main loop without its vector work"), (2, "whole, main loop without its LDS operand reads"),
-                   (4, "whole, main loop without its copies"), (7, "whole, main loop of matrix instructions only")]
+                   (4, "whole, main loop without its copies"), (32, "whole, main loop's copies all of one tile (no trip beyond the nearest cache)"),
+                   (64, "whole, main loop's copies of the head's first 32 tiles over and over (no trip beyond the L2)"),
+                   (7, "whole, main loop of matrix instructions only")]
 
 
 def _need_cut_off_builds():

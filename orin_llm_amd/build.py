@@ -19,7 +19,7 @@ BENCH_SOURCE = os.path.join(HERE, "csrc", "bench_aids.hip")
 PROBE_FLAGS = (1, 3, 7, 15, 31)
 PROBE_LIB = os.path.join(HERE, "liborin_fa_probe_{}.so")
 # ... and of the prefill kernel (-DORIN_FA_PREFILL_PROBE=flags, see fa_prefill.hip)
-PPROBE_FLAGS = (1, 2, 4, 7, 8, 16)
+PPROBE_FLAGS = (1, 2, 4, 7, 8, 16, 32, 64)
 PPROBE_LIB = os.path.join(HERE, "liborin_fa_pprobe_{}.so")
 OBJ_DIR = os.path.join(HERE, "_obj")
 SOURCES = [os.path.join(HERE, "csrc", n)

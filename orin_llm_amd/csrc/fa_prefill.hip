@@ -56,7 +56,10 @@ __device__ long long g_prefill_stamps[kStampWgs * kPrefillWaves * kStampSlots];
 // each part costs.  In the main loop -- 1: no vector work (the softmax of the step), 2: no LDS operand
 // reads, 4: no copies of the next tiles (7: matrix instructions only).  8: the kernel leaves behind the
 // main loop (no last products, no merge, no store).  16: it leaves once the waves have handed their
-// accumulators over (no barrier, no merge, no store).  0 in the library proper, where none of this exists.
+// accumulators over (no barrier, no merge, no store).  32: every copy of the main loop fetches the tile at
+// offset 0 (the same work for the load unit and LDS, but no trip beyond the nearest cache).  64: they fetch
+// tile (t mod 32): half a megabyte per KV head, which stays in the L2 and does not fit the vector cache.  0 in the
+// library proper, where none of this exists.
 #ifndef ORIN_FA_PREFILL_PROBE
 #define ORIN_FA_PREFILL_PROBE 0
 #endif
@@ -382,7 +385,11 @@ __global__ __launch_bounds__(kPrefillWaves * 64) void fa_prefill_kernel(
     // Main-loop copies: every tile they name is either wholly inside the visible range, and its
     // base travels as the scalar offset, or below zero (steps past the wave's last tile), and then
     // tile 0 is copied instead, into a buffer nobody reads any more.
-    auto tile_soff = [&](int tile) { return __builtin_amdgcn_readfirstlane((tile > 0 ? tile : 0) * G::kTileB); };
+    auto tile_soff = [&](int tile) {
+        if constexpr ((kPProbe & 32) != 0) return 0;
+        if constexpr ((kPProbe & 64) != 0) return __builtin_amdgcn_readfirstlane(((tile > 0 ? tile : 0) & 31) * G::kTileB);
+        return __builtin_amdgcn_readfirstlane((tile > 0 ? tile : 0) * G::kTileB);
+    };
     auto copy_one = [&](auto ic, const i32x4& d, unsigned lds_dst, int soff) { // copy number i (of kCopies) of such a tile
         constexpr int i = decltype(ic)::value;
         constexpr int half = i / 4, sub = i % 4;
