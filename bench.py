@@ -5,7 +5,7 @@
 
 The LAST line of stdout is one compact JSON object (under 4 KB: metric, value, roofline, cpu_baseline, parity and
 the few figures of the target workloads under "targets"); every workload's full result goes to
-gpurun_out/bench_full.json.  --full also runs the neighbouring operators' workloads (rope, kv_store, kv_shift,
+the file --full-record names.  --full also runs the neighbouring operators' workloads (rope, kv_store, kv_shift,
 fused decode entry points, long-context prefill, logits); measurement aids (timelines, cut-off builds, read-pattern
 and hand-off stand-ins: bench_aids.py) run only when named with --workload.  A "step" is one pass of the attention operator over a whole layer
 stack of synthetic inputs already resident in HBM (independent seeds and buffers per layer):
