@@ -284,6 +284,50 @@ def test_decode_rope_store_equals_the_four_calls(fa, H, G, d, n_ctx, n_rot, neox
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,n_ctx,neox", [(12, 2, 128, 32768, True), (32, 8, 64, 8192, False)])
+def test_decode_rope_store_over_a_sweep_of_positions(fa, H, G, d, n_ctx, neox):
+    """The one call against the four it stands for at every position 2^e - 1, 2^e, 2^e + 1 and at a handful in
+    between: the wave that owns the new row's tile, the number of tiles a split takes and the number of splits
+    with any tile all change with the position, which the captured launch reads on the device.  Same cache bytes
+    and same output, bit for bit, from one graph replayed throughout."""
+    import torch
+    scale, theta = float(1.0 / np.sqrt(d)), (1.0e6 if neox else 5.0e5)
+    rng = np.random.default_rng(n_ctx + H)
+    base_k = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    base_v = rng.standard_normal((G, n_ctx, d)).astype(np.float16).view(np.int16)
+    q, k_new, v_new = torch.zeros((H, d), device="cuda"), torch.zeros((G, d), device="cuda"), torch.zeros((G, d), device="cuda")
+    dpos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ka, va = torch.from_numpy(base_k).cuda(), torch.from_numpy(base_v).cuda()
+    kb, vb = ka.clone(), va.clone()
+    out_a, out_b = torch.empty((H, d), device="cuda"), torch.empty((H, d), device="cuda")
+    rope_ind = fa.rope_neox_ind if neox else fa.rope_normal_ind
+    g = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(g):
+            fa.set_stream(torch.cuda.current_stream().cuda_stream)
+            fa.flash_attention_decode_rope_store_ind(q, k_new, v_new, kb, vb, out_b, H, G, d, n_ctx, dpos, scale, d, theta, None, neox, None)
+    finally:
+        fa.set_stream(torch.cuda.current_stream().cuda_stream)
+    positions = sorted({p for e in range(0, 16) for p in (2 ** e - 1, 2 ** e, 2 ** e + 1) if 0 <= p < n_ctx}
+                       | {int(x) for x in rng.integers(0, n_ctx, 24)} | {n_ctx - 1, n_ctx - 33, n_ctx - 257})
+    for pos in positions:
+        q.copy_(torch.from_numpy(rng.standard_normal((H, d)).astype(np.float32)))
+        k_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        v_new.copy_(torch.from_numpy(rng.standard_normal((G, d)).astype(np.float32) * 3.0))
+        dpos.fill_(pos)
+        q_rot, k_rot = q.clone(), k_new.clone()
+        rope_ind(q_rot, H, d, d, theta, dpos, None)
+        rope_ind(k_rot, G, d, d, theta, dpos, None)
+        fa.kv_store_ind(ka, va, k_rot, v_new, G, d, n_ctx, dpos)
+        fa.flash_attention_decode_ind(q_rot, ka, va, out_a, H, G, d, n_ctx, dpos, scale)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ka, kb) and torch.equal(va, vb), pos
+        assert torch.equal(out_a.view(torch.int32), out_b.view(torch.int32)), pos
+    print(f"{len(positions)} positions of a {n_ctx}-row cache", flush=True)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("H,G,d,n_ctx,n_past,batch,n_rot,neox,ff", [
     (12, 2, 128, 4096, 3584, 512, 128, True, False),   # Qwen2.5-1.5B chunk
     (32, 8, 128, 1024, 100, 300, 128, False, True),    # Llama-3 ("normal" pairing, frequency factors)
